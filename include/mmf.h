@@ -1,0 +1,152 @@
+/* libmmf_hip -- C ABI of the MI355X (gfx950) kernels for the MatMul-free LM hot path.
+ *
+ * The reference (ridgerchu/matmulfreellm, package `mmfreelm`) has no FFI: the path sits
+ * behind Python callables (torch.autograd.Function wrappers around Triton kernels).  Each
+ * entry point below names the reference callable it replaces; a Python host binds them
+ * with ctypes and passes tensor.data_ptr() values.
+ *
+ * Conventions
+ *   - every function returns 0 on success, a negative MMF_ERR_* code for a rejected
+ *     argument, or a positive hipError_t from the launch; nothing throws;
+ *   - all pointers are DEVICE pointers owned by the caller; no entry point allocates,
+ *     frees, synchronises or keeps a pointer after it returns; work is enqueued on
+ *     `stream` (a hipStream_t passed as void*; NULL = the default stream);
+ *   - `dtype` arguments: 0 = fp32, 1 = bf16, 2 = fp16 (MMF_F32 / MMF_BF16 / MMF_F16);
+ *   - matrices are row-major and contiguous unless a leading dimension is given;
+ *   - 16-byte alignment is required of every matrix base pointer whose row length is a
+ *     multiple of 8 elements (torch allocations always are), of packed weights and codes.
+ *
+ * Arithmetic (identical on every call, independent of launch shape): fp32 math with one
+ * rounding per operation (no fused multiply-add), sums of squares in fp64, correctly
+ * rounded divide/sqrt, round-half-to-even for integer codes, and a fixed polynomial exp.
+ */
+#ifndef MMF_H_
+#define MMF_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MMF_F32 0
+#define MMF_BF16 1
+#define MMF_F16 2
+
+#ifndef MMF_ERR_ARG
+#define MMF_ERR_ARG (-1)   /* bad shape, null pointer, unsupported dtype combination */
+#define MMF_ERR_WIDE (-2)  /* row wider than the fused kernels hold in registers / LDS */
+#define MMF_ERR_ALIGN (-3) /* pointer not 16-byte aligned where required */
+#endif
+
+/* ---- weights: absmean ternarisation + 2-bit packing --------------------------------
+ * Replaces weight_quant(), mmfreelm/ops/fusedbitnet.py:32-46, which the reference re-runs
+ * on the latent matrix in every forward (fusedbitnet.py:456).
+ *
+ * w [N, K] latent weights (dtype w_dtype, nn.Linear layout).  Writes
+ *   packed : mmf_packed_bytes(N, K) bytes, blocks of 32 rows x 128 inputs, 2 bits per
+ *            weight holding t + 1, padded with t = 0 to multiples of 32 / 128;
+ *   wdeq   : 1 float, the de-quantisation step  dtype(1 / dtype(1 / mean|w|)).
+ * workspace: mmf_ternarize_workspace_bytes() bytes of scratch (8-byte aligned). */
+int64_t mmf_packed_bytes(int64_t N, int64_t K);
+int64_t mmf_ternarize_workspace_bytes(void);
+int mmf_ternarize_pack(const void* w, int w_dtype, int64_t N, int64_t K, void* packed, float* wdeq,
+                       void* workspace, void* stream);
+/* packed -> int8 codes [N, K] in {-1, 0, 1} (inspection / tests). */
+int mmf_unpack_ternary(const void* packed, int64_t N, int64_t K, int8_t* codes, void* stream);
+
+/* ---- RMSNorm -------------------------------------------------------------------------
+ * Replaces rms_norm_fn / LayerNormFn.forward with is_rms_norm=True,
+ * mmfreelm/modules/layernorm.py:445-482, kernel :104-165 (module RMSNorm :586-623).
+ * y = T((x [+ residual]) * rstd * weight); residual_out (optional) receives the fp32 sum
+ * rounded to residual_dtype (= x_dtype or fp32).  weight may be NULL; weight_dtype is
+ * fp32 or x_dtype. */
+int mmf_rmsnorm(const void* x, const void* residual, const void* weight, void* y, void* residual_out,
+                int64_t M, int64_t K, float eps, int x_dtype, int residual_dtype, int weight_dtype,
+                void* stream);
+
+/* Replaces the gated variant, mmfreelm/modules/fused_norm_gate.py:420-460, kernel :68-131
+ * (module FusedRMSNormSwishGate :514-536):  y = T(norm(x) * gate * sigmoid(gate)).
+ * x may be a column slice of a wider matrix (row stride ldx elements); gate, y are [M, K]. */
+int mmf_rmsnorm_swishgate(const void* x, int64_t ldx, const void* gate, const void* residual, const void* weight,
+                          void* y, void* residual_out, int64_t M, int64_t K, float eps, int x_dtype,
+                          int residual_dtype, int weight_dtype, void* stream);
+
+/* Replaces swiglu(), mmfreelm/modules/activations.py:115-119,143-153:
+ * out[r, c] = T((x[r,c] * y[r,c]) / (1 + exp(-x[r,c]))); x and y may be column slices of a
+ * wider matrix (leading dimensions ldx, ldy in elements), out is [rows, cols] contiguous. */
+int mmf_swiglu(const void* x, int64_t ldx, const void* y, int64_t ldy, void* out, int64_t rows,
+               int64_t cols, int dtype, void* stream);
+
+/* ---- activations: RMSNorm + per-row absmax int8 codes ---------------------------------
+ * Replaces _layer_norm_fwd_quant / its kernel, mmfreelm/ops/fusedbitnet.py:63-190, and
+ * activation_quant(), fusedbitnet.py:15-29.  Instead of a de-quantised tensor it emits
+ *   q    : int8 codes, zero padded to Kp = ceil128(K) columns; tiled = 0: row-major
+ *          [M, Kp]; tiled = 1: [ceil32(M)/32][Kp/16][32 rows][16 bytes] (the matrix-core
+ *          operand layout); mmf_codes_bytes(M, K, tiled) bytes;
+ *   deq  : [M] fp32, 1 / scale with scale = 127 / max(max|y|, 1e-5);
+ *   qsum : [M] int32, sum of the row's codes. */
+int64_t mmf_codes_bytes(int64_t M, int64_t K, int tiled);
+int mmf_rmsnorm_quant(const void* x, const void* residual, const void* weight, int8_t* q, float* deq,
+                      int* qsum, void* residual_out, int64_t M, int64_t K, float eps, int x_dtype,
+                      int residual_dtype, int weight_dtype, int tiled, void* stream);
+
+/* ---- BitLinear contraction ------------------------------------------------------------
+ * Both replace F.linear(y, weight_quant(W)) at mmfreelm/ops/fusedbitnet.py:456-458 (class
+ * FusedBitLinear :584-610, layer_norm_linear_quant_fn :513-536):
+ *   out[m, n] = T( fp32(sum_k q[m,k] * t[n,k]) * deq[m] * wdeq[n / seg_rows] (+ bias[n]) ),
+ * and, when `addend` ([M, N], same dtype and leading dimension as out) is given,
+ *   out = T(out + addend)  -- the block's residual add (modeling_hgrn_bit.py:109) fused in.
+ * `packed` may be several matrices with the same K packed one after the other (each a
+ * multiple of 32 rows); wdeq then holds one step per seg_rows output rows.
+ *
+ * mmf_bitlinear_gemv: decode-sized M; norm + quantiser + contraction in one launch, x is
+ *   the un-normalised input [M, K] (K <= mmf_bitlinear_gemv_max_k()).
+ * mmf_bitlinear_mfma: int8 matrix-core contraction on codes from mmf_rmsnorm_quant
+ *   (tiled = 1); out has leading dimension ldo; config < 0 picks the tile shape from M. */
+int64_t mmf_bitlinear_gemv_max_k(void);
+int mmf_bitlinear_gemv(const void* x, const void* norm_weight, const void* packed, const float* wdeq,
+                       int64_t seg_rows, const void* bias, const void* addend, void* out, int64_t M, int64_t K,
+                       int64_t N, float eps, int x_dtype, int norm_weight_dtype, void* stream);
+int mmf_bitlinear_mfma(const int8_t* codes_tiled, const float* deq, const int* qsum, const void* packed,
+                       const float* wdeq, int64_t seg_rows, const void* bias, const void* addend, void* out,
+                       int64_t ldo, int64_t M, int64_t K, int64_t N, int out_dtype, int config, void* stream);
+
+/* ---- HGRN recurrence ------------------------------------------------------------------
+ * x, g, o: [BH, T, D] contiguous (BH = batch * heads); h0 / ht: [BH, D] fp32 or NULL.
+ * mmf_hgrn_recurrent replaces fused_recurrent_hgrn, mmfreelm/ops/hgrn/recurrent_fuse.py:
+ *   176-185 (kernel :32-68): h = g*h + x with g the decay itself.
+ * mmf_hgrn_chunk replaces chunk_hgrn, mmfreelm/ops/hgrn/chunk.py:287-296 (kernels :49-116):
+ *   h = exp(g)*h + x with g the log decay, chunked over T (1 <= chunk <= 64).
+ * The final state is fp32 in both (the reference rounds the recurrent one to x's dtype). */
+int mmf_hgrn_recurrent(const void* x, const void* g, const float* h0, void* o, float* ht, int64_t BH,
+                       int64_t T, int64_t D, int dtype, void* stream);
+int mmf_hgrn_chunk(const void* x, const void* g, const float* h0, void* o, float* ht, int64_t BH,
+                   int64_t T, int64_t D, int chunk, int dtype, void* stream);
+
+/* Gate math of HGRNBitAttention.forward, mmfreelm/layers/hgrn_bit.py:113-120, fused:
+ *   g_out = T(lb + (1 - lb) * sigmoid(f))  (lower_bound NULL: T(sigmoid(f)))
+ *   x_out = T((i * (1 - g_out)) / (1 + exp(-i))), 0 where mask[row] == 0.
+ * i_in / f_in: [rows, D] with leading dimensions ldi / ldf; lower_bound [D] fp32 or NULL;
+ * mask [rows] bytes or NULL.  mmf_hgrn_step fuses the same math with one recurrence step
+ * (T = 1 decode): state [rows, D] fp32 is updated in place, o = T(state). */
+int mmf_hgrn_gate(const void* i_in, int64_t ldi, const void* f_in, int64_t ldf, const float* lower_bound,
+                  const uint8_t* mask, void* x_out, void* g_out, int64_t rows, int64_t D, int dtype,
+                  void* stream);
+int mmf_hgrn_step(const void* i_in, int64_t ldi, const void* f_in, int64_t ldf, const float* lower_bound,
+                  const uint8_t* mask, float* state, void* o, int64_t rows, int64_t D, int dtype,
+                  void* stream);
+
+/* ---- the two ends of a decode step ------------------------------------------------------
+ * mmf_embedding replaces nn.Embedding.forward at mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py:212:
+ *   out[r, :] = table[ids[r], :]  (ids int64; an id outside [0, vocab) reads row 0).
+ * mmf_argmax is the greedy choice over the logits of HGRNBitForCausalLM.forward
+ *   (modeling_hgrn_bit.py:386): out[r] = lowest index of the row maximum (int64). */
+int mmf_embedding(const void* table, const int64_t* ids, void* out, int64_t rows, int64_t H, int64_t vocab,
+                  int dtype, void* stream);
+int mmf_argmax(const void* logits, int64_t ld, int64_t rows, int64_t V, int64_t* out, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MMF_H_ */

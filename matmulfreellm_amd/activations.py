@@ -1,0 +1,7 @@
+"""swiglu (interface of mmfreelm/modules/activations.py:178)."""
+from . import functional as F_
+
+
+def swiglu(x, y):
+    """x * sigmoid(x) * y computed in fp32 as (x*y)/(1+exp(-x)), returned in x.dtype."""
+    return F_.swiglu(x, y)

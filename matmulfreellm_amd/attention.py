@@ -1,0 +1,130 @@
+"""HGRNBitAttention: the HGRN token mixer built from BitLinear projections.
+
+Interface of mmfreelm/layers/hgrn_bit.py:22-162.  Data flow of forward (:83-142):
+    i, f, g = i_proj(h), f_proj(h), g_proj(h)           three BitLinear H -> H
+    f = sigmoid(f); f = lb + (1 - lb) * f  (layer > 0)   gate math, one fused kernel
+    i = swiglu(i, 1 - f); i *= mask
+    o, state = recurrence(i, f, state)                   h_t = f_t * h_{t-1} + i_t
+    o = g_norm(g, o)                                     RMSNorm(g) * o * sigmoid(o)
+    o = o_proj(o)
+The three input projections run as one contraction over the stacked packed weights when
+their inner norm weights are equal (they then share the int8 codes of h).
+"""
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from . import functional as F_
+from .bitlinear import FusedBitLinear as BitLinear
+from .fused_norm_gate import FusedRMSNormSwishGate
+
+
+class HGRNBitAttention(nn.Module):
+
+    def __init__(self, mode: str = "fused_recurrent", hidden_size: int = 1024, num_heads: Optional[int] = None,
+                 expand_ratio: Optional[int] = 1, use_short_conv: bool = False, conv_size: int = 4,
+                 conv_bias: bool = False, share_conv_kernel: bool = True, layernorm_eps: float = 1e-5,
+                 layer_idx: int = None):
+        super().__init__()
+        if num_heads is None:
+            num_heads = 1
+        self.mode = mode
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.expand_ratio = expand_ratio
+        self.input_dim = int(hidden_size * expand_ratio)
+        self.head_dim = self.input_dim // self.num_heads
+        self.use_short_conv = use_short_conv
+        self.conv_size = conv_size
+        self.conv_bias = conv_bias
+        self.share_conv_kernel = share_conv_kernel
+        self.layer_idx = layer_idx
+
+        assert mode in ["fused_recurrent", "chunk"], f"Not supported mode `{mode}`."
+        assert self.hidden_size % num_heads == 0, f"hidden size must be divisible by num_heads of {num_heads}"
+        if use_short_conv:
+            # The reference's call site for the convolution is broken (three positionals into a
+            # two-argument forward, mmfreelm/layers/hgrn_bit.py:101) and the option defaults to off.
+            raise NotImplementedError("use_short_conv=True is not supported")
+
+        self.i_proj = BitLinear(hidden_size, self.input_dim, bias=False)
+        self.f_proj = BitLinear(hidden_size, self.input_dim, bias=False)
+        self.g_proj = BitLinear(hidden_size, self.input_dim, bias=False)
+        self.g_norm = FusedRMSNormSwishGate(self.input_dim, layernorm_eps)
+        self.o_proj = BitLinear(self.input_dim, hidden_size, bias=False)
+        self.apply(self._initialize_weights)
+        self._ifg_key, self._ifg = None, None
+
+    def _initialize_weights(self, module):
+        if getattr(module, "_is_hf_initialized", False):
+            return
+        if isinstance(module, nn.Linear):
+            nn.init.xavier_uniform_(module.weight, gain=2 ** -2.5)
+            if module.bias is not None:
+                nn.init.zeros_(module.bias)
+        module._is_hf_initialized = True
+
+    # ---- stacked i/f/g projection ------------------------------------------------------
+    def _stacked_ifg(self):
+        """PackedWeight of [i; f; g] if the three inner norms are identical, else None."""
+        projs = (self.i_proj, self.f_proj, self.g_proj)
+        key = tuple((p.weight.data_ptr(), p.weight._version, p.norm.weight.data_ptr(), p.norm.weight._version,
+                     p.weight.dtype, p.weight.device) for p in projs)
+        if key != self._ifg_key:
+            self._ifg_key = key
+            same = (self.input_dim % 32 == 0 and all(p.bias is None for p in projs)
+                    and all(p.norm.eps == projs[0].norm.eps and p.fused_eps == projs[0].fused_eps for p in projs)
+                    and torch.equal(self.i_proj.norm.weight, self.f_proj.norm.weight)
+                    and torch.equal(self.i_proj.norm.weight, self.g_proj.norm.weight))
+            self._ifg = F_.stack_packed([p.packed_weight() for p in projs]) if same else None
+        return self._ifg
+
+    def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
+                past_key_values=None, use_cache: Optional[bool] = False, output_attentions: Optional[bool] = False,
+                lower_bound: Optional[torch.Tensor] = None, **kwargs) -> Tuple[torch.Tensor, None, object]:
+        B, T, _ = hidden_states.shape
+        D = self.input_dim
+        last_state = past_key_values[self.layer_idx] if use_cache else None
+
+        stacked = self._stacked_ifg()
+        if stacked is not None:
+            p = self.i_proj
+            eps = p.norm.eps if p.fused_eps is None else p.fused_eps
+            ifg = F_.bitlinear(hidden_states, p.norm.weight, stacked, eps=eps)
+            i, f, g = ifg[..., :D], ifg[..., D:2 * D], ifg[..., 2 * D:]
+        else:
+            i, f, g = self.i_proj(hidden_states), self.f_proj(hidden_states), self.g_proj(hidden_states)
+
+        lb = lower_bound if (lower_bound is not None and self.layer_idx > 0) else None
+        recurrent_state = last_state[-1] if use_cache else None
+
+        if T == 1 and recurrent_state is not None and recurrent_state.dtype == torch.float32 \
+                and recurrent_state.is_contiguous():
+            # decode: gate math and the single recurrence step in one kernel, state updated in place
+            o = F_.hgrn_step(i, f, recurrent_state.view(B, D), lb, attention_mask)
+        else:
+            x_in, gate = F_.hgrn_gate(i, f, lb, attention_mask)
+            x4, g4 = x_in.view(B, 1, T, D), gate.view(B, 1, T, D)      # heads are independent channels
+            h0 = recurrent_state.reshape(B, 1, D) if recurrent_state is not None else None
+            if self.mode == "chunk" and T > 1:
+                raise NotImplementedError("chunk mode takes log-domain gates; the model path uses fused_recurrent")
+            o, new_state = F_.hgrn_recurrent(x4, g4, initial_state=h0, output_final_state=bool(use_cache))
+            o = o.view(B, T, D)
+            if use_cache:
+                recurrent_state = new_state.view(B, self.num_heads, self.head_dim)
+
+        if past_key_values is not None:
+            past_key_values.update((recurrent_state,), self.layer_idx, T)
+
+        o = self.g_norm(g, o)
+        o = self.o_proj(o)
+        return o, None, past_key_values
+
+    def init_state(self, batch_size: int) -> Tuple[torch.Tensor]:
+        """Zero recurrent state [B, num_heads, head_dim], kept in fp32."""
+        param = next(self.parameters())
+        return (torch.zeros(batch_size, self.num_heads, self.head_dim, dtype=torch.float32, device=param.device),)
+
+    def state_size(self, **kwargs) -> int:
+        return self.hidden_size

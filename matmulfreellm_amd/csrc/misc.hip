@@ -1,0 +1,86 @@
+// Embedding row gather and greedy argmax: the two ends of a decode step, kept as plain
+// kernels so the whole step can be captured into one HIP graph without library calls.
+//
+// mmf_embedding replaces nn.Embedding.forward at mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py:212;
+// mmf_argmax replaces the argmax over the vocabulary that greedy decoding performs on the
+// logits of HGRNBitForCausalLM.forward (modeling_hgrn_bit.py:386).  Ties go to the lowest
+// index (BitLinear logits are integer accumulators times two scalars, so exact ties happen).
+#include "mmf_common.h"
+
+namespace {
+
+template <typename T>
+__global__ __launch_bounds__(256) void embedding_kernel(const T* __restrict__ table, const int64_t* __restrict__ ids,
+                                                        T* __restrict__ out, int64_t rows, int64_t H, int64_t vocab) {
+    const int64_t r = blockIdx.x;
+    int64_t id = ids[r];
+    if (id < 0 || id >= vocab) id = 0;   // out-of-range ids read row 0 instead of faulting
+    const T* src = table + id * H;
+    T* dst = out + r * H;
+    for (int64_t c = threadIdx.x; c < H; c += 256) dst[c] = src[c];
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void argmax_kernel(const T* __restrict__ logits, int64_t ld, int64_t V,
+                                                     int64_t* __restrict__ out) {
+    __shared__ float best_v[4];
+    __shared__ int64_t best_i[4];
+    const int64_t r = blockIdx.x;
+    const T* row = logits + r * ld;
+    float bv = -INFINITY;
+    int64_t bi = V;   // larger than any valid index
+    for (int64_t c = threadIdx.x; c < V; c += 256) {
+        const float v = mmf_to_float(row[c]);
+        if (v > bv || (v == bv && c < bi) || (bi == V && !(v != v))) { bv = v; bi = c; }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, 64);
+        const int64_t oi = __shfl_xor(bi, o, 64);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) { best_v[w] = bv; best_i[w] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < 4; ++i)
+            if (best_v[i] > bv || (best_v[i] == bv && best_i[i] < bi)) { bv = best_v[i]; bi = best_i[i]; }
+        out[r] = bi < V ? bi : 0;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int mmf_embedding(const void* table, const int64_t* ids, void* out, int64_t rows, int64_t H, int64_t vocab, int dtype,
+                  void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (rows < 0 || H <= 0 || vocab <= 0) return MMF_ERR_ARG;
+    if (rows == 0) return 0;
+    if (!table || !ids || !out) return MMF_ERR_ARG;
+    switch (dtype) {
+        case MMF_F32: embedding_kernel<float><<<(unsigned)rows, 256, 0, stream>>>(static_cast<const float*>(table), ids, static_cast<float*>(out), rows, H, vocab); break;
+        case MMF_BF16: embedding_kernel<bf16_t><<<(unsigned)rows, 256, 0, stream>>>(static_cast<const bf16_t*>(table), ids, static_cast<bf16_t*>(out), rows, H, vocab); break;
+        case MMF_F16: embedding_kernel<f16_t><<<(unsigned)rows, 256, 0, stream>>>(static_cast<const f16_t*>(table), ids, static_cast<f16_t*>(out), rows, H, vocab); break;
+        default: return MMF_ERR_ARG;
+    }
+    MMF_CHECK_LAUNCH();
+    return 0;
+}
+
+int mmf_argmax(const void* logits, int64_t ld, int64_t rows, int64_t V, int64_t* out, int dtype, void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (rows < 0 || V <= 0 || ld < V) return MMF_ERR_ARG;
+    if (rows == 0) return 0;
+    if (!logits || !out) return MMF_ERR_ARG;
+    switch (dtype) {
+        case MMF_F32: argmax_kernel<float><<<(unsigned)rows, 256, 0, stream>>>(static_cast<const float*>(logits), ld, V, out); break;
+        case MMF_BF16: argmax_kernel<bf16_t><<<(unsigned)rows, 256, 0, stream>>>(static_cast<const bf16_t*>(logits), ld, V, out); break;
+        case MMF_F16: argmax_kernel<f16_t><<<(unsigned)rows, 256, 0, stream>>>(static_cast<const f16_t*>(logits), ld, V, out); break;
+        default: return MMF_ERR_ARG;
+    }
+    MMF_CHECK_LAUNCH();
+    return 0;
+}
+
+}  // extern "C"

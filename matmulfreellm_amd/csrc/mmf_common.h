@@ -1,0 +1,206 @@
+// Shared device helpers for the MatMul-free LM hot-path kernels (gfx950, wave64).
+//
+// Arithmetic contract used by every kernel in this directory:
+//  * all floating-point math is fp32 (fp64 only for sums of squares / |w|), one
+//    IEEE-rounded operation at a time: the files are compiled with
+//    -ffp-contract=off and the helpers below use the __f*_rn intrinsics, so no
+//    multiply-add is ever fused;
+//  * division and sqrt are the correctly rounded ones;
+//  * rounding to integer codes is round-half-to-even (rintf);
+//  * exp is mmf_exp() below, built from add/mul only, so a CPU restatement can
+//    reproduce every result bit for bit.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+// Keep every multiply and add separately rounded in all code that includes this header,
+// whatever -ffp-contract the translation unit is built with.
+#pragma clang fp contract(off)
+
+#include "../../include/mmf.h"   // dtype ids, error codes, entry-point declarations
+
+#define MMF_CHECK_LAUNCH()                          \
+    do {                                            \
+        hipError_t e__ = hipGetLastError();         \
+        if (e__ != hipSuccess) return (int)e__;     \
+    } while (0)
+
+struct bf16_t { uint16_t v; };
+struct f16_t { _Float16 v; };
+
+// ---------------------------------------------------------------- scalar conversions
+__device__ __forceinline__ float mmf_to_float(float x) { return x; }
+__device__ __forceinline__ float mmf_to_float(bf16_t x) { return __uint_as_float(((uint32_t)x.v) << 16); }
+__device__ __forceinline__ float mmf_to_float(f16_t x) { return (float)x.v; }
+
+__device__ __forceinline__ uint16_t mmf_f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);  // quiet NaN
+    u += 0x7fffu + ((u >> 16) & 1u);                                            // nearest even
+    return (uint16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ T mmf_from_float(float f);
+template <> __device__ __forceinline__ float mmf_from_float<float>(float f) { return f; }
+template <> __device__ __forceinline__ bf16_t mmf_from_float<bf16_t>(float f) { bf16_t r; r.v = mmf_f32_to_bf16_bits(f); return r; }
+template <> __device__ __forceinline__ f16_t mmf_from_float<f16_t>(float f) { f16_t r; r.v = (_Float16)f; return r; }
+
+// Round an fp32 value to T and bring it back (what a materialised tensor would hold).
+template <typename T> __device__ __forceinline__ float mmf_round_to(float f) { return mmf_to_float(mmf_from_float<T>(f)); }
+
+// ---------------------------------------------------------------- 8-element vectors
+// Rows are processed 8 elements at a time: one 16-byte load for bf16/f16, two for fp32.
+template <typename T> struct Vec8;
+template <> struct Vec8<float> { float4 a, b; };
+template <> struct Vec8<bf16_t> { uint4 a; };
+template <> struct Vec8<f16_t> { uint4 a; };
+
+template <typename T>
+__device__ __forceinline__ void mmf_load8(const T* __restrict__ p, int64_t k0, int64_t K, bool vec_ok, float (&out)[8]) {
+    if (vec_ok) {
+        if constexpr (sizeof(T) == 4) {
+            const float4* q = reinterpret_cast<const float4*>(p + k0);
+            float4 a = q[0], b = q[1];
+            out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+            out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+        } else {
+            uint4 a = *reinterpret_cast<const uint4*>(p + k0);
+            const T* e = reinterpret_cast<const T*>(&a);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) out[i] = mmf_to_float(e[i]);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] = (k0 + i < K) ? mmf_to_float(p[k0 + i]) : 0.0f;
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ void mmf_store8(T* __restrict__ p, int64_t k0, int64_t K, bool vec_ok, const float (&in)[8]) {
+    if (vec_ok) {
+        if constexpr (sizeof(T) == 4) {
+            float4* q = reinterpret_cast<float4*>(p + k0);
+            q[0] = make_float4(in[0], in[1], in[2], in[3]);
+            q[1] = make_float4(in[4], in[5], in[6], in[7]);
+        } else {
+            uint4 a;
+            T* e = reinterpret_cast<T*>(&a);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) e[i] = mmf_from_float<T>(in[i]);
+            *reinterpret_cast<uint4*>(p + k0) = a;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (k0 + i < K) p[k0 + i] = mmf_from_float<T>(in[i]);
+    }
+}
+
+// ---------------------------------------------------------------- deterministic exp
+// Cody-Waite reduction by ln2, degree-5 Horner polynomial, two-step 2^n scaling.
+// Every operation is a separately rounded fp32 add or multiply.
+__device__ __forceinline__ float mmf_exp(float x) {
+    if (x != x) return x;
+    float xc = fminf(fmaxf(x, -104.0f), 89.0f);
+    float n = rintf(__fmul_rn(xc, 1.44269504088896341f));
+    float r = __fsub_rn(xc, __fmul_rn(n, 0.693359375f));
+    r = __fsub_rn(r, __fmul_rn(n, -2.12194440e-4f));
+    float z = __fmul_rn(r, r);
+    float p = 1.9875691500e-4f;
+    p = __fadd_rn(__fmul_rn(p, r), 1.3981999507e-3f);
+    p = __fadd_rn(__fmul_rn(p, r), 8.3334519073e-3f);
+    p = __fadd_rn(__fmul_rn(p, r), 4.1665795894e-2f);
+    p = __fadd_rn(__fmul_rn(p, r), 1.6666665459e-1f);
+    p = __fadd_rn(__fmul_rn(p, r), 5.0000001201e-1f);
+    float y = __fmul_rn(p, z);
+    y = __fadd_rn(y, r);
+    y = __fadd_rn(y, 1.0f);
+    int ni = (int)n;
+    int n1 = ni >> 1;
+    int n2 = ni - n1;
+    y = __fmul_rn(y, __int_as_float((n1 + 127) << 23));
+    y = __fmul_rn(y, __int_as_float((n2 + 127) << 23));
+    return y;
+}
+
+// 1 / (1 + exp(-x))
+__device__ __forceinline__ float mmf_sigmoid(float x) {
+    return __fdiv_rn(1.0f, __fadd_rn(1.0f, mmf_exp(-x)));
+}
+
+// ---------------------------------------------------------------- reductions (wave64 butterfly)
+__device__ __forceinline__ double mmf_wave_sum(double v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float mmf_wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ int mmf_wave_sum(int v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// Block-wide reductions for blocks of NW waves; `red` is LDS scratch of >= NW entries
+// that the caller does not otherwise touch between the two barriers.  The per-wave
+// partials are combined in index order by every thread, so all threads (and all
+// blocks reducing the same data) see the same bits.
+template <int NW>
+__device__ __forceinline__ double mmf_block_sum(double v, double* red) {
+    v = mmf_wave_sum(v);
+    if constexpr (NW == 1) return v;
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    double s = red[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) s += red[i];
+    __syncthreads();
+    return s;
+}
+template <int NW>
+__device__ __forceinline__ float mmf_block_max(float v, float* red) {
+    v = mmf_wave_max(v);
+    if constexpr (NW == 1) return v;
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float s = red[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) s = fmaxf(s, red[i]);
+    __syncthreads();
+    return s;
+}
+template <int NW>
+__device__ __forceinline__ int mmf_block_sum(int v, int* red) {
+    v = mmf_wave_sum(v);
+    if constexpr (NW == 1) return v;
+    const int w = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    int s = red[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) s += red[i];
+    __syncthreads();
+    return s;
+}
+
+// rstd = 1 / sqrt( fp32(sumsq / K) + eps )
+__device__ __forceinline__ float mmf_rstd(double sumsq, int64_t K, float eps) {
+    float var = (float)(sumsq / (double)K);
+    return __fdiv_rn(1.0f, sqrtf(__fadd_rn(var, eps)));   // sqrtf: correctly rounded (__fsqrt_rn is the native approximation)
+}
+
+// int8 code of one normalised value:  clamp(rint(y * scale), -128, 127)
+__device__ __forceinline__ int mmf_code(float y, float scale) {
+    float r = rintf(__fmul_rn(y, scale));
+    r = fminf(fmaxf(r, -128.0f), 127.0f);
+    return (int)r;
+}
+
+__host__ __device__ static inline int64_t mmf_ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+__host__ __device__ static inline int64_t mmf_round_up(int64_t a, int64_t b) { return mmf_ceil_div(a, b) * b; }

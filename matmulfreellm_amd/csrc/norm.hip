@@ -1,0 +1,290 @@
+// One-pass row kernels: RMSNorm, RMSNorm * swish-gate, RMSNorm + int8 quantiser, swiglu.
+//
+// One workgroup of 256 threads owns one row; the row lives in registers (8-element
+// vectors, up to NV per thread), sums of squares are reduced in fp64 with a wave64
+// butterfly plus a 4-entry LDS exchange, so HBM sees each input once and each output
+// once.  Replaces the Triton row kernels at mmfreelm/modules/layernorm.py:104-165,
+// mmfreelm/modules/fused_norm_gate.py:68-131, mmfreelm/ops/fusedbitnet.py:63-131 and
+// the jiterator kernel at mmfreelm/modules/activations.py:115-119.
+#include "mmf_common.h"
+#include "../../include/mmf.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / 64;
+
+enum RowMode : int { ROW_NORM = 0, ROW_GATE = 1, ROW_QUANT = 2 };
+
+struct RowArgs {
+    const void* x;          // [M, K]
+    const void* residual;   // [M, K] or null            (dtype TR)
+    const void* gate;       // [M, K] or null            (ROW_GATE, dtype T)
+    const void* weight;     // [K] or null               (dtype TW)
+    void* y;                // [M, K] T                  (ROW_NORM / ROW_GATE)
+    void* residual_out;     // [M, K] TR or null
+    int8_t* q;              // codes                     (ROW_QUANT)
+    float* deq;             // [M]
+    int* qsum;              // [M]
+    int64_t M, K, Kp, ldx;   // ldx: row stride of x in elements
+    float eps;
+    int q_tiled;            // 0: row-major [M, Kp]; 1: [ceil32(M)/32][Kp/16][32][16]
+};
+
+template <typename T, typename TR, typename TW, int MODE, int NV>
+__global__ __launch_bounds__(kThreads) void row_kernel(RowArgs a) {
+    __shared__ double red_d[kWaves];
+    __shared__ float red_f[kWaves];
+    __shared__ int red_i[kWaves];
+
+    const int64_t row = blockIdx.x;
+    const int64_t K = a.K;
+    const bool vec_ok = (K % 8) == 0;
+    const T* x = static_cast<const T*>(a.x) + row * a.ldx;
+    const TR* res = a.residual ? static_cast<const TR*>(a.residual) + row * K : nullptr;
+    TR* res_out = a.residual_out ? static_cast<TR*>(a.residual_out) + row * K : nullptr;
+    const TW* w = static_cast<const TW*>(a.weight);
+
+    float xv[NV][8];
+    double ss = 0.0;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
+        if (k0 < K) {
+            mmf_load8<T>(x, k0, K, vec_ok, xv[v]);
+            if (res) {
+                float rv[8];
+                mmf_load8<TR>(res, k0, K, vec_ok, rv);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) xv[v][i] = __fadd_rn(xv[v][i], rv[i]);
+            }
+            if (res_out) mmf_store8<TR>(res_out, k0, K, vec_ok, xv[v]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) xv[v][i] = 0.0f;
+        }
+    }
+    ss = mmf_block_sum<kWaves>(ss, red_d);
+    const float rstd = mmf_rstd(ss, K, a.eps);
+
+    float amax = 0.0f;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
+        if (k0 < K) {
+            float wv[8];
+            if (w) mmf_load8<TW>(w, k0, K, vec_ok, wv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float y = __fmul_rn(xv[v][i], rstd);
+                if (w) y = __fmul_rn(y, wv[i]);
+                xv[v][i] = y;
+                amax = fmaxf(amax, fabsf(y));
+            }
+            if constexpr (MODE == ROW_GATE) {
+                float ov[8];
+                mmf_load8<T>(static_cast<const T*>(a.gate) + row * K, k0, K, vec_ok, ov);
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    xv[v][i] = __fmul_rn(__fmul_rn(xv[v][i], ov[i]), mmf_sigmoid(ov[i]));
+            }
+            if constexpr (MODE != ROW_QUANT)
+                mmf_store8<T>(static_cast<T*>(a.y) + row * K, k0, K, vec_ok, xv[v]);
+        }
+    }
+    if constexpr (MODE != ROW_QUANT) return;
+
+    amax = mmf_block_max<kWaves>(amax, red_f);
+    const float amaxc = fmaxf(amax, 1e-5f);
+    const float scale = __fdiv_rn(127.0f, amaxc);
+    int qs = 0;
+    const int64_t Kp = a.Kp;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
+        if (k0 < Kp) {
+            uint32_t lo = 0, hi = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                int c = (k0 + i < K) ? mmf_code(xv[v][i], scale) : 0;   // xv is 0 beyond K
+                qs += c;
+                uint32_t b = (uint32_t)(c & 0xff) << (8 * (i & 3));
+                if (i < 4) lo |= b; else hi |= b;
+            }
+            int64_t off;
+            if (a.q_tiled)
+                off = ((row >> 5) * (Kp >> 4) + (k0 >> 4)) * 512 + (row & 31) * 16 + (k0 & 15);
+            else
+                off = row * Kp + k0;
+            *reinterpret_cast<uint2*>(a.q + off) = make_uint2(lo, hi);
+        }
+    }
+    qs = mmf_block_sum<kWaves>(qs, red_i);
+    if (threadIdx.x == 0) {
+        a.deq[row] = __fdiv_rn(1.0f, scale);
+        a.qsum[row] = qs;
+    }
+}
+
+template <typename T, typename TR, typename TW, int MODE>
+int launch_row(const RowArgs& a, hipStream_t s) {
+    if (a.M == 0) return 0;
+    const int64_t width = (MODE == ROW_QUANT) ? a.Kp : a.K;   // the quantiser also zero-fills the padding
+    const int64_t nv = mmf_ceil_div(width, (int64_t)kThreads * 8);
+    dim3 grid((unsigned)a.M), block(kThreads);
+    if (nv <= 1) row_kernel<T, TR, TW, MODE, 1><<<grid, block, 0, s>>>(a);
+    else if (nv <= 2) row_kernel<T, TR, TW, MODE, 2><<<grid, block, 0, s>>>(a);
+    else if (nv <= 4) row_kernel<T, TR, TW, MODE, 4><<<grid, block, 0, s>>>(a);
+    else if (nv <= 8) row_kernel<T, TR, TW, MODE, 8><<<grid, block, 0, s>>>(a);
+    else return MMF_ERR_WIDE;
+    MMF_CHECK_LAUNCH();
+    return 0;
+}
+
+template <typename T, typename TR, int MODE>
+int dispatch_w(const RowArgs& a, int x_dtype, int w_dtype, hipStream_t s) {
+    // The norm weight is either fp32 or the activation dtype.
+    if (w_dtype == MMF_F32) return launch_row<T, TR, float, MODE>(a, s);
+    if (w_dtype == x_dtype) return launch_row<T, TR, T, MODE>(a, s);
+    return MMF_ERR_ARG;
+}
+
+template <typename T, int MODE>
+int dispatch_r(const RowArgs& a, int x_dtype, int r_dtype, int w_dtype, hipStream_t s) {
+    // The residual stream is either the activation dtype or fp32 (residual_in_fp32).
+    if (r_dtype == MMF_F32) return dispatch_w<T, float, MODE>(a, x_dtype, w_dtype, s);
+    return dispatch_w<T, T, MODE>(a, x_dtype, w_dtype, s);
+}
+
+template <int MODE>
+int dispatch_x(const RowArgs& a, int x_dtype, int r_dtype, int w_dtype, hipStream_t s) {
+    const bool uses_res = a.residual || a.residual_out;
+    if (uses_res && r_dtype != MMF_F32 && r_dtype != x_dtype) return MMF_ERR_ARG;
+    if (!uses_res) r_dtype = x_dtype;
+    if (!a.weight) w_dtype = MMF_F32;
+    switch (x_dtype) {
+        case MMF_F32: return dispatch_r<float, MODE>(a, x_dtype, r_dtype, w_dtype, s);
+        case MMF_BF16: return dispatch_r<bf16_t, MODE>(a, x_dtype, r_dtype, w_dtype, s);
+        case MMF_F16: return dispatch_r<f16_t, MODE>(a, x_dtype, r_dtype, w_dtype, s);
+    }
+    return MMF_ERR_ARG;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---------------------------------------------------------------- swiglu (elementwise)
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_kernel(const T* __restrict__ x, int64_t ldx, const T* __restrict__ y,
+                                                     int64_t ldy, T* __restrict__ out, int64_t rows, int64_t cols) {
+    // cols % 8 == 0; one 8-vector per thread.
+    const int64_t vpr = cols / 8;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= rows * vpr) return;
+    const int64_t r = idx / vpr, c0 = (idx % vpr) * 8;
+    float xv[8], yv[8];
+    mmf_load8<T>(x + r * ldx, c0, cols, true, xv);
+    mmf_load8<T>(y + r * ldy, c0, cols, true, yv);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        xv[i] = __fdiv_rn(__fmul_rn(xv[i], yv[i]), __fadd_rn(1.0f, mmf_exp(-xv[i])));
+    mmf_store8<T>(out + r * cols, c0, cols, true, xv);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_scalar_kernel(const T* __restrict__ x, int64_t ldx, const T* __restrict__ y,
+                                                            int64_t ldy, T* __restrict__ out, int64_t rows, int64_t cols) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= rows * cols) return;
+    const int64_t r = idx / cols, c = idx % cols;
+    const float xv = mmf_to_float(x[r * ldx + c]), yv = mmf_to_float(y[r * ldy + c]);
+    out[r * cols + c] = mmf_from_float<T>(__fdiv_rn(__fmul_rn(xv, yv), __fadd_rn(1.0f, mmf_exp(-xv))));
+}
+
+template <typename T>
+int launch_swiglu(const void* x, int64_t ldx, const void* y, int64_t ldy, void* out, int64_t rows, int64_t cols,
+                  hipStream_t s) {
+    if (rows == 0 || cols == 0) return 0;
+    const int esz = sizeof(T);
+    const bool vec = cols % 8 == 0 && ldx % 8 == 0 && ldy % 8 == 0 && aligned16(x) && aligned16(y) && aligned16(out);
+    (void)esz;
+    if (vec) {
+        const int64_t n = rows * (cols / 8);
+        swiglu_kernel<T><<<(unsigned)mmf_ceil_div(n, 256), 256, 0, s>>>(static_cast<const T*>(x), ldx,
+                                                                       static_cast<const T*>(y), ldy,
+                                                                       static_cast<T*>(out), rows, cols);
+    } else {
+        const int64_t n = rows * cols;
+        swiglu_scalar_kernel<T><<<(unsigned)mmf_ceil_div(n, 256), 256, 0, s>>>(static_cast<const T*>(x), ldx,
+                                                                              static_cast<const T*>(y), ldy,
+                                                                              static_cast<T*>(out), rows, cols);
+    }
+    MMF_CHECK_LAUNCH();
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mmf_rmsnorm(const void* x, const void* residual, const void* weight, void* y, void* residual_out, int64_t M,
+                int64_t K, float eps, int x_dtype, int residual_dtype, int weight_dtype, void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (M < 0 || K <= 0 || (M > 0 && (!x || !y))) return MMF_ERR_ARG;
+    if (K % 8 == 0 && !(aligned16(x) && aligned16(y) && aligned16(residual) && aligned16(residual_out) && aligned16(weight)))
+        return MMF_ERR_ALIGN;
+    RowArgs a{};
+    a.x = x; a.residual = residual; a.weight = weight; a.y = y; a.residual_out = residual_out;
+    a.M = M; a.K = K; a.Kp = K; a.ldx = K; a.eps = eps;
+    return dispatch_x<ROW_NORM>(a, x_dtype, residual_dtype, weight_dtype, stream);
+}
+
+int mmf_rmsnorm_swishgate(const void* x, int64_t ldx, const void* gate, const void* residual, const void* weight, void* y,
+                          void* residual_out, int64_t M, int64_t K, float eps, int x_dtype, int residual_dtype,
+                          int weight_dtype, void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (M < 0 || K <= 0 || ldx < K || (M > 0 && (!x || !y || !gate))) return MMF_ERR_ARG;
+    if (K % 8 == 0 && ldx % 8 != 0) return MMF_ERR_ALIGN;
+    if (K % 8 == 0 && !(aligned16(x) && aligned16(y) && aligned16(gate) && aligned16(residual) &&
+                        aligned16(residual_out) && aligned16(weight)))
+        return MMF_ERR_ALIGN;
+    RowArgs a{};
+    a.x = x; a.gate = gate; a.residual = residual; a.weight = weight; a.y = y; a.residual_out = residual_out;
+    a.M = M; a.K = K; a.Kp = K; a.ldx = ldx; a.eps = eps;
+    return dispatch_x<ROW_GATE>(a, x_dtype, residual_dtype, weight_dtype, stream);
+}
+
+int64_t mmf_codes_bytes(int64_t M, int64_t K, int tiled) {
+    const int64_t Kp = mmf_round_up(K, 128);
+    return (tiled ? mmf_round_up(M, 32) : M) * Kp;
+}
+
+int mmf_rmsnorm_quant(const void* x, const void* residual, const void* weight, int8_t* q, float* deq, int* qsum,
+                      void* residual_out, int64_t M, int64_t K, float eps, int x_dtype, int residual_dtype,
+                      int weight_dtype, int tiled, void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (M < 0 || K <= 0 || (M > 0 && (!x || !q || !deq || !qsum))) return MMF_ERR_ARG;
+    if (!aligned16(q)) return MMF_ERR_ALIGN;
+    if (K % 8 == 0 && !(aligned16(x) && aligned16(residual) && aligned16(residual_out) && aligned16(weight)))
+        return MMF_ERR_ALIGN;
+    RowArgs a{};
+    a.x = x; a.residual = residual; a.weight = weight; a.residual_out = residual_out;
+    a.q = q; a.deq = deq; a.qsum = qsum;
+    a.M = M; a.K = K; a.Kp = mmf_round_up(K, 128); a.ldx = K; a.eps = eps; a.q_tiled = tiled;
+    return dispatch_x<ROW_QUANT>(a, x_dtype, residual_dtype, weight_dtype, stream);
+}
+
+int mmf_swiglu(const void* x, int64_t ldx, const void* y, int64_t ldy, void* out, int64_t rows, int64_t cols,
+               int dtype, void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (rows < 0 || cols < 0 || (rows * cols > 0 && (!x || !y || !out))) return MMF_ERR_ARG;
+    switch (dtype) {
+        case MMF_F32: return launch_swiglu<float>(x, ldx, y, ldy, out, rows, cols, stream);
+        case MMF_BF16: return launch_swiglu<bf16_t>(x, ldx, y, ldy, out, rows, cols, stream);
+        case MMF_F16: return launch_swiglu<f16_t>(x, ldx, y, ldy, out, rows, cols, stream);
+    }
+    return MMF_ERR_ARG;
+}
+
+}  // extern "C"
