@@ -1,0 +1,220 @@
+"""Whole-model single-token decode step as one HIP graph.
+
+The module path (HGRNBitForCausalLM.forward with T = 1) issues the same kernels through
+nn.Module calls and fresh output tensors; at batch 1 that host work dwarfs the ~40 us the
+weights take to stream.  DecodeEngine lays the step out once over static buffers, records it
+into a graph (torch.cuda.CUDAGraph = hipGraph) and replays it per token: embedding gather ->
+L x [RMSNorm, i/f/g BitLinear, gate + recurrence step, gated norm, o_proj BitLinear,
+residual RMSNorm, gate_proj BitLinear, swiglu, down_proj BitLinear (+residual)] -> final
+norm -> lm_head BitLinear -> argmax.  The argmax writes the token buffer the next replay's
+embedding reads, so consecutive steps need no host round trip.
+
+Every launch is the same C-ABI call with the same arithmetic as the module path, so the two
+produce identical bits (tests/test_gpu_model.py checks that).
+"""
+from typing import List, Optional
+
+import torch
+
+from . import _lib as L
+from . import functional as F_
+
+
+class DecodeEngine:
+
+    @classmethod
+    def for_model(cls, model, batch_size: int, use_graph: bool = True):
+        engines = model.__dict__.setdefault("_decode_engines", {})
+        key = (batch_size, use_graph)
+        eng = engines.get(key)
+        if eng is None or eng.stale():
+            eng = cls(model, batch_size, use_graph)
+            engines[key] = eng
+        return eng
+
+    def __init__(self, model, batch_size: int, use_graph: bool = True):
+        cfg = model.config
+        self.lib = L.load()
+        self.model = model
+        self.B = B = batch_size
+        emb = model.model.embeddings.weight
+        self.dev = dev = L.require_gpu(emb)
+        self.dtype = dt = emb.dtype
+        self.dt_id = L.dtype_id(dt)
+        self.H = H = cfg.hidden_size
+        self.V = cfg.vocab_size
+        self.L = len(model.model.layers)
+        self.eps = float(cfg.rms_norm_eps)
+        self.use_graph = use_graph
+        self._version_key = self._param_versions()
+
+        attn0 = model.model.layers[0].attn
+        self.D = D = attn0.input_dim
+        self.I = I = model.model.layers[0].mlp.intermediate_size
+        lbs = model.model.lower_bound_rows() if cfg.use_lower_bound else None
+
+        def z(*shape, dtype=dt):
+            return torch.zeros(*shape, dtype=dtype, device=dev)
+
+        # ---- per-layer operands (references keep the packed weights alive)
+        self.layers = []
+        for li, blk in enumerate(model.model.layers):
+            a, m = blk.attn, blk.mlp
+            ent = {
+                "attn_norm": blk.attn_norm.weight.detach(), "mlp_norm": blk.mlp_norm.weight.detach(),
+                "g_norm": a.g_norm.weight.detach(), "g_eps": float(a.g_norm.eps),
+                "ifg": a._stacked_ifg(),
+                "projs": [(p.packed_weight(), p.norm.weight.detach(), self._eps_of(p)) for p in (a.i_proj, a.f_proj, a.g_proj)],
+                "o": (a.o_proj.packed_weight(), a.o_proj.norm.weight.detach(), self._eps_of(a.o_proj)),
+                "gate": (m.gate_proj.packed_weight(), m.gate_proj.norm.weight.detach(), self._eps_of(m.gate_proj)),
+                "down": (m.down_proj.packed_weight(), m.down_proj.norm.weight.detach(), self._eps_of(m.down_proj)),
+                "lb": lbs[li].contiguous() if (lbs is not None and li > 0) else None,
+                "state": z(B, D, dtype=torch.float32),
+            }
+            for p in (a.i_proj, a.f_proj, a.g_proj, a.o_proj, m.gate_proj, m.down_proj):
+                if p.bias is not None:
+                    raise NotImplementedError("DecodeEngine: BitLinear bias is not on the model path")
+            self.layers.append(ent)
+        self.final_norm = model.model.norm.weight.detach()
+        self.head = (model.lm_head.packed_weight(), model.lm_head.norm.weight.detach(), self._eps_of(model.lm_head))
+        self.table = emb.detach()
+
+        # ---- static activation buffers
+        self.tok = torch.zeros(B, dtype=torch.int64, device=dev)
+        self.h = z(B, H)            # residual stream
+        self.hn = z(B, H)
+        self.ifg = z(B, 3 * D)
+        self.o = z(B, D)
+        self.o2 = z(B, D)
+        self.a = z(B, H)
+        self.res = z(B, H)
+        self.y = z(B, 2 * I)
+        self.zb = z(B, I)
+        self.logits = z(B, self.V)
+        kmax = max(H, D, I)
+        self.q = torch.zeros(self.lib.mmf_codes_bytes(B, kmax, 1), dtype=torch.int8, device=dev)
+        self.deq = z(B, dtype=torch.float32)
+        self.qsum = torch.zeros(B, dtype=torch.int32, device=dev)
+        self.gemv = B <= F_.GEMV_MAX_M
+        self.graph = None
+
+    @staticmethod
+    def _eps_of(p):
+        return float(p.norm.eps if getattr(p, "fused_eps", None) is None else p.fused_eps)
+
+    def _param_versions(self):
+        return tuple((p.data_ptr(), p._version) for p in self.model.parameters())
+
+    def stale(self):
+        return self._param_versions() != self._version_key
+
+    # ------------------------------------------------------------------ launches
+    def _bitlinear(self, x, pw_nw_eps, out, n_k, addend=None):
+        pw, nw, eps = pw_nw_eps
+        lib, s, B = self.lib, L.stream(), self.B
+        n, k = n_k
+        nw_id = L.dtype_id(nw.dtype)
+        if self.gemv and k <= lib.mmf_bitlinear_gemv_max_k():
+            L.check(lib.mmf_bitlinear_gemv(x.data_ptr(), nw.data_ptr(), pw.packed.data_ptr(), pw.wdeq.data_ptr(),
+                                           pw.seg_rows, None, L.ptr(addend), out.data_ptr(), B, k, n, eps, self.dt_id,
+                                           nw_id, s), "mmf_bitlinear_gemv")
+        else:
+            L.check(lib.mmf_rmsnorm_quant(x.data_ptr(), None, nw.data_ptr(), self.q.data_ptr(), self.deq.data_ptr(),
+                                          self.qsum.data_ptr(), None, B, k, eps, self.dt_id, self.dt_id, nw_id, 1, s),
+                    "mmf_rmsnorm_quant")
+            L.check(lib.mmf_bitlinear_mfma(self.q.data_ptr(), self.deq.data_ptr(), self.qsum.data_ptr(),
+                                           pw.packed.data_ptr(), pw.wdeq.data_ptr(), pw.seg_rows, None, L.ptr(addend),
+                                           out.data_ptr(), n, B, k, n, self.dt_id, -1, s), "mmf_bitlinear_mfma")
+
+    def _launch_step(self):
+        lib, s, B, H, D, I = self.lib, L.stream(), self.B, self.H, self.D, self.I
+        dt, esz = self.dt_id, self.h.element_size()
+        wid = L.dtype_id(self.final_norm.dtype)
+        L.check(lib.mmf_embedding(self.table.data_ptr(), self.tok.data_ptr(), self.h.data_ptr(), B, H, self.V, dt, s),
+                "mmf_embedding")
+        for ent in self.layers:
+            L.check(lib.mmf_rmsnorm(self.h.data_ptr(), None, ent["attn_norm"].data_ptr(), self.hn.data_ptr(), None, B, H,
+                                    self.eps, dt, dt, wid, s), "mmf_rmsnorm")
+            if ent["ifg"] is not None:
+                self._bitlinear(self.hn, (ent["ifg"], ent["projs"][0][1], ent["projs"][0][2]), self.ifg, (3 * D, H))
+                ip, fp, gp, ld = self.ifg.data_ptr(), self.ifg.data_ptr() + D * esz, self.ifg.data_ptr() + 2 * D * esz, 3 * D
+            else:
+                # three separate projections into the three column blocks of a [3, B, D] layout
+                bufs = self.ifg.view(3, B, D)
+                for j in range(3):
+                    self._bitlinear(self.hn, ent["projs"][j], bufs[j], (D, H))
+                ip, fp, gp, ld = bufs[0].data_ptr(), bufs[1].data_ptr(), bufs[2].data_ptr(), D
+            L.check(lib.mmf_hgrn_step(ip, ld, fp, ld, L.ptr(ent["lb"]), None, ent["state"].data_ptr(), self.o.data_ptr(),
+                                      B, D, dt, s), "mmf_hgrn_step")
+            L.check(lib.mmf_rmsnorm_swishgate(gp, ld, self.o.data_ptr(), None, ent["g_norm"].data_ptr(),
+                                              self.o2.data_ptr(), None, B, D, ent["g_eps"], dt, dt, wid, s),
+                    "mmf_rmsnorm_swishgate")
+            self._bitlinear(self.o2, ent["o"], self.a, (H, D))
+            L.check(lib.mmf_rmsnorm(self.a.data_ptr(), self.h.data_ptr(), ent["mlp_norm"].data_ptr(), self.hn.data_ptr(),
+                                    self.res.data_ptr(), B, H, self.eps, dt, dt, wid, s), "mmf_rmsnorm")
+            self._bitlinear(self.hn, ent["gate"], self.y, (2 * I, H))
+            L.check(lib.mmf_swiglu(self.y.data_ptr(), 2 * I, self.y.data_ptr() + I * esz, 2 * I, self.zb.data_ptr(), B, I,
+                                   dt, s), "mmf_swiglu")
+            self._bitlinear(self.zb, ent["down"], self.h, (H, I), addend=self.res)
+        L.check(lib.mmf_rmsnorm(self.h.data_ptr(), None, self.final_norm.data_ptr(), self.hn.data_ptr(), None, B, H,
+                                self.eps, dt, dt, wid, s), "mmf_rmsnorm")
+        self._bitlinear(self.hn, self.head, self.logits, (self.V, H))
+        L.check(lib.mmf_argmax(self.logits.data_ptr(), self.V, B, self.V, self.tok.data_ptr(), dt, s), "mmf_argmax")
+
+    def _capture(self):
+        # warm-up launches on a side stream (module loading, attribute setting), then record
+        saved = [e["state"].clone() for e in self.layers]
+        tok = self.tok.clone()
+        side = torch.cuda.Stream(device=self.dev)
+        side.wait_stream(torch.cuda.current_stream(self.dev))
+        with torch.cuda.stream(side):
+            self._launch_step()
+        torch.cuda.current_stream(self.dev).wait_stream(side)
+        torch.cuda.synchronize(self.dev)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self._launch_step()
+        torch.cuda.synchronize(self.dev)
+        for e, sv in zip(self.layers, saved):     # undo the warm-up step's state update
+            e["state"].copy_(sv)
+        self.tok.copy_(tok)
+        self.graph = g
+
+    # ------------------------------------------------------------------ public
+    def load_state(self, states: Optional[List[torch.Tensor]]):
+        """Set the per-layer recurrent states ([B, *, D] tensors, or None for zeros)."""
+        for i, e in enumerate(self.layers):
+            if states is None:
+                e["state"].zero_()
+            else:
+                e["state"].copy_(states[i].reshape(self.B, self.D).to(torch.float32))
+
+    def export_state(self):
+        return [e["state"].clone() for e in self.layers]
+
+    def advance(self):
+        """One decode step from the token buffer; leaves logits in self.logits and the greedy
+        next token in the token buffer (no host synchronisation)."""
+        with torch.cuda.device(self.dev):
+            if not self.use_graph:
+                self._launch_step()
+                return
+            if self.graph is None:
+                self._capture()
+            self.graph.replay()
+
+    def step(self, tokens: torch.Tensor) -> torch.Tensor:
+        """Feed `tokens` [B]; returns the logits buffer [B, V] (overwritten by the next step)."""
+        self.tok.copy_(tokens.reshape(self.B))
+        self.advance()
+        return self.logits
+
+    def greedy(self, first_tokens: torch.Tensor, n_steps: int) -> torch.Tensor:
+        """Run n_steps self-feeding greedy steps starting from first_tokens [B]; returns the
+        [B, n_steps] tokens chosen after each step.  One host synchronisation at the end."""
+        out = torch.empty(n_steps, self.B, dtype=torch.int64, device=self.dev)
+        self.tok.copy_(first_tokens.reshape(self.B))
+        for t in range(n_steps):
+            self.advance()
+            out[t].copy_(self.tok)
+        return out.t().contiguous()

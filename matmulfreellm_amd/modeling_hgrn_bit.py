@@ -1,0 +1,331 @@
+"""HGRNBit model family on the HIP kernels.
+
+Same module tree, parameter names and forward semantics as
+mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py (MLP :29-59, Block :62-113, PreTrainedModel
+:116-156, Model :159-278, ForCausalLM :281-409), so a checkpoint's state dict loads as is.
+Differences, all on the host side:
+  * the recurrent state cache is this package's RecurrentCache, and generation is a plain
+    greedy / top-p loop owned by the class (transformers >= 5 no longer gives
+    PreTrainedModel a generate());
+  * ``logits_to_keep`` lets a caller ask for the last positions' logits only (the
+    reference projects all T positions through the 32000-wide head);
+  * the loss head is not part of the inference path: passing ``labels`` raises.
+"""
+from __future__ import annotations
+
+import math
+import warnings
+from typing import List, Optional, Tuple, Union
+
+import torch
+import torch.nn as nn
+from transformers.modeling_outputs import BaseModelOutputWithPast, CausalLMOutputWithPast
+from transformers.modeling_utils import PreTrainedModel
+
+from . import functional as F_
+from .activations import swiglu
+from .attention import HGRNBitAttention
+from .bitlinear import FusedBitLinear as BitLinear
+from .cache import RecurrentCache
+from .configuration_hgrn_bit import HGRNBitConfig
+from .layernorm import RMSNorm
+
+
+def lower_bound_schedule(lower_bounds: torch.Tensor) -> torch.Tensor:
+    """softmax over layers, cumulative sum, minus the first row (modeling_hgrn_bit.py:231-233).
+
+    Evaluated in fp32 on the host so the values do not depend on a device reduction order;
+    returns an fp32 [L, H] tensor on the parameter's device."""
+    lb = lower_bounds.detach().to(device="cpu", dtype=torch.float32).softmax(0)
+    lb = lb.cumsum(0) - lb[0]
+    return lb.to(lower_bounds.device)
+
+
+class HGRNBitMLP(nn.Module):
+
+    def __init__(self, hidden_size: int, hidden_ratio: Optional[int] = None, intermediate_size: Optional[int] = None,
+                 hidden_act: str = "swish"):
+        super().__init__()
+        self.hidden_size = hidden_size
+        if hidden_ratio is None:
+            hidden_ratio = 4
+        if intermediate_size is None:
+            intermediate_size = int(hidden_size * hidden_ratio * 2 / 3)
+            intermediate_size = 256 * ((intermediate_size + 256 - 1) // 256)
+        self.hidden_ratio = hidden_ratio
+        self.intermediate_size = intermediate_size
+        if hidden_act not in ("swish", "silu"):
+            raise NotImplementedError(f"hidden_act={hidden_act!r}: the fused gate is swish")
+        self.gate_proj = BitLinear(self.hidden_size, self.intermediate_size * 2, bias=False)
+        self.down_proj = BitLinear(self.intermediate_size, self.hidden_size, bias=False)
+
+    def forward(self, x, residual=None):
+        """down_proj(swiglu(gate, y)); with ``residual`` the block's closing add is fused into
+        the contraction's epilogue."""
+        y = self.gate_proj(x)
+        gate, y = y.chunk(2, -1)
+        z = swiglu(gate, y)
+        if residual is None:
+            return self.down_proj(z)
+        p = self.down_proj
+        eps = p.norm.eps if p.fused_eps is None else p.fused_eps
+        return F_.bitlinear(z, p.norm.weight, p.packed_weight(), bias=p.bias, eps=eps, addend=residual.contiguous())
+
+
+class HGRNBitBlock(nn.Module):
+
+    def __init__(self, config: HGRNBitConfig, layer_idx: int):
+        super().__init__()
+        self.hidden_size = config.hidden_size
+        self.attn_norm = RMSNorm(hidden_size=config.hidden_size, eps=config.rms_norm_eps)
+        self.attn = HGRNBitAttention(
+            mode=config.attn_mode, hidden_size=config.hidden_size, num_heads=config.num_heads,
+            expand_ratio=config.expand_ratio, use_short_conv=config.use_short_conv, conv_size=config.conv_size,
+            share_conv_kernel=config.share_conv_kernel, layernorm_eps=config.rms_norm_eps, layer_idx=layer_idx)
+        self.mlp_norm = RMSNorm(hidden_size=config.hidden_size, eps=config.rms_norm_eps)
+        self.mlp = HGRNBitMLP(hidden_size=config.hidden_size, hidden_ratio=config.hidden_ratio,
+                              intermediate_size=config.intermediate_size, hidden_act=config.hidden_act)
+
+    def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
+                past_key_values=None, use_cache: Optional[bool] = False, output_attentions: Optional[bool] = False,
+                lower_bound: Optional[torch.Tensor] = None, **kwargs):
+        residual = hidden_states
+        hidden_states = self.attn_norm(hidden_states)
+        hidden_states, attentions, past_key_values = self.attn(
+            hidden_states=hidden_states, attention_mask=attention_mask, past_key_values=past_key_values,
+            use_cache=use_cache, output_attentions=output_attentions, lower_bound=lower_bound)
+        hidden_states, residual = self.mlp_norm(hidden_states, residual, True)
+        hidden_states = self.mlp(hidden_states, residual=residual)      # = residual + mlp(hidden_states)
+        return hidden_states, attentions, past_key_values
+
+
+class HGRNBitPreTrainedModel(PreTrainedModel):
+    config_class = HGRNBitConfig
+    base_model_prefix = "model"
+    supports_gradient_checkpointing = False
+    _no_split_modules = ["HGRNBitBlock"]
+
+    def _init_weights(self, module: nn.Module, rescale_prenorm_residual: bool = True, num_residuals_per_layer: int = 2):
+        if isinstance(module, (nn.Linear, nn.Conv1d)):
+            nn.init.normal_(module.weight, mean=0.0, std=self.config.initializer_range)
+            if module.bias is not None:
+                nn.init.zeros_(module.bias)
+        elif isinstance(module, nn.Embedding):
+            nn.init.normal_(module.weight, mean=0.0, std=self.config.initializer_range)
+            if module.padding_idx is not None:
+                module.weight.data[module.padding_idx].zero_()
+        elif isinstance(module, HGRNBitModel) and getattr(module, "lower_bounds", None) is not None:
+            nn.init.zeros_(module.lower_bounds)
+        if hasattr(module, "weight") and module.weight is not None and type(module).__name__ in (
+                "RMSNorm", "FusedRMSNormSwishGate"):
+            nn.init.ones_(module.weight)
+        if rescale_prenorm_residual:
+            for name, p in module.named_parameters():
+                if name in ["o_proj.weight", "down_proj.weight"]:
+                    with torch.no_grad():
+                        p /= math.sqrt(num_residuals_per_layer * self.config.num_hidden_layers)
+
+
+class HGRNBitModel(HGRNBitPreTrainedModel):
+
+    def __init__(self, config: HGRNBitConfig):
+        super().__init__(config)
+        self.padding_idx = config.pad_token_id
+        self.vocab_size = config.vocab_size
+        self.embeddings = nn.Embedding(config.vocab_size, config.hidden_size, self.padding_idx)
+        if config.use_lower_bound:
+            self.lower_bounds = nn.Parameter(torch.zeros(config.num_hidden_layers, config.hidden_size))
+        self.layers = nn.ModuleList([HGRNBitBlock(config, i) for i in range(config.num_hidden_layers)])
+        self.norm = RMSNorm(config.hidden_size, eps=config.rms_norm_eps)
+        self.gradient_checkpointing = False
+        self._lb_key, self._lb = None, None
+        self.post_init()
+
+    def get_input_embeddings(self):
+        return self.embeddings
+
+    def set_input_embeddings(self, value):
+        self.embeddings = value
+
+    def lower_bound_rows(self):
+        """fp32 [L, H] lower bounds, recomputed only when the parameter changes."""
+        p = self.lower_bounds
+        key = (p.data_ptr(), p._version, p.device)
+        if key != self._lb_key:
+            self._lb_key, self._lb = key, lower_bound_schedule(p)
+        return self._lb
+
+    @torch.no_grad()
+    def forward(self, input_ids: Optional[torch.LongTensor] = None, attention_mask: Optional[torch.Tensor] = None,
+                inputs_embeds: Optional[torch.FloatTensor] = None, past_key_values=None,
+                use_cache: Optional[bool] = None, output_attentions: Optional[bool] = None,
+                output_hidden_states: Optional[bool] = None, return_dict: Optional[bool] = None
+                ) -> Union[Tuple, BaseModelOutputWithPast]:
+        if output_attentions:
+            warnings.warn("`HGRNBitModel` does not `output_attentions` now, setting it to `False`.")
+        output_attentions = False
+        output_hidden_states = bool(output_hidden_states) if output_hidden_states is not None else \
+            bool(getattr(self.config, "output_hidden_states", False))
+        use_cache = use_cache if use_cache is not None else (self.config.use_cache if not self.training else False)
+        return_dict = return_dict if return_dict is not None else bool(getattr(self.config, "return_dict", True))
+
+        if input_ids is not None and inputs_embeds is not None:
+            raise ValueError("You cannot specify both input_ids and inputs_embeds at the same time")
+        elif input_ids is not None:
+            batch_size = input_ids.shape[0]
+        elif inputs_embeds is not None:
+            batch_size = inputs_embeds.shape[0]
+        else:
+            raise ValueError("You have to specify either input_ids or inputs_embeds")
+
+        if inputs_embeds is None:
+            inputs_embeds = F_.embedding(self.embeddings.weight, input_ids)
+        hidden_states = inputs_embeds
+
+        if use_cache:
+            if past_key_values is None:
+                past_key_values = [layer.attn.init_state(batch_size) for layer in self.layers]
+            if not isinstance(past_key_values, RecurrentCache):
+                past_key_values = RecurrentCache.from_legacy_cache(past_key_values)
+
+        all_hidden_states = () if output_hidden_states else None
+        lower_bounds = self.lower_bound_rows() if self.config.use_lower_bound else None
+        for i, layer in enumerate(self.layers):
+            if output_hidden_states:
+                all_hidden_states += (hidden_states,)
+            lower_bound = lower_bounds[i] if lower_bounds is not None else None
+            hidden_states, _, past_key_values = layer(
+                hidden_states, attention_mask=attention_mask, past_key_values=past_key_values, use_cache=use_cache,
+                output_attentions=False, lower_bound=lower_bound)
+
+        hidden_states = self.norm(hidden_states)
+        if output_hidden_states:
+            all_hidden_states += (hidden_states,)
+
+        next_cache = past_key_values if use_cache else None
+        if not return_dict:
+            return tuple(x for x in [hidden_states, next_cache, all_hidden_states] if x is not None)
+        return BaseModelOutputWithPast(last_hidden_state=hidden_states, past_key_values=next_cache,
+                                       hidden_states=all_hidden_states, attentions=None)
+
+
+class HGRNBitForCausalLM(HGRNBitPreTrainedModel):
+    _tied_weights_keys = {}
+
+    def __init__(self, config):
+        super().__init__(config)
+        self.model = HGRNBitModel(config)
+        self.vocab_size = config.vocab_size
+        self.lm_head = BitLinear(config.hidden_size, config.vocab_size, bias=False)
+        self.post_init()
+
+    def get_input_embeddings(self):
+        return self.model.embeddings
+
+    def set_input_embeddings(self, value):
+        self.model.embeddings = value
+
+    def get_output_embeddings(self):
+        return self.lm_head
+
+    def set_output_embeddings(self, new_embeddings):
+        self.lm_head = new_embeddings
+
+    def set_decoder(self, decoder):
+        self.model = decoder
+
+    def get_decoder(self):
+        return self.model
+
+    def prepare_inputs_for_generation(self, input_ids: torch.LongTensor = None, past_key_values=None,
+                                      attention_mask: Optional[torch.Tensor] = None,
+                                      inputs_embeds: Optional[torch.Tensor] = None, **kwargs):
+        """modeling_hgrn_bit.py:326-354: keep only the last token once a cache exists."""
+        if past_key_values is not None:
+            if not isinstance(past_key_values, RecurrentCache):
+                past_key_values = RecurrentCache.from_legacy_cache(past_key_values, input_ids.shape[1] - 1)
+            input_ids = input_ids[:, -1:]
+            if attention_mask is not None:
+                attention_mask = attention_mask[:, -1:]
+        if inputs_embeds is not None and past_key_values is None:
+            model_inputs = {"inputs_embeds": inputs_embeds}
+        else:
+            model_inputs = {"input_ids": input_ids.contiguous()}
+        model_inputs.update({"past_key_values": past_key_values, "use_cache": kwargs.get("use_cache"),
+                             "attention_mask": attention_mask})
+        return model_inputs
+
+    @torch.no_grad()
+    def forward(self, input_ids: torch.LongTensor = None, attention_mask: Optional[torch.Tensor] = None,
+                inputs_embeds: Optional[torch.Tensor] = None, past_key_values=None,
+                labels: Optional[torch.LongTensor] = None, use_cache: Optional[bool] = None,
+                output_attentions: Optional[bool] = None, output_hidden_states: Optional[bool] = None,
+                return_dict: Optional[bool] = None, logits_to_keep: int = 0) -> Union[Tuple, CausalLMOutputWithPast]:
+        if labels is not None:
+            raise NotImplementedError("the loss head (fused cross entropy) is a training component; "
+                                      "this package implements the inference forward only")
+        return_dict = return_dict if return_dict is not None else bool(getattr(self.config, "return_dict", True))
+        outputs = self.model(input_ids=input_ids, attention_mask=attention_mask, inputs_embeds=inputs_embeds,
+                             past_key_values=past_key_values, use_cache=use_cache,
+                             output_attentions=output_attentions, output_hidden_states=output_hidden_states,
+                             return_dict=True)
+        hidden_states = outputs.last_hidden_state
+        if logits_to_keep:
+            hidden_states = hidden_states[:, -logits_to_keep:, :]
+        logits = self.lm_head(hidden_states)
+        if not return_dict:
+            return tuple(x for x in (logits, outputs.past_key_values, outputs.hidden_states) if x is not None)
+        return CausalLMOutputWithPast(loss=None, logits=logits, past_key_values=outputs.past_key_values,
+                                      hidden_states=outputs.hidden_states, attentions=None)
+
+    # ------------------------------------------------------------------ generation
+    @torch.no_grad()
+    def generate(self, input_ids: torch.LongTensor, attention_mask: Optional[torch.Tensor] = None,
+                 max_new_tokens: Optional[int] = None, max_length: Optional[int] = None, do_sample: bool = False,
+                 top_p: float = 1.0, temperature: float = 1.0, eos_token_id: Optional[int] = None,
+                 use_graph: bool = True, generator: Optional[torch.Generator] = None, **kwargs) -> torch.LongTensor:
+        """Greedy (default) or top-p sampling; returns [B, T + new] token ids like HF's generate.
+
+        Prefill runs the module path with last-position logits only; decode runs the captured
+        whole-step HIP graph of DecodeEngine when use_graph is set (greedy, no padding mask)."""
+        if max_new_tokens is None:
+            max_new_tokens = (max_length - input_ids.shape[1]) if max_length is not None else 20
+        B = input_ids.shape[0]
+        out = self(input_ids=input_ids, attention_mask=attention_mask, use_cache=True, logits_to_keep=1)
+        cache = out.past_key_values
+        logits = out.logits[:, -1, :]
+        tokens = [input_ids]
+        finished = torch.zeros(B, dtype=torch.bool, device=input_ids.device)
+        engine = None
+        if use_graph and not do_sample and max_new_tokens > 1:
+            from .decode import DecodeEngine
+            engine = DecodeEngine.for_model(self, B)
+            engine.load_state([c[-1] for c in cache])
+        for step in range(max_new_tokens):
+            if do_sample:
+                nxt = _sample_top_p(logits.float(), top_p, temperature, generator)
+            else:
+                nxt = F_.argmax(logits)
+            if eos_token_id is not None:
+                nxt = torch.where(finished, torch.full_like(nxt, eos_token_id), nxt)
+                finished |= nxt == eos_token_id
+            tokens.append(nxt.view(B, 1))
+            if step == max_new_tokens - 1 or (eos_token_id is not None and bool(finished.all())):
+                break
+            if engine is not None:
+                logits = engine.step(nxt)
+            else:
+                out = self(input_ids=nxt.view(B, 1), past_key_values=cache, use_cache=True)
+                cache = out.past_key_values
+                logits = out.logits[:, -1, :]
+        return torch.cat(tokens, dim=1)
+
+
+def _sample_top_p(logits, top_p, temperature, generator):
+    probs = torch.softmax(logits / max(temperature, 1e-6), dim=-1)
+    sp, si = torch.sort(probs, dim=-1, descending=True)
+    keep = (sp.cumsum(-1) - sp) < top_p
+    sp = sp * keep
+    sp = sp / sp.sum(-1, keepdim=True)
+    choice = torch.multinomial(sp, 1, generator=generator)
+    return si.gather(-1, choice).squeeze(-1)

@@ -154,20 +154,21 @@ def test_rmsnorm_quant_codes(dev, dtype, mk, tiled):
 
 
 def test_rmsnorm_quant_ties_and_zero_rows(dev):
-    # rows built so that y*scale lands exactly on .5 ties: amax = 127 -> scale = 1 after a unit-rms trick is not
-    # possible through the norm, so test the stage on rows whose rstd is a power of two.
-    k = 256
-    base = torch.zeros(4, k)
-    base[0, 0] = 16.0                       # mean(x^2) = 1 -> rstd = 1 (eps negligible in fp32)
-    base[1, :] = 0.0                        # all-zero row: codes 0, scale 127/1e-5
-    base[2, :4] = torch.tensor([127.0, 0.5, 1.5, 2.5])
-    base[3, :4] = torch.tensor([-127.0, -0.5, -1.5, -2.5])
-    x = base.float()
-    q_ref, deq_ref, qsum_ref, _ = on.rms_norm_quant_spec(x, None, eps=0.0)
-    q, deq, qsum = F().rmsnorm_quant(x.to(dev), None, eps=0.0)
-    assert torch.equal(q[:, :k].cpu(), q_ref)
-    assert torch.equal(deq.cpu(), deq_ref) and torch.equal(qsum.cpu(), qsum_ref)
-    assert q[1].abs().sum().item() == 0
+    """Rows whose mean square is exactly 1 (so rstd = 1, scale = 127/127 = 1) put y*scale on exact .5 ties:
+    the codes must be the round-half-to-even integers, sign-symmetric; an all-zero row gives all-zero codes."""
+    k = 16384
+    row = torch.zeros(k)
+    vals = torch.tensor([127.0, 0.5, 1.5, 2.5, 15.0, 4.0, 2.0, 1.0, 0.5])     # sum of squares = 16384 = k
+    row[:9] = vals
+    x = torch.stack([row, -row, torch.zeros(k)]).float()
+    q_ref, deq_ref, qsum_ref, _ = on.rms_norm_quant_spec(x, None, eps=1e-8)
+    assert q_ref[0, :9].tolist() == [127, 0, 2, 2, 15, 4, 2, 1, 0]             # hand-computed known answer
+    assert q_ref[1, :9].tolist() == [-127, 0, -2, -2, -15, -4, -2, -1, 0]
+    for dtype in (torch.float32, torch.bfloat16):
+        q, deq, qsum = F().rmsnorm_quant(x.to(dtype).to(dev), None, eps=1e-8)
+        assert torch.equal(q[:, :k].cpu(), q_ref)
+        assert torch.equal(deq.cpu(), deq_ref) and torch.equal(qsum.cpu(), qsum_ref)
+        assert q[2].abs().sum().item() == 0
 
 
 # ------------------------------------------------------------------ BitLinear
