@@ -59,12 +59,29 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
         if (kb < KB) wreg[i] = a.packed[(nb * KB + kb) * 64 + lane];
     }
 
-    // ---- prologue: RMSNorm + absmax int8 codes of row `row` into LDS
+    // ---- prologue: RMSNorm + absmax int8 codes of row `row` into LDS.  All global loads the
+    // kernel will ever need (x, norm weight, and the epilogue's scale / bias / addend) are
+    // issued here, back to back, so the kernel pays one memory round trip, not four.
     const bool vec_ok = (K % 8) == 0;
     const T* x = static_cast<const T*>(a.x) + row * K;
     const TW* nw = static_cast<const TW*>(a.norm_w);
     float xv[NV][8];
+    float wv[NV][8];
+    float ep_wdeq = 0.0f, ep_bias = 0.0f, ep_add = 0.0f;
+    if (threadIdx.x < 32) {
+        const int64_t n = nb * 32 + threadIdx.x;
+        if (n < a.N) {
+            ep_wdeq = a.wdeq[n / a.seg_rows];
+            if (a.bias) ep_bias = mmf_to_float(static_cast<const T*>(a.bias)[n]);
+            if (a.addend) ep_add = mmf_to_float(static_cast<const T*>(a.addend)[row * a.N + n]);
+        }
+    }
     double ss = 0.0;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int64_t k0 = ((int64_t)v * kGemvThreads + threadIdx.x) * 8;
+        if (k0 < K && nw) mmf_load8<TW>(nw, k0, K, vec_ok, wv[v]);
+    }
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
         const int64_t k0 = ((int64_t)v * kGemvThreads + threadIdx.x) * 8;
@@ -84,12 +101,10 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
     for (int v = 0; v < NV; ++v) {
         const int64_t k0 = ((int64_t)v * kGemvThreads + threadIdx.x) * 8;
         if (k0 < K) {
-            float wv[8];
-            if (nw) mmf_load8<TW>(nw, k0, K, vec_ok, wv);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 float y = __fmul_rn(xv[v][i], rstd);
-                if (nw) y = __fmul_rn(y, wv[i]);
+                if (nw) y = __fmul_rn(y, wv[v][i]);
                 xv[v][i] = y;
                 amax = fmaxf(amax, fabsf(y));
             }
@@ -144,9 +159,9 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
         const int64_t n = nb * 32 + threadIdx.x;
         if (n < a.N) {
             const float deq = __fdiv_rn(1.0f, scale);
-            float o = __fmul_rn(__fmul_rn((float)(tot - qs), deq), a.wdeq[n / a.seg_rows]);
-            if (a.bias) o = __fadd_rn(o, mmf_to_float(static_cast<const T*>(a.bias)[n]));
-            if (a.addend) o = __fadd_rn(mmf_round_to<T>(o), mmf_to_float(static_cast<const T*>(a.addend)[row * a.N + n]));
+            float o = __fmul_rn(__fmul_rn((float)(tot - qs), deq), ep_wdeq);
+            if (a.bias) o = __fadd_rn(o, ep_bias);
+            if (a.addend) o = __fadd_rn(mmf_round_to<T>(o), ep_add);
             static_cast<T*>(a.out)[row * a.N + n] = mmf_from_float<T>(o);
         }
     }

@@ -45,8 +45,21 @@ __global__ __launch_bounds__(kThreads) void row_kernel(RowArgs a) {
     TR* res_out = a.residual_out ? static_cast<TR*>(a.residual_out) + row * K : nullptr;
     const TW* w = static_cast<const TW*>(a.weight);
 
+    // Every global load of the row is issued up front (x, residual, norm weight, gate) so
+    // their latencies overlap; the reductions below then run on registers only.
     float xv[NV][8];
+    float wv[NV][8];
+    float ov[MODE == ROW_GATE ? NV : 1][8];
     double ss = 0.0;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
+        if (k0 < K) {
+            if (w) mmf_load8<TW>(w, k0, K, vec_ok, wv[v]);
+            if constexpr (MODE == ROW_GATE)
+                mmf_load8<T>(static_cast<const T*>(a.gate) + row * K, k0, K, vec_ok, ov[v]);
+        }
+    }
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
         const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
@@ -74,21 +87,17 @@ __global__ __launch_bounds__(kThreads) void row_kernel(RowArgs a) {
     for (int v = 0; v < NV; ++v) {
         const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
         if (k0 < K) {
-            float wv[8];
-            if (w) mmf_load8<TW>(w, k0, K, vec_ok, wv);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 float y = __fmul_rn(xv[v][i], rstd);
-                if (w) y = __fmul_rn(y, wv[i]);
+                if (w) y = __fmul_rn(y, wv[v][i]);
                 xv[v][i] = y;
                 amax = fmaxf(amax, fabsf(y));
             }
             if constexpr (MODE == ROW_GATE) {
-                float ov[8];
-                mmf_load8<T>(static_cast<const T*>(a.gate) + row * K, k0, K, vec_ok, ov);
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
-                    xv[v][i] = __fmul_rn(__fmul_rn(xv[v][i], ov[i]), mmf_sigmoid(ov[i]));
+                    xv[v][i] = __fmul_rn(__fmul_rn(xv[v][i], ov[v][i]), mmf_sigmoid(ov[v][i]));
             }
             if constexpr (MODE != ROW_QUANT)
                 mmf_store8<T>(static_cast<T*>(a.y) + row * K, k0, K, vec_ok, xv[v]);

@@ -316,10 +316,3 @@ def test_embedding_and_argmax(dev):
     for r in range(2, 5):
         row = logits[r].float()
         assert am[r].item() == int((row == row.max()).nonzero()[0])
-
-
-def test_cpu_tensors_are_rejected():
-    import matmulfreellm_amd.functional as F_
-    from matmulfreellm_amd._lib import MMFError
-    with pytest.raises(MMFError):
-        F_.rmsnorm(torch.randn(2, 64), torch.ones(64))

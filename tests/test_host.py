@@ -1,0 +1,104 @@
+"""Host-side checks that need no GPU: the shared library loads and exports every symbol the public header
+declares, argument validation, the cache and config mirrors, and loud failure on CPU tensors."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "mmf.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mmf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from matmulfreellm_amd import _lib
+    assert os.path.exists(_lib.LIB_PATH), "build the library first: python -m matmulfreellm_amd.build"
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    syms = header_symbols()
+    assert len(syms) >= 18
+    for s in syms:
+        assert hasattr(lib, s), f"{s} declared in include/mmf.h but not exported"
+    assert sorted(_lib.SIGNATURES) == syms, "ctypes signature table and header disagree"
+
+
+def test_size_helpers_need_no_gpu():
+    from matmulfreellm_amd import _lib
+    lib = _lib.load()
+    assert lib.mmf_packed_bytes(2048, 2048) == 2048 * 2048 // 4
+    assert lib.mmf_packed_bytes(33, 129) == 2 * 2 * 1024                # padded to 64 x 256
+    assert lib.mmf_codes_bytes(5, 300, 0) == 5 * 384 and lib.mmf_codes_bytes(5, 300, 1) == 32 * 384
+    assert lib.mmf_ternarize_workspace_bytes() == 8192
+    assert lib.mmf_bitlinear_gemv_max_k() == 8192
+
+
+def test_argument_errors_are_codes_not_crashes():
+    from matmulfreellm_amd import _lib
+    lib = _lib.load()
+    assert lib.mmf_rmsnorm(None, None, None, None, None, 4, 64, 1e-6, 1, 1, 1, None) == -1       # null x
+    assert lib.mmf_rmsnorm(None, None, None, None, None, 0, 64, 1e-6, 1, 1, 1, None) == 0        # empty is fine
+    assert lib.mmf_hgrn_chunk(None, None, None, None, None, 0, 0, 64, 100, 1, None) == -1        # chunk > 64
+    assert lib.mmf_bitlinear_mfma(None, None, None, None, None, 32, None, None, None, 8, 4, 64, 16, 1, -1, None) == -1
+
+
+def test_cpu_tensors_fail_loudly():
+    import matmulfreellm_amd as mm
+    from matmulfreellm_amd._lib import MMFError
+    with pytest.raises(MMFError):
+        mm.RMSNorm(64)(torch.randn(2, 64))
+    with pytest.raises(MMFError):
+        mm.FusedBitLinear(64, 32)(torch.randn(2, 64))
+    with pytest.raises(MMFError):
+        mm.fused_recurrent_hgrn(torch.randn(1, 1, 4, 8), torch.rand(1, 1, 4, 8))
+    with pytest.raises(MMFError):
+        mm.swiglu(torch.randn(4), torch.randn(4))
+
+
+def test_recurrent_cache_semantics():
+    from matmulfreellm_amd import RecurrentCache
+    c = RecurrentCache.from_legacy_cache([(torch.zeros(2, 1, 4),), (torch.zeros(2, 1, 4),)])
+    assert len(c) == 2 and c.get_seq_length() == 0
+    s0 = c[0][0]
+    c.update((torch.ones(2, 1, 4),), 0)
+    assert c.get_seq_length() == 0 and torch.equal(s0, torch.ones(2, 1, 4))      # copied in place
+    c.update((torch.ones(2, 1, 4),), 1)
+    assert c.get_seq_length() == 1                                                 # counted at the last layer
+    with pytest.raises(KeyError):
+        c[2]
+    c.reorder_cache(torch.tensor([1, 0]))
+    assert isinstance(c.to_legacy_cache(), tuple) and c.get_max_length() is None
+
+
+def test_config_and_module_tree_mirror_the_reference():
+    import matmulfreellm_amd as mm
+    cfg = mm.HGRNBitConfig()
+    assert (cfg.vocab_size, cfg.hidden_size, cfg.num_hidden_layers, cfg.num_heads, cfg.use_lower_bound,
+            cfg.rms_norm_eps, cfg.attn_mode, cfg.model_type) == (32000, 2048, 24, 1, True, 1e-6, "fused_recurrent", "hgrn_bit")
+    with torch.device("meta"):
+        model = mm.HGRNBitForCausalLM(mm.HGRNBitConfig(hidden_size=512, num_hidden_layers=2))
+    keys = set(model.state_dict().keys())
+    for k in ["model.embeddings.weight", "model.lower_bounds", "model.layers.0.attn_norm.weight",
+              "model.layers.1.attn.i_proj.weight", "model.layers.1.attn.f_proj.norm.weight",
+              "model.layers.0.attn.g_norm.weight", "model.layers.0.attn.o_proj.weight", "model.layers.0.mlp_norm.weight",
+              "model.layers.0.mlp.gate_proj.weight", "model.layers.0.mlp.down_proj.norm.weight", "model.norm.weight",
+              "lm_head.weight", "lm_head.norm.weight"]:
+        assert k in keys, k
+    assert model.model.layers[0].mlp.intermediate_size == 1536
+    assert tuple(model.model.layers[0].mlp.gate_proj.weight.shape) == (3072, 512)
+    assert model.lm_head.norm.eps == 1e-8
+
+
+def test_layer_norm_linear_quant_fn_rejects_unsupported_forms():
+    import matmulfreellm_amd as mm
+    x, w = torch.randn(2, 64), torch.randn(8, 64)
+    with pytest.raises(NotImplementedError):
+        mm.layer_norm_linear_quant_fn(x, torch.ones(64), None, w, None, is_rms_norm=False)
+    with pytest.raises(NotImplementedError):
+        mm.layer_norm_linear_quant_fn(x, torch.ones(64), torch.zeros(64), w, None, is_rms_norm=True)
+    with pytest.raises(NotImplementedError):
+        mm.HGRNBitAttention(hidden_size=64, num_heads=1, use_short_conv=True)
