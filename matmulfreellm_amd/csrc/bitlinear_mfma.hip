@@ -166,6 +166,99 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// Decode-sized M (<= 64): the contraction is a weight stream, not a GEMM, and the enemy is
+// latency, so nothing is staged and nothing waits on a barrier until the very end.
+// One workgroup of 8 waves owns one 32-row n-block; wave w takes the k-blocks w, w+8, ...
+// A fragments (1 KiB each, L2 resident: the whole A is M x K bytes) and the packed B block
+// are loaded straight into registers, three k-blocks in flight per wave; the 8 partial
+// accumulators meet in LDS and all 512 threads run the epilogue.
+template <typename T, int MB>
+__global__ __launch_bounds__(512) void bitlinear_mfma_skinny_kernel(MfmaArgs p) {
+    constexpr int NWV = 8, PF = 3, MAXK = 8;            // Kp <= 8 * 8 * 128
+    __shared__ int red[NWV][MB][16][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t nb = blockIdx.x;
+    const int64_t KB = p.Kp >> 7, KG = p.Kp >> 4;
+    const int64_t MBtot = (p.M + 31) >> 5;
+
+    v16i acc[MB];
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+
+    uint4 breg[PF];
+    v4i areg[PF][MB][4];
+    auto load_stage = [&](int st, int64_t kb) {
+        if (kb < KB) {
+            breg[st] = p.b[(nb * KB + kb) * 64 + lane];
+#pragma unroll
+            for (int i = 0; i < MB; ++i)
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    areg[st][i][ks] = (v4i){0, 0, 0, 0};
+                    if (i < MBtot)
+                        areg[st][i][ks] = *reinterpret_cast<const v4i*>(p.a + ((int64_t)i * KG + kb * 8 + ks * 2) * 512 + lane * 16);
+                }
+        }
+    };
+#pragma unroll
+    for (int st = 0; st < PF; ++st) load_stage(st, wave + (int64_t)st * NWV);
+#pragma unroll
+    for (int it = 0; it < MAXK; ++it) {
+        const int st = it % PF;
+        const int64_t kb = wave + (int64_t)it * NWV;
+        if (kb < KB) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const uint32_t w = ks == 0 ? breg[st].x : ks == 1 ? breg[st].y : ks == 2 ? breg[st].z : breg[st].w;
+                v4i bf;
+                bf[0] = (int)(w & 0x03030303u);
+                bf[1] = (int)((w >> 2) & 0x03030303u);
+                bf[2] = (int)((w >> 4) & 0x03030303u);
+                bf[3] = (int)((w >> 6) & 0x03030303u);
+#pragma unroll
+                for (int i = 0; i < MB; ++i)
+                    acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[st][i][ks], bf, acc[i], 0, 0, 0);
+            }
+        }
+        if (it + PF < MAXK) load_stage(st, wave + (int64_t)(it + PF) * NWV);
+    }
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) red[wave][i][r][lane] = acc[i][r];
+    __syncthreads();
+
+    const T* bias = static_cast<const T*>(p.bias);
+    const T* addend = static_cast<const T*>(p.addend);
+    T* out = static_cast<T*>(p.out);
+#pragma unroll
+    for (int j = 0; j < MB * 2; ++j) {
+        const int e = threadIdx.x + j * 512;             // (mb, r, lane) flattened
+        const int l = e & 63, r = (e >> 6) & 15, mb = e >> 10;
+        int tot = 0;
+#pragma unroll
+        for (int w = 0; w < NWV; ++w) tot += red[w][mb][r][l];
+        const int64_t m = (int64_t)mb * 32 + 8 * (r >> 2) + 4 * (l >> 5) + (r & 3);
+        const int64_t n = nb * 32 + (l & 31);
+        if (m < p.M && n < p.N) {
+            float o = __fmul_rn(__fmul_rn((float)(tot - p.qsum[m]), p.deq[m]), p.wdeq[n / p.seg_rows]);
+            if (bias) o = __fadd_rn(o, mmf_to_float(bias[n]));
+            if (addend) o = __fadd_rn(mmf_round_to<T>(o), mmf_to_float(addend[m * p.ldo + n]));
+            out[m * p.ldo + n] = mmf_from_float<T>(o);
+        }
+    }
+}
+
+template <typename T, int MB>
+int launch_skinny(const MfmaArgs& a, hipStream_t s) {
+    bitlinear_mfma_skinny_kernel<T, MB><<<dim3((unsigned)mmf_ceil_div(a.N, 32)), dim3(512), 0, s>>>(a);
+    MMF_CHECK_LAUNCH();
+    return 0;
+}
+
 template <typename T, int WGM, int WGN, int WM, int WN>
 int launch_mfma(MfmaArgs a, hipStream_t s) {
     constexpr int BM = WGM * WM * 32, BN = WGN * WN * 32;
@@ -185,9 +278,18 @@ int launch_mfma(MfmaArgs a, hipStream_t s) {
 
 template <typename T>
 int dispatch_mfma(const MfmaArgs& a, int config, hipStream_t s) {
-    // config < 0: pick by M.  Tiles (BM x BN): 0: 32x256, 1: 64x256, 2: 128x256, 3: 256x256.
-    if (config < 0) config = a.M <= 32 ? 0 : a.M <= 64 ? 1 : a.M <= 128 ? 2 : 3;
+    // config < 0: pick by M.  Tiled kernels (BM x BN): 0: 32x256, 1: 64x256, 2: 128x256, 3: 256x256,
+    // 4: 256x256 with 2x4 accumulators per wave.  5 / 6: the decode-sized weight-stream kernel
+    // for M <= 32 / M <= 64 (needs Kp <= 8192).
+    if (config < 0) {
+        if (a.M <= 64 && a.Kp <= 8192) config = a.M <= 32 ? 5 : 6;
+        else config = a.M <= 32 ? 0 : a.M <= 64 ? 1 : a.M <= 128 ? 2 : 3;
+    }
+    if ((config == 5 && a.M > 32) || (config == 6 && a.M > 64) || ((config == 5 || config == 6) && a.Kp > 8192))
+        return MMF_ERR_ARG;
     switch (config) {
+        case 5: return launch_skinny<T, 1>(a, s);
+        case 6: return launch_skinny<T, 2>(a, s);
         case 0: return launch_mfma<T, 1, 8, 1, 1>(a, s);
         case 1: return launch_mfma<T, 1, 8, 2, 1>(a, s);
         case 2: return launch_mfma<T, 2, 4, 2, 2>(a, s);

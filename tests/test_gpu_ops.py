@@ -205,10 +205,13 @@ def test_bitlinear_bias_and_known_answers(dev):
     _bitlinear_case(dev, torch.bfloat16, 40, 2048, 512, "mfma", bias=True)
 
 
-@pytest.mark.parametrize("config", [0, 1, 2, 3, 4])
-def test_bitlinear_mfma_all_tile_configs(dev, config):
+@pytest.mark.parametrize("config,m,k,n", [(0, 300, 1024, 640), (1, 300, 1024, 640), (2, 300, 1024, 640), (3, 300, 1024, 640),
+                                          (4, 300, 1024, 640), (0, 20, 2048, 512), (1, 64, 2048, 512),
+                                          (5, 32, 2048, 640), (5, 7, 5632, 2048), (5, 1, 300, 70), (6, 64, 2048, 6144),
+                                          (6, 40, 5632, 2048), (6, 64, 8192, 96), (6, 33, 6912, 2560)])
+def test_bitlinear_mfma_all_tile_configs(dev, config, m, k, n):
+    """Every tile shape of the matrix-core contraction (0-4 tiled through LDS, 5/6 the decode-sized stream kernel)."""
     torch.manual_seed(8)
-    m, k, n = 300, 1024, 640
     x = torch.randn(m, k).bfloat16()
     w = (torch.randn(n, k) * 0.02).bfloat16()
     nw = torch.ones(k).bfloat16()
@@ -216,7 +219,7 @@ def test_bitlinear_mfma_all_tile_configs(dev, config):
     pw = F().ternarize_pack(w.to(dev))
     q, deq, qsum = F().rmsnorm_quant(x.to(dev), nw.to(dev), eps=1e-8, tiled=True)
     out = F().bitlinear_mfma(q, deq, qsum, pw, m, torch.bfloat16, config=config)
-    assert assert_same(out, ref, 1e-2, f"mfma config {config}") == 0
+    assert assert_same(out, ref, 1e-2, f"mfma config {config} M={m} K={k} N={n}") == 0
 
 
 def test_bitlinear_full_size_gate_proj(dev):
