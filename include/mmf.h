@@ -105,6 +105,26 @@ int mmf_rmsnorm_quant(const void* x, const void* residual, const void* weight, i
  * mmf_bitlinear_mfma: int8 matrix-core contraction on codes from mmf_rmsnorm_quant
  *   (tiled = 1); out has leading dimension ldo; config < 0 picks the tile shape from M. */
 int64_t mmf_bitlinear_gemv_max_k(void);
+/* mmf_bitlinear_gemv_fused: the same launch with the elementwise ops the model runs around a
+ * BitLinear folded in (a decode step is latency bound: one launch per BitLinear, none between).
+ *   prologue (what the BitLinear sees as input, v, rounded to the activation dtype like the
+ *   tensor it replaces):
+ *     0 PLAIN      v = x
+ *     1 NORM       v = RMSNorm(x; w1, eps1)             block norm, modeling_hgrn_bit.py:98
+ *     2 RESNORM    s = x + aux; res_out = s; v = RMSNorm(s; w1, eps1)   fused residual norm, :107
+ *     3 GATEDNORM  v = RMSNorm(x; w1, eps1) * aux * sigmoid(aux)        g_norm, layers/hgrn_bit.py:139
+ *     4 SWIGLU     v = (x * aux) / (1 + exp(-x))        MLP activation, modeling_hgrn_bit.py:58
+ *   epilogue (r = the BitLinear output):
+ *     0 PLAIN   out[M, N] = r (+ bias), or T(r + addend)
+ *     1 STEP    packed = [i; f; g] stacked (N = 3D): gate math of layers/hgrn_bit.py:113-117 and one
+ *               recurrence step on state[M, D] (fp32, in place); out = o [M, D], g_out = raw g [M, D]
+ *     2 SWIGLU  packed = [gate; up] rows (N = 2I): out[M, I] = swiglu(gate, up)
+ * x / aux are [M, K] with row strides ldx / ldaux; all weights (w1, norm_weight) share weight_dtype. */
+int mmf_bitlinear_gemv_fused(int prologue, int epilogue, const void* x, int64_t ldx, const void* aux, int64_t ldaux,
+                             void* res_out, const void* w1, float eps1, const void* norm_weight, float eps,
+                             const void* packed, const float* wdeq, int64_t seg_rows, const void* bias,
+                             const void* addend, void* out, void* g_out, const float* lower_bound, float* state,
+                             int64_t M, int64_t K, int64_t N, int x_dtype, int weight_dtype, void* stream);
 int mmf_bitlinear_gemv(const void* x, const void* norm_weight, const void* packed, const float* wdeq,
                        int64_t seg_rows, const void* bias, const void* addend, void* out, int64_t M, int64_t K,
                        int64_t N, float eps, int x_dtype, int norm_weight_dtype, void* stream);

@@ -23,16 +23,16 @@ from . import functional as F_
 class DecodeEngine:
 
     @classmethod
-    def for_model(cls, model, batch_size: int, use_graph: bool = True):
+    def for_model(cls, model, batch_size: int, use_graph: bool = True, fuse: bool = True):
         engines = model.__dict__.setdefault("_decode_engines", {})
-        key = (batch_size, use_graph)
+        key = (batch_size, use_graph, fuse)
         eng = engines.get(key)
         if eng is None or eng.stale():
-            eng = cls(model, batch_size, use_graph)
+            eng = cls(model, batch_size, use_graph, fuse)
             engines[key] = eng
         return eng
 
-    def __init__(self, model, batch_size: int, use_graph: bool = True):
+    def __init__(self, model, batch_size: int, use_graph: bool = True, fuse: bool = True):
         cfg = model.config
         self.lib = L.load()
         self.model = model
@@ -96,6 +96,7 @@ class DecodeEngine:
         self.deq = z(B, dtype=torch.float32)
         self.qsum = torch.zeros(B, dtype=torch.int32, device=dev)
         self.gemv = B <= F_.GEMV_MAX_M
+        self.fused = fuse and self._can_fuse()
         self.graph = None
 
     @staticmethod
@@ -126,7 +127,49 @@ class DecodeEngine:
                                            pw.packed.data_ptr(), pw.wdeq.data_ptr(), pw.seg_rows, None, L.ptr(addend),
                                            out.data_ptr(), n, B, k, n, self.dt_id, -1, s), "mmf_bitlinear_mfma")
 
+    # prologue / epilogue ids of mmf_bitlinear_gemv_fused
+    PLAIN, NORM, RESNORM, GATEDNORM, SWIGLU = 0, 1, 2, 3, 4
+    E_PLAIN, E_STEP, E_SWIGLU = 0, 1, 2
+
+    def _fused(self, pro, epi, x, ldx, aux, ldaux, res_out, w1, eps1, pw_nw_eps, out, g_out, lb, state, n, k,
+               addend=None):
+        pw, nw, eps = pw_nw_eps
+        L.check(self.lib.mmf_bitlinear_gemv_fused(
+            pro, epi, x.data_ptr(), ldx, L.ptr(aux), ldaux, L.ptr(res_out), L.ptr(w1), eps1, nw.data_ptr(), eps,
+            pw.packed.data_ptr(), pw.wdeq.data_ptr(), pw.seg_rows, None, L.ptr(addend), out.data_ptr(), L.ptr(g_out),
+            L.ptr(lb), L.ptr(state), self.B, k, n, self.dt_id, L.dtype_id(nw.dtype), L.stream()), "mmf_bitlinear_gemv_fused")
+
+    def _launch_step_fused(self):
+        """Batch <= GEMV_MAX_M: four launches per layer, every elementwise op folded into a GEMV."""
+        lib, s, B, H, D, I = self.lib, L.stream(), self.B, self.H, self.D, self.I
+        L.check(lib.mmf_embedding(self.table.data_ptr(), self.tok.data_ptr(), self.h.data_ptr(), B, H, self.V,
+                                  self.dt_id, s), "mmf_embedding")
+        g_buf = self.ifg.view(-1)[:B * D].view(B, D)
+        for ent in self.layers:
+            self._fused(self.NORM, self.E_STEP, self.h, H, None, 0, None, ent["attn_norm"], self.eps,
+                        (ent["ifg"], ent["projs"][0][1], ent["projs"][0][2]), self.o, g_buf, ent["lb"], ent["state"],
+                        3 * D, H)
+            self._fused(self.GATEDNORM, self.E_PLAIN, g_buf, D, self.o, D, None, ent["g_norm"], ent["g_eps"], ent["o"],
+                        self.a, None, None, None, H, D)
+            self._fused(self.RESNORM, self.E_SWIGLU, self.a, H, self.h, H, self.res, ent["mlp_norm"], self.eps,
+                        ent["gate"], self.zb, None, None, None, 2 * I, H)
+            self._fused(self.PLAIN, self.E_PLAIN, self.zb, I, None, 0, None, None, 0.0, ent["down"], self.h, None, None,
+                        None, H, I, addend=self.res)
+        self._fused(self.NORM, self.E_PLAIN, self.h, H, None, 0, None, self.final_norm, self.eps, self.head, self.logits,
+                    None, None, None, self.V, H)
+        L.check(lib.mmf_argmax(self.logits.data_ptr(), self.V, B, self.V, self.tok.data_ptr(), self.dt_id, s), "mmf_argmax")
+
+    def _can_fuse(self):
+        kmax = self.lib.mmf_bitlinear_gemv_max_k()
+        same_dt = all(t.dtype == self.final_norm.dtype for e in self.layers
+                      for t in (e["attn_norm"], e["mlp_norm"], e["g_norm"], e["o"][1], e["gate"][1], e["down"][1],
+                                e["projs"][0][1])) and self.head[1].dtype == self.final_norm.dtype
+        return (self.gemv and same_dt and all(e["ifg"] is not None for e in self.layers)
+                and max(self.H, self.D, self.I) <= kmax and self.D % 32 == 0 and self.I % 32 == 0)
+
     def _launch_step(self):
+        if self.fused:
+            return self._launch_step_fused()
         lib, s, B, H, D, I = self.lib, L.stream(), self.B, self.H, self.D, self.I
         dt, esz = self.dt_id, self.h.element_size()
         wid = L.dtype_id(self.final_norm.dtype)

@@ -68,12 +68,13 @@ def test_prefill_then_greedy_decode(dev, tiny_fp32, tiny_bf16, dtype_name, batch
     from matmulfreellm_amd.decode import DecodeEngine
     out = model(input_ids=ids.to(dev), use_cache=True, logits_to_keep=1)
     assert torch.equal(out.logits[:, -1].cpu(), ref_logits[0])
-    for use_graph in (False, True):
-        eng = DecodeEngine.for_model(model, batch, use_graph=use_graph)
+    for use_graph, fuse in ((False, True), (True, True), (False, False), (True, False)):
+        eng = DecodeEngine.for_model(model, batch, use_graph=use_graph, fuse=fuse)
+        assert eng.fused == (fuse and batch <= 4)
         eng.load_state([c[-1] for c in out.past_key_values])
         for t in range(1, 6):
             lg = eng.step(ref_toks[:, t - 1].to(dev)).cpu()
-            assert torch.equal(lg, ref_logits[t]), f"decode step {t} logits differ (graph={use_graph})"
+            assert torch.equal(lg, ref_logits[t]), f"decode step {t} logits differ (graph={use_graph}, fused={fuse})"
     # self-feeding replay loop
     eng = DecodeEngine.for_model(model, batch, use_graph=True)
     eng.load_state([c[-1] for c in out.past_key_values])
