@@ -38,16 +38,18 @@ struct MfmaArgs {
     void* out;            // [M, N]
     int64_t M, N, Kp, seg_rows, ldo;
     int tiles_m, tiles_n;
+    int vec_store;        // outputs can be written as aligned 16-byte vectors
 };
 
-template <typename T, int WGM, int WGN, int WM, int WN>
+template <typename T, int WGM, int WGN, int WM, int WN, int KSL>
 __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs p) {
     constexpr int NT = 64 * WGM * WGN;
     constexpr int BMB = WGM * WM;                 // m-blocks (of 32 rows) per workgroup tile
     constexpr int BNB = WGN * WN;                 // n-blocks per workgroup tile
-    constexpr int PIECES = BMB * 256;             // 16-byte pieces of one A slab (BMB x 4 KiB)
+    constexpr int CH = KSL * 4096;                // bytes of one m-block's slab (KSL k-blocks of 128)
+    constexpr int PIECES = BMB * (CH / 16);       // 16-byte pieces of one A slab
     constexpr int NPA = (PIECES + NT - 1) / NT;   // pieces per thread
-    extern __shared__ __align__(16) unsigned char smem[];   // 2 x BMB x 4096 bytes
+    extern __shared__ __align__(16) unsigned char smem[];   // 2 x BMB x CH bytes
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
@@ -72,15 +74,15 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
     uint4 areg[NPA];
-    uint4 breg[WN], bnext[WN];
+    uint4 breg[KSL][WN], bnext[KSL][WN];
 
     auto load_a = [&](int64_t kb) {
 #pragma unroll
         for (int i = 0; i < NPA; ++i) {
             const int pc = threadIdx.x + i * NT;
-            const int chunk = pc >> 8, within = pc & 255;
+            const int chunk = pc / (CH / 16), within = pc % (CH / 16);
             areg[i] = make_uint4(0, 0, 0, 0);
-            if (pc < PIECES && mb0 + chunk < MB)
+            if (pc < PIECES && mb0 + chunk < MB && kb * 8 + (within >> 5) < KG)
                 areg[i] = *reinterpret_cast<const uint4*>(p.a + ((mb0 + chunk) * KG + kb * 8) * 512 + within * 16);
         }
     };
@@ -88,15 +90,17 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs
 #pragma unroll
         for (int i = 0; i < NPA; ++i) {
             const int pc = threadIdx.x + i * NT;
-            if (pc < PIECES) *reinterpret_cast<uint4*>(smem + buf * (BMB * 4096) + pc * 16) = areg[i];
+            if (pc < PIECES) *reinterpret_cast<uint4*>(smem + buf * (BMB * CH) + pc * 16) = areg[i];
         }
     };
-    auto load_b = [&](int64_t kb, uint4 (&dst)[WN]) {
+    auto load_b = [&](int64_t kb, uint4 (&dst)[KSL][WN]) {
 #pragma unroll
-        for (int j = 0; j < WN; ++j) {
-            dst[j] = make_uint4(0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u);   // all codes 1 = ternary 0
-            if (nb0 + j < NB) dst[j] = p.b[((nb0 + j) * KB + kb) * 64 + lane];
-        }
+        for (int q = 0; q < KSL; ++q)
+#pragma unroll
+            for (int j = 0; j < WN; ++j) {
+                dst[q][j] = make_uint4(0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u);   // all codes 1 = ternary 0
+                if (nb0 + j < NB && kb + q < KB) dst[q][j] = p.b[((nb0 + j) * KB + kb + q) * 64 + lane];
+            }
     };
 
     load_a(0);
@@ -104,22 +108,31 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs
     store_a(0);
     __syncthreads();
 
-    for (int64_t kb = 0; kb < KB; ++kb) {
-        const int buf = (int)(kb & 1);
-        const bool more = kb + 1 < KB;
+    for (int64_t kb = 0; kb < KB; kb += KSL) {
+        const int buf = (int)((kb / KSL) & 1);
+        const bool more = kb + KSL < KB;
         if (more) {
-            load_a(kb + 1);
-            load_b(kb + 1, bnext);
+            load_a(kb + KSL);
+            load_b(kb + KSL, bnext);
         }
-        const unsigned char* abase = smem + buf * (BMB * 4096) + (wm * WM) * 4096 + lane * 16;
+        const unsigned char* abase = smem + buf * (BMB * CH) + (wm * WM) * CH + lane * 16;
+        // Software pipeline over the 32-wide k-steps of the slab: the LDS reads of step ks+1
+        // are issued before the MFMAs of step ks.
+        v4i af[2][WM];
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            v4i af[WM], bf[WN];
+        for (int i = 0; i < WM; ++i) af[0][i] = *reinterpret_cast<const v4i*>(abase + i * CH);
 #pragma unroll
-            for (int i = 0; i < WM; ++i) af[i] = *reinterpret_cast<const v4i*>(abase + i * 4096 + ks * 1024);
+        for (int ks = 0; ks < 4 * KSL; ++ks) {
+            if (ks + 1 < 4 * KSL) {
+#pragma unroll
+                for (int i = 0; i < WM; ++i)
+                    af[(ks + 1) & 1][i] = *reinterpret_cast<const v4i*>(abase + i * CH + (ks + 1) * 1024);
+            }
+            v4i bf[WN];
 #pragma unroll
             for (int j = 0; j < WN; ++j) {
-                const uint32_t w = ks == 0 ? breg[j].x : ks == 1 ? breg[j].y : ks == 2 ? breg[j].z : breg[j].w;
+                const uint4 bq = breg[ks >> 2][j];
+                const uint32_t w = (ks & 3) == 0 ? bq.x : (ks & 3) == 1 ? bq.y : (ks & 3) == 2 ? bq.z : bq.w;
                 bf[j][0] = (int)(w & 0x03030303u);
                 bf[j][1] = (int)((w >> 2) & 0x03030303u);
                 bf[j][2] = (int)((w >> 4) & 0x03030303u);
@@ -129,38 +142,115 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs
             for (int i = 0; i < WM; ++i)
 #pragma unroll
                 for (int j = 0; j < WN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][i], bf[j], acc[i][j], 0, 0, 0);
         }
         if (more) {
             store_a(buf ^ 1);
 #pragma unroll
-            for (int j = 0; j < WN; ++j) breg[j] = bnext[j];
+            for (int q = 0; q < KSL; ++q)
+#pragma unroll
+                for (int j = 0; j < WN; ++j) breg[q][j] = bnext[q][j];
         }
         __syncthreads();
     }
 
     // ---- epilogue.  Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
-    // column l%32 of the 32x32 block.
+    // column l%32 of the 32x32 block.  Everything that depends only on the column (weight
+    // scale, bias, bounds) or only on the row (deq, qsum) is fetched once, not per element.
     const T* bias = static_cast<const T*>(p.bias);
     const T* addend = static_cast<const T*>(p.addend);
     T* out = static_cast<T*>(p.out);
+    float wdq[WN], bs[WN];
+    int64_t ncol[WN];
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+        ncol[j] = (nb0 + j) * 32 + (lane & 31);
+        const bool ok = ncol[j] < p.N;
+        wdq[j] = ok ? p.wdeq[(uint32_t)ncol[j] / (uint32_t)p.seg_rows] : 0.0f;
+        bs[j] = (ok && bias) ? mmf_to_float(bias[ncol[j]]) : 0.0f;
+        if (!ok) ncol[j] = -1;
+    }
+    constexpr int E = sizeof(T);
+    constexpr int RS = WN * 32 * E + 16;          // LDS row stride of a wave's 32 x (WN*32) staging tile
+    constexpr int CPR = WN * 32 * E / 16;         // 16-byte chunks per row
+    unsigned char* stage = smem + wave * (32 * RS);
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
-        const int64_t mb = mb0 + wm * WM + i;
+        const int64_t mblk = (mb0 + wm * WM + i) * 32;
+        const int64_t mrow0 = mblk + 4 * (lane >> 5);
+        float dqv[16];
+        int qsv[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int64_t m = mb * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            if (m >= p.M) continue;
-            const float dq = p.deq[m];
-            const int qs = p.qsum[m];
+            const int64_t m = mrow0 + 8 * (r >> 2) + (r & 3);
+            dqv[r] = m < p.M ? p.deq[m] : 0.0f;
+            qsv[r] = m < p.M ? p.qsum[m] : 0;
+        }
+        if (p.vec_store) {
+            // Stage the wave's 32 x (WN*32) outputs through LDS so every lane stores 16 bytes and a
+            // store instruction covers whole 128-byte row segments (2-byte scattered stores cost
+            // more than the whole K loop).  The region is private to the wave: no block barrier.
 #pragma unroll
-            for (int j = 0; j < WN; ++j) {
-                const int64_t n = (nb0 + j) * 32 + (lane & 31);
-                if (n >= p.N) continue;
-                float o = __fmul_rn(__fmul_rn((float)(acc[i][j][r] - qs), dq), p.wdeq[n / p.seg_rows]);
-                if (bias) o = __fadd_rn(o, mmf_to_float(bias[n]));
-                if (addend) o = __fadd_rn(mmf_round_to<T>(o), mmf_to_float(addend[m * p.ldo + n]));
-                out[m * p.ldo + n] = mmf_from_float<T>(o);
+            for (int j = 0; j < WN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; r += 2) {
+                    float o0 = __fmul_rn(__fmul_rn((float)(acc[i][j][r] - qsv[r]), dqv[r]), wdq[j]);
+                    float o1 = __fmul_rn(__fmul_rn((float)(acc[i][j][r + 1] - qsv[r + 1]), dqv[r + 1]), wdq[j]);
+                    if (bias) { o0 = __fadd_rn(o0, bs[j]); o1 = __fadd_rn(o1, bs[j]); }
+                    const int row0 = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if constexpr (E == 2) {
+                        // lanes 2k / 2k+1 trade one value so each holds two adjacent columns of one row
+                        const T t0 = mmf_from_float<T>(o0), t1 = mmf_from_float<T>(o1);
+                        const uint32_t b0 = *reinterpret_cast<const uint16_t*>(&t0), b1 = *reinterpret_cast<const uint16_t*>(&t1);
+                        const uint32_t recv = __shfl_xor((lane & 1) ? b0 : b1, 1, 64);
+                        const uint32_t word = (lane & 1) ? (recv | (b1 << 16)) : (b0 | (recv << 16));
+                        const int row = row0 + (lane & 1);
+                        *reinterpret_cast<uint32_t*>(stage + row * RS + (j * 32 + (lane & 30)) * 2) = word;
+                    } else {
+                        *reinterpret_cast<float*>(stage + row0 * RS + (j * 32 + (lane & 31)) * 4) = o0;
+                        *reinterpret_cast<float*>(stage + (row0 + 1) * RS + (j * 32 + (lane & 31)) * 4) = o1;
+                    }
+                }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int c0 = 0; c0 < 32 * CPR; c0 += 64) {
+                const int c = c0 + lane;
+                const int row = c / CPR, cc = c % CPR;
+                const int64_t m = mblk + row, n = nb0 * 32 + cc * (16 / E);
+                if (m < p.M && n < p.N) {
+                    uint4 v = *reinterpret_cast<const uint4*>(stage + row * RS + cc * 16);
+                    if (addend) {
+                        const uint4 av = *reinterpret_cast<const uint4*>(addend + m * p.ldo + n);
+                        const T* pe = reinterpret_cast<const T*>(&v);
+                        const T* ae = reinterpret_cast<const T*>(&av);
+                        uint4 ov;
+                        T* oe = reinterpret_cast<T*>(&ov);
+#pragma unroll
+                        for (int e = 0; e < 16 / E; ++e) oe[e] = mmf_from_float<T>(__fadd_rn(mmf_to_float(pe[e]), mmf_to_float(ae[e])));
+                        v = ov;
+                    }
+                    *reinterpret_cast<uint4*>(out + m * p.ldo + n) = v;
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t m = mrow0 + 8 * (r >> 2) + (r & 3);
+                if (m >= p.M) continue;
+                T* orow = out + m * p.ldo;
+#pragma unroll
+                for (int j = 0; j < WN; ++j) {
+                    if (ncol[j] < 0) continue;
+                    float o = __fmul_rn(__fmul_rn((float)(acc[i][j][r] - qsv[r]), dqv[r]), wdq[j]);
+                    if (bias) o = __fadd_rn(o, bs[j]);
+                    if (addend) o = __fadd_rn(mmf_round_to<T>(o), mmf_to_float(addend[m * p.ldo + ncol[j]]));
+                    orow[ncol[j]] = mmf_from_float<T>(o);
+                }
             }
         }
     }
@@ -244,7 +334,7 @@ __global__ __launch_bounds__(512) void bitlinear_mfma_skinny_kernel(MfmaArgs p) 
         const int64_t m = (int64_t)mb * 32 + 8 * (r >> 2) + 4 * (l >> 5) + (r & 3);
         const int64_t n = nb * 32 + (l & 31);
         if (m < p.M && n < p.N) {
-            float o = __fmul_rn(__fmul_rn((float)(tot - p.qsum[m]), p.deq[m]), p.wdeq[n / p.seg_rows]);
+            float o = __fmul_rn(__fmul_rn((float)(tot - p.qsum[m]), p.deq[m]), p.wdeq[(uint32_t)n / (uint32_t)p.seg_rows]);
             if (bias) o = __fadd_rn(o, mmf_to_float(bias[n]));
             if (addend) o = __fadd_rn(mmf_round_to<T>(o), mmf_to_float(addend[m * p.ldo + n]));
             out[m * p.ldo + n] = mmf_from_float<T>(o);
@@ -259,13 +349,18 @@ int launch_skinny(const MfmaArgs& a, hipStream_t s) {
     return 0;
 }
 
-template <typename T, int WGM, int WGN, int WM, int WN>
+template <typename T, int WGM, int WGN, int WM, int WN, int KSL = 1>
 int launch_mfma(MfmaArgs a, hipStream_t s) {
     constexpr int BM = WGM * WM * 32, BN = WGN * WN * 32;
     a.tiles_m = (int)mmf_ceil_div(a.M, BM);
     a.tiles_n = (int)mmf_ceil_div(a.N, BN);
-    const size_t lds = 2u * (WGM * WM) * 4096u;
-    auto kern = bitlinear_mfma_kernel<T, WGM, WGN, WM, WN>;
+    size_t lds = 2u * (WGM * WM) * 4096u * KSL;
+    const size_t lds_epi = (size_t)(WGM * WGN) * 32u * (WN * 32u * sizeof(T) + 16u);   // per-wave output staging
+    if (lds_epi > lds) lds = lds_epi;
+    const int per_vec = 16 / (int)sizeof(T);
+    a.vec_store = (a.N % per_vec == 0) && (a.ldo % per_vec == 0) && ((reinterpret_cast<uintptr_t>(a.out) & 15u) == 0) &&
+                  ((reinterpret_cast<uintptr_t>(a.addend) & 15u) == 0);
+    auto kern = bitlinear_mfma_kernel<T, WGM, WGN, WM, WN, KSL>;
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)lds);
@@ -295,6 +390,9 @@ int dispatch_mfma(const MfmaArgs& a, int config, hipStream_t s) {
         case 2: return launch_mfma<T, 2, 4, 2, 2>(a, s);
         case 3: return launch_mfma<T, 2, 4, 4, 2>(a, s);
         case 4: return launch_mfma<T, 4, 2, 2, 4>(a, s);
+        case 7: return launch_mfma<T, 2, 4, 4, 2, 2>(a, s);
+        case 8: return launch_mfma<T, 2, 4, 2, 2, 2>(a, s);
+        case 9: return launch_mfma<T, 1, 8, 4, 2, 2>(a, s);
     }
     return MMF_ERR_ARG;
 }
@@ -308,7 +406,7 @@ int mmf_bitlinear_mfma(const int8_t* codes_tiled, const float* deq, const int* q
                        int64_t M,
                        int64_t K, int64_t N, int out_dtype, int config, void* stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (M < 0 || K <= 0 || N <= 0 || seg_rows <= 0 || ldo < N) return MMF_ERR_ARG;
+    if (M < 0 || K <= 0 || N <= 0 || seg_rows <= 0 || ldo < N || N > 0x7fffffff) return MMF_ERR_ARG;
     if (M == 0) return 0;
     if (!codes_tiled || !deq || !qsum || !packed || !wdeq || !out) return MMF_ERR_ARG;
     if ((reinterpret_cast<uintptr_t>(codes_tiled) & 15u) || (reinterpret_cast<uintptr_t>(packed) & 15u)) return MMF_ERR_ALIGN;

@@ -20,30 +20,38 @@ __global__ __launch_bounds__(256) void embedding_kernel(const T* __restrict__ ta
     for (int64_t c = threadIdx.x; c < H; c += 256) dst[c] = src[c];
 }
 
+// One workgroup of 512 threads per row; 8 elements (16 B for 16-bit types) per thread per pass, so a
+// 32000-wide row is 8 passes of independent loads.  Lowest index wins ties; NaNs never win.
 template <typename T>
-__global__ __launch_bounds__(256) void argmax_kernel(const T* __restrict__ logits, int64_t ld, int64_t V,
+__global__ __launch_bounds__(512) void argmax_kernel(const T* __restrict__ logits, int64_t ld, int64_t V,
                                                      int64_t* __restrict__ out) {
-    __shared__ float best_v[4];
-    __shared__ int64_t best_i[4];
+    __shared__ float best_v[8];
+    __shared__ int64_t best_i[8];
     const int64_t r = blockIdx.x;
     const T* row = logits + r * ld;
+    const bool vec_ok = (V % 8) == 0 && (ld % 8) == 0 && (reinterpret_cast<uintptr_t>(logits) & 15u) == 0;
     float bv = -INFINITY;
-    int64_t bi = V;   // larger than any valid index
-    for (int64_t c = threadIdx.x; c < V; c += 256) {
-        const float v = mmf_to_float(row[c]);
-        if (v > bv || (v == bv && c < bi) || (bi == V && !(v != v))) { bv = v; bi = c; }
+    int64_t bi = V;   // larger than any valid index: "nothing yet"
+    for (int64_t c0 = (int64_t)threadIdx.x * 8; c0 < V; c0 += 512 * 8) {
+        float v[8];
+        mmf_load8<T>(row, c0, V, vec_ok, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int64_t c = c0 + i;
+            if (c < V && (v[i] > bv || (bi == V && v[i] == v[i]))) { bv = v[i]; bi = c; }   // ascending c: first max kept
+        }
     }
     for (int o = 32; o > 0; o >>= 1) {
         const float ov = __shfl_xor(bv, o, 64);
         const int64_t oi = __shfl_xor(bi, o, 64);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        if (oi < V && (bi == V || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
     }
     const int w = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) { best_v[w] = bv; best_i[w] = bi; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int i = 1; i < 4; ++i)
-            if (best_v[i] > bv || (best_v[i] == bv && best_i[i] < bi)) { bv = best_v[i]; bi = best_i[i]; }
+        for (int i = 1; i < 8; ++i)
+            if (best_i[i] < V && (bi == V || best_v[i] > bv || (best_v[i] == bv && best_i[i] < bi))) { bv = best_v[i]; bi = best_i[i]; }
         out[r] = bi < V ? bi : 0;
     }
 }
@@ -74,9 +82,9 @@ int mmf_argmax(const void* logits, int64_t ld, int64_t rows, int64_t V, int64_t*
     if (rows == 0) return 0;
     if (!logits || !out) return MMF_ERR_ARG;
     switch (dtype) {
-        case MMF_F32: argmax_kernel<float><<<(unsigned)rows, 256, 0, stream>>>(static_cast<const float*>(logits), ld, V, out); break;
-        case MMF_BF16: argmax_kernel<bf16_t><<<(unsigned)rows, 256, 0, stream>>>(static_cast<const bf16_t*>(logits), ld, V, out); break;
-        case MMF_F16: argmax_kernel<f16_t><<<(unsigned)rows, 256, 0, stream>>>(static_cast<const f16_t*>(logits), ld, V, out); break;
+        case MMF_F32: argmax_kernel<float><<<(unsigned)rows, 512, 0, stream>>>(static_cast<const float*>(logits), ld, V, out); break;
+        case MMF_BF16: argmax_kernel<bf16_t><<<(unsigned)rows, 512, 0, stream>>>(static_cast<const bf16_t*>(logits), ld, V, out); break;
+        case MMF_F16: argmax_kernel<f16_t><<<(unsigned)rows, 512, 0, stream>>>(static_cast<const f16_t*>(logits), ld, V, out); break;
         default: return MMF_ERR_ARG;
     }
     MMF_CHECK_LAUNCH();
