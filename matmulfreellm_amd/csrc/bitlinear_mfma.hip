@@ -41,6 +41,103 @@ struct MfmaArgs {
     int vec_store;        // outputs can be written as aligned 16-byte vectors
 };
 
+// Pack rounded outputs: two floats -> one dword of bf16/f16 (round to nearest even).
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+    const T ta = mmf_from_float<T>(a), tb = mmf_from_float<T>(b);
+    return (uint32_t)(*reinterpret_cast<const uint16_t*>(&ta)) | ((uint32_t)(*reinterpret_cast<const uint16_t*>(&tb)) << 16);
+}
+
+// Epilogue of the tiled kernels.  The MFMAs are issued with the weights as the first operand,
+// so an accumulator holds the TRANSPOSED 32x32 block: register r of lane l is output column
+// n = 8*(r/4) + 4*(l/32) + r%4 and output row m = l%32.  A lane therefore needs one (deq, qsum)
+// pair per block and holds four consecutive columns in registers 4g..4g+3, which pack into one
+// 8-byte piece with no cross-lane traffic.  The wave stages its 32 x (WN*32) outputs in a
+// private LDS region and writes them out as aligned 16-byte vectors (128-byte row segments).
+template <typename T, int WM, int WN>
+__device__ __forceinline__ void mfma_epilogue(const MfmaArgs& p, v16i (&acc)[WM][WN], unsigned char* smem, int lane, int wave,
+                                              int wm, int64_t mb0, int64_t nb0) {
+    const T* bias = static_cast<const T*>(p.bias);
+    const T* addend = static_cast<const T*>(p.addend);
+    T* out = static_cast<T*>(p.out);
+    const int64_t NB = (p.N + 31) >> 5;
+    float wdq[WN];
+#pragma unroll
+    for (int j = 0; j < WN; ++j)   // seg_rows is a multiple of 32: one weight scale per n-block
+        wdq[j] = (nb0 + j < NB) ? p.wdeq[(uint32_t)((nb0 + j) * 32) / (uint32_t)p.seg_rows] : 0.0f;
+    constexpr int E = sizeof(T);
+    constexpr int RS = WN * 32 * E + 16;          // LDS row stride of a wave's 32 x (WN*32) staging tile
+    constexpr int CPR = WN * 32 * E / 16;         // 16-byte chunks per row
+    unsigned char* stage = smem + wave * (32 * RS);
+    const int half = lane >> 5, mloc = lane & 31;
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+        const int64_t mblk = (mb0 + wm * WM + i) * 32;
+        const int64_t m = mblk + mloc;
+        const float dq = m < p.M ? p.deq[m] : 0.0f;
+        const int qs = m < p.M ? p.qsum[m] : 0;
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int ncol = j * 32 + 8 * g + 4 * half;          // first of 4 consecutive columns, tile-relative
+                float o[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    o[t] = __fmul_rn(__fmul_rn((float)(acc[i][j][4 * g + t] - qs), dq), wdq[j]);
+                    if (bias) {
+                        const int64_t n = nb0 * 32 + ncol + t;
+                        o[t] = __fadd_rn(o[t], n < p.N ? mmf_to_float(bias[n]) : 0.0f);
+                    }
+                }
+                if (p.vec_store) {
+                    if constexpr (E == 2)
+                        *reinterpret_cast<uint2*>(stage + mloc * RS + ncol * 2) = make_uint2(pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]));
+                    else
+                        *reinterpret_cast<float4*>(stage + mloc * RS + ncol * 4) = make_float4(o[0], o[1], o[2], o[3]);
+                } else if (m < p.M) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const int64_t n = nb0 * 32 + ncol + t;
+                        if (n < p.N) {
+                            float v = o[t];
+                            if (addend) v = __fadd_rn(mmf_round_to<T>(v), mmf_to_float(addend[m * p.ldo + n]));
+                            out[m * p.ldo + n] = mmf_from_float<T>(v);
+                        }
+                    }
+                }
+            }
+        if (p.vec_store) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int c0 = 0; c0 < 32 * CPR; c0 += 64) {
+                const int c = c0 + lane;
+                const int row = c / CPR, cc = c % CPR;
+                const int64_t mr = mblk + row, n = nb0 * 32 + cc * (16 / E);
+                if (mr < p.M && n < p.N) {
+                    uint4 v = *reinterpret_cast<const uint4*>(stage + row * RS + cc * 16);
+                    if (addend) {
+                        const uint4 av = *reinterpret_cast<const uint4*>(addend + mr * p.ldo + n);
+                        const T* pe = reinterpret_cast<const T*>(&v);
+                        const T* ae = reinterpret_cast<const T*>(&av);
+                        uint4 ov;
+                        T* oe = reinterpret_cast<T*>(&ov);
+#pragma unroll
+                        for (int e = 0; e < 16 / E; ++e) oe[e] = mmf_from_float<T>(__fadd_rn(mmf_to_float(pe[e]), mmf_to_float(ae[e])));
+                        v = ov;
+                    }
+                    *reinterpret_cast<uint4*>(out + mr * p.ldo + n) = v;
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+    }
+}
+
 template <typename T, int WGM, int WGN, int WM, int WN, int KSL>
 __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs p) {
     constexpr int NT = 64 * WGM * WGN;
@@ -142,7 +239,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs
             for (int i = 0; i < WM; ++i)
 #pragma unroll
                 for (int j = 0; j < WN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][i], bf[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[ks & 1][i], acc[i][j], 0, 0, 0);
         }
         if (more) {
             store_a(buf ^ 1);
@@ -154,106 +251,140 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs
         __syncthreads();
     }
 
-    // ---- epilogue.  Accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
-    // column l%32 of the 32x32 block.  Everything that depends only on the column (weight
-    // scale, bias, bounds) or only on the row (deq, qsum) is fetched once, not per element.
-    const T* bias = static_cast<const T*>(p.bias);
-    const T* addend = static_cast<const T*>(p.addend);
-    T* out = static_cast<T*>(p.out);
-    float wdq[WN], bs[WN];
-    int64_t ncol[WN];
+    mfma_epilogue<T, WM, WN>(p, acc, smem, lane, wave, wm, mb0, nb0);
+}
+
+// ------------------------------------------------------------------------------------------
+// Same tiling, but the A slab goes global -> LDS by DMA (global_load_lds_dwordx4: lane l's 16
+// bytes land at the wave-uniform LDS base + 16*l, which is exactly the fragment-tiled layout),
+// so no VGPRs stage it and no ds_write sits in the instruction stream; B is prefetched one
+// 128-wide k-block ahead in registers whatever the slab depth.  One barrier per slab of
+// KSL*128 inputs.
+typedef __attribute__((address_space(3))) void* mmf_lds_ptr;
+typedef __attribute__((address_space(1))) const void* mmf_glb_ptr;
+
+template <typename T, int WGM, int WGN, int WM, int WN, int KSL>
+__global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_dma_kernel(MfmaArgs p) {
+    constexpr int NW = WGM * WGN;
+    constexpr int BMB = WGM * WM;
+    constexpr int BNB = WGN * WN;
+    constexpr int CH = KSL * 4096;                 // bytes of one m-block's slab
+    constexpr int WPIECES = BMB * CH / 1024;       // 1 KiB wave-loads per slab
+    constexpr int NDMA = (WPIECES + NW - 1) / NW;  // per wave
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    int64_t wg = blockIdx.x;
+    const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
+    if (total % 8 == 0) wg = (wg % 8) * (total / 8) + wg / 8;
+    const int64_t tile_m = wg / p.tiles_n, tile_n = wg % p.tiles_n;
+    const int64_t MB = (p.M + 31) >> 5, NB = (p.N + 31) >> 5;
+    const int64_t KB = p.Kp >> 7, KG = p.Kp >> 4;
+    const int64_t mb0 = tile_m * BMB, nb0 = tile_n * BNB + wn * WN;
+
+    v16i acc[WM][WN];
 #pragma unroll
-    for (int j = 0; j < WN; ++j) {
-        ncol[j] = (nb0 + j) * 32 + (lane & 31);
-        const bool ok = ncol[j] < p.N;
-        wdq[j] = ok ? p.wdeq[(uint32_t)ncol[j] / (uint32_t)p.seg_rows] : 0.0f;
-        bs[j] = (ok && bias) ? mmf_to_float(bias[ncol[j]]) : 0.0f;
-        if (!ok) ncol[j] = -1;
-    }
-    constexpr int E = sizeof(T);
-    constexpr int RS = WN * 32 * E + 16;          // LDS row stride of a wave's 32 x (WN*32) staging tile
-    constexpr int CPR = WN * 32 * E / 16;         // 16-byte chunks per row
-    unsigned char* stage = smem + wave * (32 * RS);
+    for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int i = 0; i < WM; ++i) {
-        const int64_t mblk = (mb0 + wm * WM + i) * 32;
-        const int64_t mrow0 = mblk + 4 * (lane >> 5);
-        float dqv[16];
-        int qsv[16];
+        for (int j = 0; j < WN; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int64_t m = mrow0 + 8 * (r >> 2) + (r & 3);
-            dqv[r] = m < p.M ? p.deq[m] : 0.0f;
-            qsv[r] = m < p.M ? p.qsum[m] : 0;
-        }
-        if (p.vec_store) {
-            // Stage the wave's 32 x (WN*32) outputs through LDS so every lane stores 16 bytes and a
-            // store instruction covers whole 128-byte row segments (2-byte scattered stores cost
-            // more than the whole K loop).  The region is private to the wave: no block barrier.
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+    // wave-load w of a slab: m-block chunk = w / (CH/1024), 1 KiB piece `within` of that chunk's slab
+    auto dma_slab = [&](int64_t kb, int buf) {
 #pragma unroll
-            for (int j = 0; j < WN; ++j)
-#pragma unroll
-                for (int r = 0; r < 16; r += 2) {
-                    float o0 = __fmul_rn(__fmul_rn((float)(acc[i][j][r] - qsv[r]), dqv[r]), wdq[j]);
-                    float o1 = __fmul_rn(__fmul_rn((float)(acc[i][j][r + 1] - qsv[r + 1]), dqv[r + 1]), wdq[j]);
-                    if (bias) { o0 = __fadd_rn(o0, bs[j]); o1 = __fadd_rn(o1, bs[j]); }
-                    const int row0 = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                    if constexpr (E == 2) {
-                        // lanes 2k / 2k+1 trade one value so each holds two adjacent columns of one row
-                        const T t0 = mmf_from_float<T>(o0), t1 = mmf_from_float<T>(o1);
-                        const uint32_t b0 = *reinterpret_cast<const uint16_t*>(&t0), b1 = *reinterpret_cast<const uint16_t*>(&t1);
-                        const uint32_t recv = __shfl_xor((lane & 1) ? b0 : b1, 1, 64);
-                        const uint32_t word = (lane & 1) ? (recv | (b1 << 16)) : (b0 | (recv << 16));
-                        const int row = row0 + (lane & 1);
-                        *reinterpret_cast<uint32_t*>(stage + row * RS + (j * 32 + (lane & 30)) * 2) = word;
-                    } else {
-                        *reinterpret_cast<float*>(stage + row0 * RS + (j * 32 + (lane & 31)) * 4) = o0;
-                        *reinterpret_cast<float*>(stage + (row0 + 1) * RS + (j * 32 + (lane & 31)) * 4) = o1;
-                    }
-                }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-            for (int c0 = 0; c0 < 32 * CPR; c0 += 64) {
-                const int c = c0 + lane;
-                const int row = c / CPR, cc = c % CPR;
-                const int64_t m = mblk + row, n = nb0 * 32 + cc * (16 / E);
-                if (m < p.M && n < p.N) {
-                    uint4 v = *reinterpret_cast<const uint4*>(stage + row * RS + cc * 16);
-                    if (addend) {
-                        const uint4 av = *reinterpret_cast<const uint4*>(addend + m * p.ldo + n);
-                        const T* pe = reinterpret_cast<const T*>(&v);
-                        const T* ae = reinterpret_cast<const T*>(&av);
-                        uint4 ov;
-                        T* oe = reinterpret_cast<T*>(&ov);
-#pragma unroll
-                        for (int e = 0; e < 16 / E; ++e) oe[e] = mmf_from_float<T>(__fadd_rn(mmf_to_float(pe[e]), mmf_to_float(ae[e])));
-                        v = ov;
-                    }
-                    *reinterpret_cast<uint4*>(out + m * p.ldo + n) = v;
-                }
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        } else {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int64_t m = mrow0 + 8 * (r >> 2) + (r & 3);
-                if (m >= p.M) continue;
-                T* orow = out + m * p.ldo;
-#pragma unroll
-                for (int j = 0; j < WN; ++j) {
-                    if (ncol[j] < 0) continue;
-                    float o = __fmul_rn(__fmul_rn((float)(acc[i][j][r] - qsv[r]), dqv[r]), wdq[j]);
-                    if (bias) o = __fadd_rn(o, bs[j]);
-                    if (addend) o = __fadd_rn(mmf_round_to<T>(o), mmf_to_float(addend[m * p.ldo + ncol[j]]));
-                    orow[ncol[j]] = mmf_from_float<T>(o);
-                }
+        for (int i = 0; i < NDMA; ++i) {
+            const int w = i * NW + wave;
+            if (w < WPIECES) {
+                const int chunk = w / (CH / 1024), within = w % (CH / 1024);
+                int64_t mb = mb0 + chunk;
+                if (mb >= MB) mb = MB - 1;                       // rows past M are never stored: any valid data will do
+                int64_t kg = kb * 8 + within * 2;                // 16-input groups; one 1 KiB piece = 2 groups
+                if (kg + 2 > KG) kg = KG - 2;                    // k-blocks past Kp are skipped by the compute loop
+                const unsigned char* g = reinterpret_cast<const unsigned char*>(p.a) + (mb * KG + kg) * 512 + lane * 16;
+                __builtin_amdgcn_global_load_lds((mmf_glb_ptr)g, (mmf_lds_ptr)(smem + buf * (BMB * CH) + w * 1024), 16, 0, 0);
             }
         }
+    };
+    auto load_b = [&](int64_t kb, uint4 (&dst)[WN]) {
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+            dst[j] = make_uint4(0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u);
+            if (nb0 + j < NB && kb < KB) dst[j] = p.b[((nb0 + j) * KB + kb) * 64 + lane];
+        }
+    };
+
+    uint4 breg[WN], bnext[WN];
+    dma_slab(0, 0);
+    load_b(0, breg);
+    __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): this wave's DMA has landed
+    __syncthreads();
+
+    for (int64_t kb0 = 0; kb0 < KB; kb0 += KSL) {
+        const int buf = (int)((kb0 / KSL) & 1);
+        if (kb0 + KSL < KB) dma_slab(kb0 + KSL, buf ^ 1);
+        const unsigned char* abase = smem + buf * (BMB * CH) + (wm * WM) * CH + lane * 16;
+#pragma unroll
+        for (int q = 0; q < KSL; ++q) {
+            const int64_t kb = kb0 + q;
+            if (kb < KB) {                                       // uniform over the workgroup
+                load_b(kb + 1, bnext);
+                v4i af[2][WM];
+#pragma unroll
+                for (int i = 0; i < WM; ++i) af[0][i] = *reinterpret_cast<const v4i*>(abase + i * CH + q * 4096);
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    if (ks + 1 < 4) {
+#pragma unroll
+                        for (int i = 0; i < WM; ++i)
+                            af[(ks + 1) & 1][i] = *reinterpret_cast<const v4i*>(abase + i * CH + q * 4096 + (ks + 1) * 1024);
+                    }
+                    v4i bf[WN];
+#pragma unroll
+                    for (int j = 0; j < WN; ++j) {
+                        const uint32_t w = ks == 0 ? breg[j].x : ks == 1 ? breg[j].y : ks == 2 ? breg[j].z : breg[j].w;
+                        bf[j][0] = (int)(w & 0x03030303u);
+                        bf[j][1] = (int)((w >> 2) & 0x03030303u);
+                        bf[j][2] = (int)((w >> 4) & 0x03030303u);
+                        bf[j][3] = (int)((w >> 6) & 0x03030303u);
+                    }
+#pragma unroll
+                    for (int i = 0; i < WM; ++i)
+#pragma unroll
+                        for (int j = 0; j < WN; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[ks & 1][i], acc[i][j], 0, 0, 0);
+                }
+#pragma unroll
+                for (int j = 0; j < WN; ++j) breg[j] = bnext[j];
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0): next slab's DMA (and B prefetch) complete
+        __syncthreads();
     }
+    mfma_epilogue<T, WM, WN>(p, acc, smem, lane, wave, wm, mb0, nb0);
+}
+
+template <typename T, int WGM, int WGN, int WM, int WN, int KSL>
+int launch_mfma_dma(MfmaArgs a, hipStream_t s) {
+    constexpr int BM = WGM * WM * 32, BN = WGN * WN * 32;
+    a.tiles_m = (int)mmf_ceil_div(a.M, BM);
+    a.tiles_n = (int)mmf_ceil_div(a.N, BN);
+    size_t lds = 2u * (WGM * WM) * 4096u * KSL;
+    const size_t lds_epi = (size_t)(WGM * WGN) * 32u * (WN * 32u * sizeof(T) + 16u);
+    if (lds_epi > lds) lds = lds_epi;
+    const int per_vec = 16 / (int)sizeof(T);
+    a.vec_store = (a.N % per_vec == 0) && (a.ldo % per_vec == 0) && ((reinterpret_cast<uintptr_t>(a.out) & 15u) == 0) &&
+                  ((reinterpret_cast<uintptr_t>(a.addend) & 15u) == 0);
+    auto kern = bitlinear_mfma_dma_kernel<T, WGM, WGN, WM, WN, KSL>;
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)lds);
+        if (e != hipSuccess) return (int)e;
+    }
+    kern<<<dim3((unsigned)((int64_t)a.tiles_m * a.tiles_n)), dim3(64 * WGM * WGN), lds, s>>>(a);
+    MMF_CHECK_LAUNCH();
+    return 0;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -393,6 +524,11 @@ int dispatch_mfma(const MfmaArgs& a, int config, hipStream_t s) {
         case 7: return launch_mfma<T, 2, 4, 4, 2, 2>(a, s);
         case 8: return launch_mfma<T, 2, 4, 2, 2, 2>(a, s);
         case 9: return launch_mfma<T, 1, 8, 4, 2, 2>(a, s);
+        case 10: return launch_mfma_dma<T, 2, 4, 4, 2, 2>(a, s);
+        case 11: return launch_mfma_dma<T, 1, 8, 4, 2, 4>(a, s);
+        case 12: return launch_mfma_dma<T, 2, 4, 2, 2, 4>(a, s);
+        case 13: return launch_mfma_dma<T, 1, 8, 4, 2, 2>(a, s);
+        case 14: return launch_mfma_dma<T, 2, 4, 4, 2, 1>(a, s);
     }
     return MMF_ERR_ARG;
 }
@@ -406,7 +542,7 @@ int mmf_bitlinear_mfma(const int8_t* codes_tiled, const float* deq, const int* q
                        int64_t M,
                        int64_t K, int64_t N, int out_dtype, int config, void* stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (M < 0 || K <= 0 || N <= 0 || seg_rows <= 0 || ldo < N || N > 0x7fffffff) return MMF_ERR_ARG;
+    if (M < 0 || K <= 0 || N <= 0 || seg_rows <= 0 || seg_rows % 32 != 0 || ldo < N || N > 0x7fffffff) return MMF_ERR_ARG;
     if (M == 0) return 0;
     if (!codes_tiled || !deq || !qsum || !packed || !wdeq || !out) return MMF_ERR_ARG;
     if ((reinterpret_cast<uintptr_t>(codes_tiled) & 15u) || (reinterpret_cast<uintptr_t>(packed) & 15u)) return MMF_ERR_ALIGN;

@@ -34,10 +34,9 @@ __device__ __forceinline__ float mmf_to_float(bf16_t x) { return __uint_as_float
 __device__ __forceinline__ float mmf_to_float(f16_t x) { return (float)x.v; }
 
 __device__ __forceinline__ uint16_t mmf_f32_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);  // quiet NaN
-    u += 0x7fffu + ((u >> 16) & 1u);                                            // nearest even
-    return (uint16_t)(u >> 16);
+    // round to nearest even; gfx950 has a hardware convert (v_cvt_pk_bf16_f32) the compiler selects
+    const __bf16 b = (__bf16)f;
+    return *reinterpret_cast<const uint16_t*>(&b);
 }
 
 template <typename T> __device__ __forceinline__ T mmf_from_float(float f);
