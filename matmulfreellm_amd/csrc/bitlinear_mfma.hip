@@ -54,17 +54,33 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
 // pair per block and holds four consecutive columns in registers 4g..4g+3, which pack into one
 // 8-byte piece with no cross-lane traffic.  The wave stages its 32 x (WN*32) outputs in a
 // private LDS region and writes them out as aligned 16-byte vectors (128-byte row segments).
+// Per-lane row scales and per-block weight scales of the epilogue, fetched at kernel start so
+// their latency hides behind the whole K loop.
+template <int WM, int WN>
+struct EpiScales { float dq[WM]; int qs[WM]; float wdq[WN]; };
+
+template <int WM, int WN>
+__device__ __forceinline__ void mfma_prefetch_scales(const MfmaArgs& p, EpiScales<WM, WN>& sc, int lane, int wm,
+                                                     int64_t mb0, int64_t nb0) {
+    const int64_t NB = (p.N + 31) >> 5;
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+        const int64_t m = (mb0 + wm * WM + i) * 32 + (lane & 31);
+        sc.dq[i] = m < p.M ? p.deq[m] : 0.0f;
+        sc.qs[i] = m < p.M ? p.qsum[m] : 0;
+    }
+#pragma unroll
+    for (int j = 0; j < WN; ++j)   // seg_rows is a multiple of 32: one weight scale per n-block
+        sc.wdq[j] = (nb0 + j < NB) ? p.wdeq[(uint32_t)((nb0 + j) * 32) / (uint32_t)p.seg_rows] : 0.0f;
+}
+
 template <typename T, int WM, int WN>
-__device__ __forceinline__ void mfma_epilogue(const MfmaArgs& p, v16i (&acc)[WM][WN], unsigned char* smem, int lane, int wave,
-                                              int wm, int64_t mb0, int64_t nb0) {
+__device__ __forceinline__ void mfma_epilogue(const MfmaArgs& p, v16i (&acc)[WM][WN], const EpiScales<WM, WN>& sc,
+                                              unsigned char* smem, int lane, int wave, int wm, int64_t mb0, int64_t nb0) {
     const T* bias = static_cast<const T*>(p.bias);
     const T* addend = static_cast<const T*>(p.addend);
     T* out = static_cast<T*>(p.out);
-    const int64_t NB = (p.N + 31) >> 5;
-    float wdq[WN];
-#pragma unroll
-    for (int j = 0; j < WN; ++j)   // seg_rows is a multiple of 32: one weight scale per n-block
-        wdq[j] = (nb0 + j < NB) ? p.wdeq[(uint32_t)((nb0 + j) * 32) / (uint32_t)p.seg_rows] : 0.0f;
+    const float (&wdq)[WN] = sc.wdq;
     constexpr int E = sizeof(T);
     constexpr int RS = WN * 32 * E + 16;          // LDS row stride of a wave's 32 x (WN*32) staging tile
     constexpr int CPR = WN * 32 * E / 16;         // 16-byte chunks per row
@@ -74,8 +90,8 @@ __device__ __forceinline__ void mfma_epilogue(const MfmaArgs& p, v16i (&acc)[WM]
     for (int i = 0; i < WM; ++i) {
         const int64_t mblk = (mb0 + wm * WM + i) * 32;
         const int64_t m = mblk + mloc;
-        const float dq = m < p.M ? p.deq[m] : 0.0f;
-        const int qs = m < p.M ? p.qsum[m] : 0;
+        const float dq = sc.dq[i];
+        const int qs = sc.qs[i];
 #pragma unroll
         for (int j = 0; j < WN; ++j)
 #pragma unroll
@@ -161,6 +177,8 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs
     const int64_t MB = (p.M + 31) >> 5, NB = (p.N + 31) >> 5;
     const int64_t KB = p.Kp >> 7, KG = p.Kp >> 4;
     const int64_t mb0 = tile_m * BMB, nb0 = tile_n * BNB + wn * WN;
+    EpiScales<WM, WN> sc;
+    mfma_prefetch_scales<WM, WN>(p, sc, lane, wm, mb0, nb0);
 
     v16i acc[WM][WN];
 #pragma unroll
@@ -251,7 +269,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs
         __syncthreads();
     }
 
-    mfma_epilogue<T, WM, WN>(p, acc, smem, lane, wave, wm, mb0, nb0);
+    mfma_epilogue<T, WM, WN>(p, acc, sc, smem, lane, wave, wm, mb0, nb0);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -282,6 +300,8 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_dma_kernel(Mfma
     const int64_t MB = (p.M + 31) >> 5, NB = (p.N + 31) >> 5;
     const int64_t KB = p.Kp >> 7, KG = p.Kp >> 4;
     const int64_t mb0 = tile_m * BMB, nb0 = tile_n * BNB + wn * WN;
+    EpiScales<WM, WN> sc;
+    mfma_prefetch_scales<WM, WN>(p, sc, lane, wm, mb0, nb0);
 
     v16i acc[WM][WN];
 #pragma unroll
@@ -362,7 +382,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_dma_kernel(Mfma
         __builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0): next slab's DMA (and B prefetch) complete
         __syncthreads();
     }
-    mfma_epilogue<T, WM, WN>(p, acc, smem, lane, wave, wm, mb0, nb0);
+    mfma_epilogue<T, WM, WN>(p, acc, sc, smem, lane, wave, wm, mb0, nb0);
 }
 
 template <typename T, int WGM, int WGN, int WM, int WN, int KSL>
@@ -504,12 +524,18 @@ int launch_mfma(MfmaArgs a, hipStream_t s) {
 
 template <typename T>
 int dispatch_mfma(const MfmaArgs& a, int config, hipStream_t s) {
-    // config < 0: pick by M.  Tiled kernels (BM x BN): 0: 32x256, 1: 64x256, 2: 128x256, 3: 256x256,
-    // 4: 256x256 with 2x4 accumulators per wave.  5 / 6: the decode-sized weight-stream kernel
-    // for M <= 32 / M <= 64 (needs Kp <= 8192).
+    // config < 0: pick by shape.
+    //   5 / 6   decode-sized weight-stream kernel, M <= 32 / M <= 64 (needs Kp <= 8192)
+    //   0 - 4   tiled, A staged through registers: 32x256, 64x256, 128x256, 256x256, 256x256 (2x4 accs per wave)
+    //   10 - 14 tiled, A staged by DMA: 256x256 (slab 256), 128x512 (slab 512), 128x256 (slab 512),
+    //           128x512 (slab 256), 256x256 (slab 128)
     if (config < 0) {
+        const int64_t tiles256 = mmf_ceil_div(a.M, 256) * mmf_ceil_div(a.N, 256);
         if (a.M <= 64 && a.Kp <= 8192) config = a.M <= 32 ? 5 : 6;
-        else config = a.M <= 32 ? 0 : a.M <= 64 ? 1 : a.M <= 128 ? 2 : 3;
+        else if (a.M <= 32) config = 0;
+        else if (a.M <= 64) config = 1;
+        else if (a.M <= 128 || tiles256 < 512) config = 12;     // few tiles: smaller ones fill the 256 CUs better
+        else config = 14;
     }
     if ((config == 5 && a.M > 32) || (config == 6 && a.M > 64) || ((config == 5 || config == 6) && a.Kp > 8192))
         return MMF_ERR_ARG;
@@ -521,9 +547,6 @@ int dispatch_mfma(const MfmaArgs& a, int config, hipStream_t s) {
         case 2: return launch_mfma<T, 2, 4, 2, 2>(a, s);
         case 3: return launch_mfma<T, 2, 4, 4, 2>(a, s);
         case 4: return launch_mfma<T, 4, 2, 2, 4>(a, s);
-        case 7: return launch_mfma<T, 2, 4, 4, 2, 2>(a, s);
-        case 8: return launch_mfma<T, 2, 4, 2, 2, 2>(a, s);
-        case 9: return launch_mfma<T, 1, 8, 4, 2, 2>(a, s);
         case 10: return launch_mfma_dma<T, 2, 4, 4, 2, 2>(a, s);
         case 11: return launch_mfma_dma<T, 1, 8, 4, 2, 4>(a, s);
         case 12: return launch_mfma_dma<T, 2, 4, 2, 2, 4>(a, s);

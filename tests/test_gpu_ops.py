@@ -210,7 +210,7 @@ def test_bitlinear_bias_and_known_answers(dev):
                                           (5, 32, 2048, 640), (5, 7, 5632, 2048), (5, 1, 300, 70), (6, 64, 2048, 6144),
                                           (6, 40, 5632, 2048), (6, 64, 8192, 96), (6, 33, 6912, 2560),
                                           (10, 300, 1024, 640), (11, 300, 1152, 640), (12, 300, 1024, 648), (13, 200, 128, 520),
-                                          (14, 520, 2048, 1032), (10, 4096, 2048, 1024)])
+                                          (14, 520, 2048, 1032), (10, 4096, 2048, 1024), (-1, 4096, 512, 2048), (-1, 100, 512, 256)])
 def test_bitlinear_mfma_all_tile_configs(dev, config, m, k, n):
     """Every tile shape of the matrix-core contraction (0-4 tiled through LDS, 5/6 the decode-sized stream kernel)."""
     torch.manual_seed(8)
