@@ -97,47 +97,31 @@ def decode_bench(model, batch, steps, warmup, dev, prompt_len=128):
     return ms, eng
 
 
+# HBM bytes per GEMV launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain copy of
+# known size); see profiles/bitlinear_gemv_decode_bs1_hbm_traffic.txt for the runs and the scale factors.
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3617160
+
+
 def gemv_roofline(eng, iters=20):
-    """Replay a graph that holds exactly the BitLinear GEMV launches of one batch-1 decode step."""
-    from matmulfreellm_amd import _lib as L
-    lib = eng.lib
-    H, D, I, V = eng.H, eng.D, eng.I, eng.V
-    launches = []      # (x, (pw, nw, eps), out, N, K)
-    for ent in eng.layers:
-        if ent["ifg"] is not None:
-            launches.append((eng.hn, (ent["ifg"], ent["projs"][0][1], ent["projs"][0][2]), eng.ifg, 3 * D, H))
-        else:
-            for j in range(3):
-                launches.append((eng.hn, ent["projs"][j], eng.ifg, D, H))
-        launches.append((eng.o2, ent["o"], eng.a, H, D))
-        launches.append((eng.hn, ent["gate"], eng.y, 2 * I, H))
-        launches.append((eng.zb, ent["down"], eng.a, H, I))
-    launches.append((eng.hn, eng.head, eng.logits, V, H))
-    esz = eng.h.element_size()
-    total_bytes = sum(n * k // 4 + k * esz + n * esz + k * nw.element_size() for (_, (pw, nw, _), _, n, k) in launches)
-
-    def launch_all():
-        s = L.stream()
-        for x, (pw, nw, eps), out, n, k in launches:
-            L.check(lib.mmf_bitlinear_gemv(x.data_ptr(), nw.data_ptr(), pw.packed.data_ptr(), pw.wdeq.data_ptr(),
-                                           pw.seg_rows, None, None, out.data_ptr(), 1, k, n, eps, eng.dt_id,
-                                           L.dtype_id(nw.dtype), s), "mmf_bitlinear_gemv")
-
+    """Replay a graph that holds exactly the fused BitLinear GEMV launches of one batch-1 decode step (the step
+    without its embedding gather and argmax): 4 per layer + lm_head, each with the model's own packed weights."""
+    assert eng.fused and eng.B == 1
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
-        launch_all()
+        eng._launch_step_fused(ends=False)
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        launch_all()
+        eng._launch_step_fused(ends=False)
     ms = timed(graph.replay, iters)
-    n = len(launches)
+    n = 4 * eng.L + 1
+    total_bytes = eng.fused_step_bytes()
     us_per_launch = ms * 1e3 / n
     achieved = (total_bytes / n) / (us_per_launch * 1e-6) / 1e9
     return {"bound": "hbm", "kernel": "bitlinear_gemv_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-            "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
             "launches_per_step": n, "algorithmic_bytes_per_launch": total_bytes // n,
             "avg_launch_us": round(us_per_launch, 3)}
 
@@ -234,6 +218,8 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--shape", default="1.3B", choices=list(SHAPES))
     ap.add_argument("--no-extra", action="store_true", help="skip the batch-64 / matrix-core / scan / norm / CPU legs")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -246,6 +232,13 @@ def main():
     model = build_model(args.shape, torch.bfloat16, dev)
     n_tern = sum(p.numel() for n, p in model.named_parameters() if n.endswith("proj.weight") or n == "lm_head.weight")
 
+    if args.calib_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)          # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
     ms, eng = decode_bench(model, args.batch, args.steps, args.warmup, dev)
     tok_s = args.batch * 1e3 / ms
     result = {

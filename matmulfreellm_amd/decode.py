@@ -139,11 +139,13 @@ class DecodeEngine:
             pw.packed.data_ptr(), pw.wdeq.data_ptr(), pw.seg_rows, None, L.ptr(addend), out.data_ptr(), L.ptr(g_out),
             L.ptr(lb), L.ptr(state), self.B, k, n, self.dt_id, L.dtype_id(nw.dtype), L.stream()), "mmf_bitlinear_gemv_fused")
 
-    def _launch_step_fused(self):
-        """Batch <= GEMV_MAX_M: four launches per layer, every elementwise op folded into a GEMV."""
+    def _launch_step_fused(self, ends=True):
+        """Batch <= GEMV_MAX_M: four launches per layer, every elementwise op folded into a GEMV.
+        ends=False leaves out the embedding gather and the argmax (the 4L+1 GEMV launches only)."""
         lib, s, B, H, D, I = self.lib, L.stream(), self.B, self.H, self.D, self.I
-        L.check(lib.mmf_embedding(self.table.data_ptr(), self.tok.data_ptr(), self.h.data_ptr(), B, H, self.V,
-                                  self.dt_id, s), "mmf_embedding")
+        if ends:
+            L.check(lib.mmf_embedding(self.table.data_ptr(), self.tok.data_ptr(), self.h.data_ptr(), B, H, self.V,
+                                      self.dt_id, s), "mmf_embedding")
         g_buf = self.ifg.view(-1)[:B * D].view(B, D)
         for ent in self.layers:
             self._fused(self.NORM, self.E_STEP, self.h, H, None, 0, None, ent["attn_norm"], self.eps,
@@ -157,7 +159,21 @@ class DecodeEngine:
                         None, H, I, addend=self.res)
         self._fused(self.NORM, self.E_PLAIN, self.h, H, None, 0, None, self.final_norm, self.eps, self.head, self.logits,
                     None, None, None, self.V, H)
-        L.check(lib.mmf_argmax(self.logits.data_ptr(), self.V, B, self.V, self.tok.data_ptr(), self.dt_id, s), "mmf_argmax")
+        if ends:
+            L.check(lib.mmf_argmax(self.logits.data_ptr(), self.V, B, self.V, self.tok.data_ptr(), self.dt_id, s),
+                    "mmf_argmax")
+
+    def fused_step_bytes(self):
+        """Algorithmic bytes of the 4L+1 fused GEMV launches of one batch-B step: 2-bit weights once, plus each
+        launch's activation / norm-weight / state reads and its outputs."""
+        B, H, D, I, V, e = self.B, self.H, self.D, self.I, self.V, self.h.element_size()
+        per_layer = ((3 * D * H + H * D + 2 * I * H + H * I) // 4        # packed weights of i/f/g, o, gate, down
+                     + B * (H * e + 2 * D * e + 8 * D) + 2 * H * e + 4 * D  # A: x; o, g out; state rd+wr; two norm weights, lb
+                     + B * (2 * D * e + H * e) + 2 * D * e                  # B: g, o in; a out; two norm weights
+                     + B * (2 * H * e + H * e + I * e) + 2 * H * e          # C: a, h in; res, z out; two norm weights
+                     + B * (I * e + 2 * H * e) + I * e)                     # D: z, res in; h out; norm weight
+        head = V * H // 4 + B * (H * e + V * e) + 2 * H * e
+        return self.L * per_layer + head
 
     def _can_fuse(self):
         kmax = self.lib.mmf_bitlinear_gemv_max_k()
