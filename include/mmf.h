@@ -91,6 +91,20 @@ int mmf_rmsnorm_quant(const void* x, const void* residual, const void* weight, i
                       int* qsum, void* residual_out, int64_t M, int64_t K, float eps, int x_dtype,
                       int residual_dtype, int weight_dtype, int tiled, void* stream);
 
+/* mmf_rmsnorm_quant_fused: the same quantiser (tiled codes) with the elementwise op that precedes a
+ * BitLinear in the model folded in, for batches that go to the matrix cores:
+ *   1 NORM       v = RMSNorm(x; w1, eps1)                                  modeling_hgrn_bit.py:98
+ *   2 RESNORM    s = x + aux; res_out = s; v = RMSNorm(s; w1, eps1)        modeling_hgrn_bit.py:107
+ *   3 STEP_GATE  x, aux, aux2 = raw i, f, g projections of ONE token per row: gate math and one recurrence
+ *                step on state[M, K] (fp32, in place) as mmf_hgrn_step, then
+ *                v = RMSNorm(g; w1, eps1) * o * sigmoid(o)                  layers/hgrn_bit.py:113-139
+ *   4 SWIGLU     v = (x * aux) / (1 + exp(-x))                             modeling_hgrn_bit.py:58
+ * v is rounded to the activation dtype like the tensor it replaces; then q = codes of RMSNorm(v; norm_weight, eps). */
+int mmf_rmsnorm_quant_fused(int prologue, const void* x, int64_t ldx, const void* aux, int64_t ldaux, const void* aux2,
+                            int64_t ldaux2, void* res_out, const void* w1, float eps1, const void* norm_weight, float eps,
+                            const float* lower_bound, float* state, int8_t* q, float* deq, int* qsum, int64_t M, int64_t K,
+                            int x_dtype, int weight_dtype, void* stream);
+
 /* ---- BitLinear contraction ------------------------------------------------------------
  * Both replace F.linear(y, weight_quant(W)) at mmfreelm/ops/fusedbitnet.py:456-458 (class
  * FusedBitLinear :584-610, layer_norm_linear_quant_fn :513-536):

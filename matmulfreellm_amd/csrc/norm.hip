@@ -181,6 +181,210 @@ int dispatch_x(const RowArgs& a, int x_dtype, int r_dtype, int w_dtype, hipStrea
     return MMF_ERR_ARG;
 }
 
+// ---------------------------------------------------------------- fused prologue + quantiser
+// The int8 quantiser with the elementwise op that precedes each BitLinear of a decode step
+// folded in (batch sizes that go to the matrix cores, where the codes must exist in memory):
+//   QPRO_NORM       v = T(RMSNorm(x; w1, eps1))                            (block norm)
+//   QPRO_RESNORM    s = x + aux; res_out = s; v = T(RMSNorm(s; w1, eps1))  (fused residual norm)
+//   QPRO_STEP_GATE  i = x, f = aux, g = aux2 (raw projections of one token): gate math, one recurrence
+//                   step on the fp32 state (in place), o = T(h); v = T(RMSNorm(g; w1, eps1) * o * sigmoid(o))
+//   QPRO_SWIGLU     v = T((x * aux) / (1 + exp(-x)))                       (MLP activation)
+// then  y = RMSNorm(v; norm_w, eps),  q = int8 absmax codes of y  (tiled operand layout).
+enum QPro : int { QPRO_NORM = 1, QPRO_RESNORM = 2, QPRO_STEP_GATE = 3, QPRO_SWIGLU = 4 };
+
+struct FusedQuantArgs {
+    const void* x; const void* aux; const void* aux2;
+    int64_t ldx, ldaux, ldaux2;
+    void* res_out;
+    const void* w1; const void* norm_w;
+    const float* lb; float* state;
+    int8_t* q; float* deq; int* qsum;
+    int64_t M, K, Kp;
+    float eps1, eps;
+};
+
+template <typename T, typename TW, int NV, int PRO>
+__global__ __launch_bounds__(kThreads) void row_quant_fused_kernel(FusedQuantArgs a) {
+    __shared__ double red_a[kWaves], red_b[kWaves];
+    __shared__ float red_f[kWaves];
+    __shared__ int red_i[kWaves];
+    const int64_t row = blockIdx.x, K = a.K, Kp = a.Kp;
+    const bool vec_ok = (K % 8) == 0 && (a.ldx % 8) == 0 && (a.ldaux % 8) == 0 && (a.ldaux2 % 8) == 0;
+    const T* x = static_cast<const T*>(a.x) + row * a.ldx;
+    const T* aux = static_cast<const T*>(a.aux) + row * a.ldaux;
+    const T* aux2 = static_cast<const T*>(a.aux2) + row * a.ldaux2;
+    const TW* w1 = static_cast<const TW*>(a.w1);
+    const TW* nw = static_cast<const TW*>(a.norm_w);
+
+    float xv[NV][8], av[PRO >= QPRO_RESNORM ? NV : 1][8], gv[PRO == QPRO_STEP_GATE ? NV : 1][8];
+    float w1v[PRO != QPRO_SWIGLU ? NV : 1][8], wv[NV][8], lbv[PRO == QPRO_STEP_GATE ? NV : 1][8], stv[PRO == QPRO_STEP_GATE ? NV : 1][8];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
+        if (k0 < K) {
+            mmf_load8<T>(x, k0, K, vec_ok, xv[v]);
+            if constexpr (PRO >= QPRO_RESNORM) mmf_load8<T>(aux, k0, K, vec_ok, av[v]);
+            if constexpr (PRO == QPRO_STEP_GATE) {
+                mmf_load8<T>(aux2, k0, K, vec_ok, gv[v]);
+                mmf_load8<float>(a.state + row * K, k0, K, (K % 8) == 0, stv[v]);
+                if (a.lb) mmf_load8<float>(a.lb, k0, K, (K % 8) == 0, lbv[v]);
+            }
+            if constexpr (PRO != QPRO_SWIGLU) mmf_load8<TW>(w1, k0, K, (K % 8) == 0, w1v[v]);
+            if (nw) mmf_load8<TW>(nw, k0, K, (K % 8) == 0, wv[v]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) xv[v][i] = 0.0f;
+        }
+    }
+    if constexpr (PRO == QPRO_RESNORM) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
+            if (k0 < K) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) xv[v][i] = __fadd_rn(xv[v][i], av[v][i]);
+                if (a.res_out) mmf_store8<T>(static_cast<T*>(a.res_out) + row * K, k0, K, (K % 8) == 0, xv[v]);
+            }
+        }
+    }
+    if constexpr (PRO == QPRO_STEP_GATE) {
+        // gate math + one recurrence step per channel; xv becomes the raw g projection, av the new o
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
+            if (k0 < K) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float iv = xv[v][i], fv = av[v][i];
+                    float s = mmf_sigmoid(fv);
+                    if (a.lb) s = __fadd_rn(lbv[v][i], __fmul_rn(__fsub_rn(1.0f, lbv[v][i]), s));
+                    const float go = mmf_round_to<T>(s);
+                    const float xo = mmf_round_to<T>(__fdiv_rn(__fmul_rn(iv, __fsub_rn(1.0f, go)), __fadd_rn(1.0f, mmf_exp(-iv))));
+                    const float h = __fadd_rn(__fmul_rn(go, stv[v][i]), xo);
+                    stv[v][i] = h;
+                    av[v][i] = mmf_round_to<T>(h);      // o, the swish gate of the gated norm
+                    xv[v][i] = gv[v][i];                // the gated norm normalises the g projection
+                }
+                mmf_store8<float>(a.state + row * K, k0, K, (K % 8) == 0, stv[v]);
+            }
+        }
+    }
+    if constexpr (PRO != QPRO_SWIGLU) {
+        double s1 = 0.0;
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s1 += (double)xv[v][i] * (double)xv[v][i];
+        s1 = mmf_wave_sum(s1);
+        if ((threadIdx.x & 63) == 0) red_a[threadIdx.x >> 6] = s1;
+        __syncthreads();
+        s1 = red_a[0] + red_a[1] + red_a[2] + red_a[3];
+        const float rstd1 = mmf_rstd(s1, K, a.eps1);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
+            if (k0 < K) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    float y = __fmul_rn(__fmul_rn(xv[v][i], rstd1), w1v[v][i]);
+                    if constexpr (PRO == QPRO_STEP_GATE) y = __fmul_rn(__fmul_rn(y, av[v][i]), mmf_sigmoid(av[v][i]));
+                    xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(y) : 0.0f;
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
+            if (k0 < K) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float g = xv[v][i];
+                    const float z = __fdiv_rn(__fmul_rn(g, av[v][i]), __fadd_rn(1.0f, mmf_exp(-g)));
+                    xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(z) : 0.0f;
+                }
+            }
+        }
+    }
+    // BitLinear's own norm + absmax codes
+    double ss = 0.0;
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
+    ss = mmf_wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red_b[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    ss = red_b[0] + red_b[1] + red_b[2] + red_b[3];
+    const float rstd = mmf_rstd(ss, K, a.eps);
+    float amax = 0.0f;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
+        if (k0 < K) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float y = __fmul_rn(xv[v][i], rstd);
+                if (nw) y = __fmul_rn(y, wv[v][i]);
+                xv[v][i] = y;
+                amax = fmaxf(amax, fabsf(y));
+            }
+        }
+    }
+    amax = mmf_wave_max(amax);
+    if ((threadIdx.x & 63) == 0) red_f[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red_f[0], red_f[1]), fmaxf(red_f[2], red_f[3]));
+    const float scale = __fdiv_rn(127.0f, fmaxf(amax, 1e-5f));
+    int qs = 0;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
+        if (k0 < Kp) {
+            uint32_t lo = 0, hi = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int c = (k0 + i < K) ? mmf_code(xv[v][i], scale) : 0;
+                qs += c;
+                const uint32_t b = (uint32_t)(c & 0xff) << (8 * (i & 3));
+                if (i < 4) lo |= b; else hi |= b;
+            }
+            const int64_t off = ((row >> 5) * (Kp >> 4) + (k0 >> 4)) * 512 + (row & 31) * 16 + (k0 & 15);
+            *reinterpret_cast<uint2*>(a.q + off) = make_uint2(lo, hi);
+        }
+    }
+    qs = mmf_wave_sum(qs);
+    if ((threadIdx.x & 63) == 0) red_i[threadIdx.x >> 6] = qs;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        a.deq[row] = __fdiv_rn(1.0f, scale);
+        a.qsum[row] = red_i[0] + red_i[1] + red_i[2] + red_i[3];
+    }
+}
+
+template <typename T, typename TW, int PRO>
+int launch_fused_quant(const FusedQuantArgs& a, hipStream_t s) {
+    const int64_t nv = mmf_ceil_div(a.Kp, (int64_t)kThreads * 8);
+    dim3 grid((unsigned)a.M), block(kThreads);
+    if (nv <= 1) row_quant_fused_kernel<T, TW, 1, PRO><<<grid, block, 0, s>>>(a);
+    else if (nv <= 2) row_quant_fused_kernel<T, TW, 2, PRO><<<grid, block, 0, s>>>(a);
+    else if (nv <= 4) row_quant_fused_kernel<T, TW, 4, PRO><<<grid, block, 0, s>>>(a);
+    else return MMF_ERR_WIDE;
+    MMF_CHECK_LAUNCH();
+    return 0;
+}
+
+template <typename T, typename TW>
+int dispatch_fused_quant(const FusedQuantArgs& a, int pro, hipStream_t s) {
+    switch (pro) {
+        case QPRO_NORM: return launch_fused_quant<T, TW, QPRO_NORM>(a, s);
+        case QPRO_RESNORM: return launch_fused_quant<T, TW, QPRO_RESNORM>(a, s);
+        case QPRO_STEP_GATE: return launch_fused_quant<T, TW, QPRO_STEP_GATE>(a, s);
+        case QPRO_SWIGLU: return launch_fused_quant<T, TW, QPRO_SWIGLU>(a, s);
+    }
+    return MMF_ERR_ARG;
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ---------------------------------------------------------------- swiglu (elementwise)
@@ -282,6 +486,39 @@ int mmf_rmsnorm_quant(const void* x, const void* residual, const void* weight, i
     a.q = q; a.deq = deq; a.qsum = qsum;
     a.M = M; a.K = K; a.Kp = mmf_round_up(K, 128); a.ldx = K; a.eps = eps; a.q_tiled = tiled;
     return dispatch_x<ROW_QUANT>(a, x_dtype, residual_dtype, weight_dtype, stream);
+}
+
+int mmf_rmsnorm_quant_fused(int prologue, const void* x, int64_t ldx, const void* aux, int64_t ldaux, const void* aux2,
+                            int64_t ldaux2, void* res_out, const void* w1, float eps1, const void* norm_weight, float eps,
+                            const float* lower_bound, float* state, int8_t* q, float* deq, int* qsum, int64_t M, int64_t K,
+                            int x_dtype, int weight_dtype, void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (M < 0 || K <= 0 || ldx < K) return MMF_ERR_ARG;
+    if (M == 0) return 0;
+    if (!x || !q || !deq || !qsum) return MMF_ERR_ARG;
+    if (prologue < QPRO_NORM || prologue > QPRO_SWIGLU) return MMF_ERR_ARG;
+    if (prologue >= QPRO_RESNORM && (!aux || ldaux < K)) return MMF_ERR_ARG;
+    if (prologue == QPRO_STEP_GATE && (!aux2 || ldaux2 < K || !state)) return MMF_ERR_ARG;
+    if (prologue != QPRO_SWIGLU && !w1) return MMF_ERR_ARG;
+    FusedQuantArgs a{};
+    a.x = x; a.aux = aux ? aux : x; a.aux2 = aux2 ? aux2 : x; a.ldx = ldx; a.ldaux = aux ? ldaux : ldx;
+    a.ldaux2 = aux2 ? ldaux2 : ldx; a.res_out = res_out; a.w1 = w1; a.norm_w = norm_weight; a.lb = lower_bound; a.state = state;
+    a.q = q; a.deq = deq; a.qsum = qsum; a.M = M; a.K = K; a.Kp = mmf_round_up(K, 128); a.eps1 = eps1; a.eps = eps;
+    if (!aligned16(q)) return MMF_ERR_ALIGN;
+    if (K % 8 == 0 && !(aligned16(x) && aligned16(a.aux) && aligned16(a.aux2) && aligned16(res_out) && aligned16(w1) &&
+                        aligned16(norm_weight) && aligned16(lower_bound) && aligned16(state)))
+        return MMF_ERR_ALIGN;
+    if (!norm_weight && !w1) weight_dtype = MMF_F32;
+    const bool wf32 = weight_dtype == MMF_F32;
+    if (!wf32 && weight_dtype != x_dtype) return MMF_ERR_ARG;
+    switch (x_dtype) {
+        case MMF_F32: return dispatch_fused_quant<float, float>(a, prologue, stream);
+        case MMF_BF16: return wf32 ? dispatch_fused_quant<bf16_t, float>(a, prologue, stream)
+                                   : dispatch_fused_quant<bf16_t, bf16_t>(a, prologue, stream);
+        case MMF_F16: return wf32 ? dispatch_fused_quant<f16_t, float>(a, prologue, stream)
+                                  : dispatch_fused_quant<f16_t, f16_t>(a, prologue, stream);
+    }
+    return MMF_ERR_ARG;
 }
 
 int mmf_swiglu(const void* x, int64_t ldx, const void* y, int64_t ldy, void* out, int64_t rows, int64_t cols,

@@ -97,6 +97,7 @@ class DecodeEngine:
         self.qsum = torch.zeros(B, dtype=torch.int32, device=dev)
         self.gemv = B <= F_.GEMV_MAX_M
         self.fused = fuse and self._can_fuse()
+        self.fused_mfma = fuse and self._can_fuse_mfma()
         self.graph = None
 
     @staticmethod
@@ -175,6 +176,49 @@ class DecodeEngine:
         head = V * H // 4 + B * (H * e + V * e) + 2 * H * e
         return self.L * per_layer + head
 
+    def _qfused(self, pro, x, ldx, aux, ldaux, aux2, ldaux2, res_out, w1, eps1, nw, eps, lb, state, k):
+        L.check(self.lib.mmf_rmsnorm_quant_fused(
+            pro, x, ldx, aux, ldaux, aux2, ldaux2, L.ptr(res_out), L.ptr(w1), eps1, nw.data_ptr(), eps, L.ptr(lb),
+            L.ptr(state), self.q.data_ptr(), self.deq.data_ptr(), self.qsum.data_ptr(), self.B, k, self.dt_id,
+            L.dtype_id(nw.dtype), L.stream()), "mmf_rmsnorm_quant_fused")
+
+    def _mfma(self, pw, out, n, k, addend=None):
+        L.check(self.lib.mmf_bitlinear_mfma(self.q.data_ptr(), self.deq.data_ptr(), self.qsum.data_ptr(),
+                                            pw.packed.data_ptr(), pw.wdeq.data_ptr(), pw.seg_rows, None, L.ptr(addend),
+                                            out.data_ptr(), n, self.B, k, n, self.dt_id, -1, L.stream()), "mmf_bitlinear_mfma")
+
+    def _launch_step_mfma_fused(self):
+        """Batch > GEMV_MAX_M: eight launches per layer -- each BitLinear is a fused prologue+quantiser row kernel
+        (norm / recurrence step + gated norm / residual norm / swiglu folded in) and a matrix-core contraction."""
+        lib, s, B, H, D, I = self.lib, L.stream(), self.B, self.H, self.D, self.I
+        esz = self.h.element_size()
+        L.check(lib.mmf_embedding(self.table.data_ptr(), self.tok.data_ptr(), self.h.data_ptr(), B, H, self.V,
+                                  self.dt_id, s), "mmf_embedding")
+        ifg, y = self.ifg.data_ptr(), self.y.data_ptr()
+        for ent in self.layers:
+            nw, eps = ent["projs"][0][1], ent["projs"][0][2]
+            self._qfused(1, self.h.data_ptr(), H, None, 0, None, 0, None, ent["attn_norm"], self.eps, nw, eps, None, None, H)
+            self._mfma(ent["ifg"], self.ifg, 3 * D, H)
+            self._qfused(3, ifg, 3 * D, ifg + D * esz, 3 * D, ifg + 2 * D * esz, 3 * D, None, ent["g_norm"], ent["g_eps"],
+                         ent["o"][1], ent["o"][2], ent["lb"], ent["state"], D)
+            self._mfma(ent["o"][0], self.a, H, D)
+            self._qfused(2, self.a.data_ptr(), H, self.h.data_ptr(), H, None, 0, self.res, ent["mlp_norm"], self.eps,
+                         ent["gate"][1], ent["gate"][2], None, None, H)
+            self._mfma(ent["gate"][0], self.y, 2 * I, H)
+            self._qfused(4, y, 2 * I, y + I * esz, 2 * I, None, 0, None, None, 0.0, ent["down"][1], ent["down"][2], None, None, I)
+            self._mfma(ent["down"][0], self.h, H, I, addend=self.res)
+        self._qfused(1, self.h.data_ptr(), H, None, 0, None, 0, None, self.final_norm, self.eps, self.head[1], self.head[2],
+                     None, None, H)
+        self._mfma(self.head[0], self.logits, self.V, H)
+        L.check(lib.mmf_argmax(self.logits.data_ptr(), self.V, B, self.V, self.tok.data_ptr(), self.dt_id, s), "mmf_argmax")
+
+    def _can_fuse_mfma(self):
+        same_dt = all(t.dtype == self.final_norm.dtype for e in self.layers
+                      for t in (e["attn_norm"], e["mlp_norm"], e["g_norm"], e["o"][1], e["gate"][1], e["down"][1],
+                                e["projs"][0][1])) and self.head[1].dtype == self.final_norm.dtype
+        return (not self.gemv and same_dt and all(e["ifg"] is not None for e in self.layers)
+                and max(self.H, self.D, self.I) <= 8192 and (3 * self.D) % 8 == 0 and (2 * self.I) % 8 == 0)
+
     def _can_fuse(self):
         kmax = self.lib.mmf_bitlinear_gemv_max_k()
         same_dt = all(t.dtype == self.final_norm.dtype for e in self.layers
@@ -186,6 +230,8 @@ class DecodeEngine:
     def _launch_step(self):
         if self.fused:
             return self._launch_step_fused()
+        if self.fused_mfma:
+            return self._launch_step_mfma_fused()
         lib, s, B, H, D, I = self.lib, L.stream(), self.B, self.H, self.D, self.I
         dt, esz = self.dt_id, self.h.element_size()
         wid = L.dtype_id(self.final_norm.dtype)

@@ -70,7 +70,7 @@ def test_prefill_then_greedy_decode(dev, tiny_fp32, tiny_bf16, dtype_name, batch
     assert torch.equal(out.logits[:, -1].cpu(), ref_logits[0])
     for use_graph, fuse in ((False, True), (True, True), (False, False), (True, False)):
         eng = DecodeEngine.for_model(model, batch, use_graph=use_graph, fuse=fuse)
-        assert eng.fused == (fuse and batch <= 4)
+        assert eng.fused == (fuse and batch <= 4) and eng.fused_mfma == (fuse and batch > 4)
         eng.load_state([c[-1] for c in out.past_key_values])
         for t in range(1, 6):
             lg = eng.step(ref_toks[:, t - 1].to(dev)).cpu()
