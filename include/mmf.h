@@ -151,8 +151,12 @@ int mmf_bitlinear_mfma(const int8_t* codes_tiled, const float* deq, const int* q
  * mmf_hgrn_recurrent replaces fused_recurrent_hgrn, mmfreelm/ops/hgrn/recurrent_fuse.py:
  *   176-185 (kernel :32-68): h = g*h + x with g the decay itself.
  * mmf_hgrn_chunk replaces chunk_hgrn, mmfreelm/ops/hgrn/chunk.py:287-296 (kernels :49-116):
- *   h = exp(g)*h + x with g the log decay, chunked over T (1 <= chunk <= 64).
- * The final state is fp32 in both (the reference rounds the recurrent one to x's dtype). */
+ *   h = exp(g)*h + x with g the log decay.  The reference's two-pass chunked evaluation is a
+ *   reassociation of this recurrence; here it is run step by step, so the result agrees with
+ *   the reference's to rounding and does not depend on `chunk` (kept for the reference's
+ *   signature; 1 <= chunk <= 64 is still checked).
+ * The final state is fp32 in both (the reference rounds the recurrent one to x's dtype).
+ * MMF_ERR_WIDE when 64 rows of D elements reach 2 GiB. */
 int mmf_hgrn_recurrent(const void* x, const void* g, const float* h0, void* o, float* ht, int64_t BH,
                        int64_t T, int64_t D, int dtype, void* stream);
 int mmf_hgrn_chunk(const void* x, const void* g, const float* h0, void* o, float* ht, int64_t BH,

@@ -3,25 +3,23 @@
 //   mmf_hgrn_recurrent : g is the decay itself (linear domain); strictly sequential
 //                        arithmetic (multiply, round, add, round) like
 //                        mmfreelm/ops/hgrn/recurrent_fuse.py:32-68 / ops/hgrn/naive.py:8-31.
-//   mmf_hgrn_chunk     : g is the log decay; the two-pass chunked algorithm of
-//                        mmfreelm/ops/hgrn/chunk.py:49-116 in ONE kernel without the two
-//                        fp32 [B,H,T,D] scratch tensors of chunk.py:232-233.
+//   mmf_hgrn_chunk     : g is the log decay (mmfreelm/ops/hgrn/chunk.py:49-116, 223-254).  The
+//                        chunked two-pass form is a reassociation of the same recurrence on
+//                        exp(g); this entry point runs that recurrence sequentially, which
+//                        needs neither of chunk.py:232-233's fp32 [B,H,T,D] scratch tensors
+//                        and agrees with the chunked form to rounding.
 //   mmf_hgrn_gate      : sigmoid / lower bound / swiglu / mask of
 //                        mmfreelm/layers/hgrn_bit.py:113-120 as one elementwise pass.
 //   mmf_hgrn_step      : the same gate math fused with one recurrence step (decode, T = 1).
 //
 // Layout: x, g, o are [BH, T, D] contiguous; a lane owns one channel d, a wave 64
-// consecutive channels (128 B per time step in bf16), a workgroup of NW waves one
+// consecutive channels (128 B per time step in bf16), a workgroup of 8 waves one
 // 64-channel column of one (b, h).  Time is cut into chunks of 64 steps; a wave holds a
-// whole chunk of x and g in registers, so all of a chunk's loads are in flight together
-// and NW chunks per workgroup overlap.
-//   recurrent: the waves take turns ("baton" = running state in LDS): on its turn a wave
-//              runs its 64 dependent steps from registers, hands the state on, and only
-//              then converts/stores its outputs and issues the loads of its next chunk,
-//              so the serial chain sees no memory latency.
-//   chunk    : every wave scans its chunk from zero state in parallel, publishes the chunk
-//              summary (last h, sum of g), every wave replays the short carry chain over
-//              the NW summaries, then fixes its chunk up from registers.
+// whole chunk of x and g in registers, and the waves take turns ("baton" = running state
+// in LDS): on its turn a wave runs its 64 dependent steps from registers and hands the
+// state on, so the serial chain sees no memory latency while the other waves' loads and
+// stores are in flight.
+#include <type_traits>
 #include "mmf_common.h"
 #include "../../include/mmf.h"
 
@@ -29,158 +27,144 @@ namespace {
 
 constexpr int kCH = 64;   // time steps per register-resident chunk
 
-template <typename T> struct Raw;
-template <> struct Raw<float> {
-    using type = float;
-    static __device__ __forceinline__ float get(float v) { return v; }
-};
-template <> struct Raw<bf16_t> {
-    using type = uint16_t;
-    static __device__ __forceinline__ float get(uint16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
-};
-template <> struct Raw<f16_t> {
-    using type = _Float16;
-    static __device__ __forceinline__ float get(_Float16 v) { return (float)v; }
-};
-
+// -------------------------------------------------------------------------- recurrence
+// A wave's memory work is spread over the rounds between its turns.  Issuing a chunk's 64
+// stores and the next chunk's 128 loads in one go overruns the 64-deep vector-memory queue and
+// puts a full memory round trip inside every round; here each of the four rounds after a turn
+// issues 16 stores and 32 loads, so a round lasts as long as one wave's 64 dependent steps and
+// the waiting waves keep ~40 KiB in flight.
+//
+// Every wave runs the same straight-line iteration (turn, four memory rounds, three idle
+// rounds: eight barriers), entered `wave` barriers late, so the register arrays are never
+// assigned under a branch and stay where they are.  Memory goes through buffer instructions:
+// the resource holds the chunk base, the lane's byte offset sits in one VGPR and the row offset
+// in one SGPR.  What must not happen is switched off without a branch: a resource of zero
+// records turns the loads past the last chunk into zeros and drops the stores of the padding
+// chunks, lanes past D carry an out-of-range offset, the tail chunk clamps its row index for
+// loads and feeds the missing steps (g, x) = (1, -0), which leaves the state bit for bit.
+template <typename R>
+__device__ __forceinline__ R buf_load(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+    if constexpr (sizeof(R) == 4) return __uint_as_float((uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+    else return (R)__builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0);
+}
 template <typename T>
-__device__ __forceinline__ void store_one(T* p, float v) { *p = mmf_from_float<T>(v); }
+__device__ __forceinline__ void buf_store(float v, __amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+    if constexpr (sizeof(T) == 4) {
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, voff, soff, 0);
+    } else {
+        T t = mmf_from_float<T>(v);
+        __builtin_amdgcn_raw_buffer_store_b16(*reinterpret_cast<uint16_t*>(&t), r, voff, soff, 0);
+    }
+}
+template <typename T, typename R>
+__device__ __forceinline__ float raw_get(R v) {
+    if constexpr (sizeof(T) == 4) return v;
+    else { T t; *reinterpret_cast<uint16_t*>(&t) = (uint16_t)v; return mmf_to_float(t); }
+}
 
-// -------------------------------------------------------------------------- recurrent
-template <typename T, int NW>
-__global__ __launch_bounds__(64 * NW) void hgrn_recurrent_kernel(const T* __restrict__ x, const T* __restrict__ g,
-                                                                 const float* __restrict__ h0, T* __restrict__ o,
-                                                                 float* __restrict__ ht, int64_t Tlen, int64_t D) {
-    using R = typename Raw<T>::type;
+// Compile-time loop: the body sees its index as a constant from the front end on, so the
+// register arrays below are split into scalars before any pass can turn a 16-bit array into
+// packed pairs (packing would make every load wait for its neighbour inside the memory rounds).
+template <int V> struct IntC { static constexpr int value = V; };
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (B < E) { f(IntC<B>{}); static_for<B + 1, E>(f); }
+}
+
+// Requires (checked by the launcher): 64 rows of D elements span < 2^31 bytes, Tlen / 64 < 2^30.
+// LOG: g holds log decays (the chunked entry point's convention); the step uses exp(g).
+template <typename T, bool LOG>
+__global__ __launch_bounds__(512) void hgrn_recurrent_pipelined_kernel(const T* __restrict__ x, const T* __restrict__ g,
+                                                                       const float* __restrict__ h0, T* __restrict__ o,
+                                                                       float* __restrict__ ht, int64_t Tlen, int64_t D) {
+    using R = typename std::conditional<sizeof(T) == 4, float, uint16_t>::type;
+    constexpr int NW = 8;
+    constexpr int kRsrcFlags = 0x00020000;                      // raw buffer, 32-bit data format, no swizzle
+    constexpr int kAll = 0x7fffffff;
     __shared__ float baton[64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t bh = blockIdx.y;
-    const int64_t d = (int64_t)blockIdx.x * 64 + lane;
+    const uint32_t d = blockIdx.x * 64u + lane;
     const bool active = d < D;
-    const int64_t base = bh * Tlen * D + d;
-    const R* xr_p = reinterpret_cast<const R*>(x);
-    const R* gr_p = reinterpret_cast<const R*>(g);
-
-    const int64_t NC = (Tlen + kCH - 1) / kCH;
-    const int64_t rounds = (NC + NW - 1) / NW * NW;
+    const uint32_t voff = active ? d * (uint32_t)sizeof(T) : 0x80000000u;   // lanes past D: always out of range
+    const int NC = (int)((Tlen + kCH - 1) / kCH);
+    const int iters = (NC + NW - 1) / NW;
+    const uint32_t rowb = (uint32_t)D * (uint32_t)sizeof(T);
+    const int64_t chunkb = (int64_t)kCH * rowb;
+    const char* xb = reinterpret_cast<const char*>(x + bh * Tlen * D);
+    const char* gb = reinterpret_cast<const char*>(g + bh * Tlen * D);
+    char* ob = reinterpret_cast<char*>(o + bh * Tlen * D);
 
     R xr[kCH], gr[kCH];
     float hs[kCH];
 
-    auto load_chunk = [&](int64_t c) {
-        const int64_t t0 = c * kCH;
-#pragma unroll
-        for (int t = 0; t < kCH; ++t) {
-            if (active && t0 + t < Tlen) {
-                xr[t] = xr_p[base + (t0 + t) * D];
-                gr[t] = gr_p[base + (t0 + t) * D];
-            }
-        }
+    auto rem_of = [&](int c) {                                  // steps of chunk c inside the sequence, as a scalar int
+        return __builtin_amdgcn_readfirstlane((int)max((int64_t)0, min((int64_t)kCH, Tlen - (int64_t)c * kCH)));
     };
 
-    if (wave == 0) baton[lane] = (h0 && active) ? h0[bh * D + d] : 0.0f;
-    if (wave < NC) load_chunk(wave);
-    __syncthreads();
+#define MMF_LOAD_QUARTER(c_, q_)                                                                                       \
+    {                                                                                                                  \
+        const int cc = (c_);                                                                                           \
+        const int rem = rem_of(cc);                                                                                    \
+        const int recs = cc < NC ? kAll : 0;                                                                           \
+        const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void*)(xb + cc * chunkb), 0, recs, kRsrcFlags); \
+        const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc((void*)(gb + cc * chunkb), 0, recs, kRsrcFlags); \
+        static_for<16 * (q_), 16 * (q_) + 16>([&](auto I) __attribute__((always_inline)) {                             \
+            constexpr int t = decltype(I)::value;                                                                      \
+            const uint32_t so = (uint32_t)max(0, min(t, rem - 1)) * rowb; /* rows past the end re-read the last one */ \
+            xr[t] = buf_load<R>(rx, voff, so);                                                                         \
+            gr[t] = buf_load<R>(rg, voff, so);                                                                         \
+        });                                                                                                            \
+    }
+#define MMF_STORE_QUARTER(c_, q_)                                                                                      \
+    {                                                                                                                  \
+        const int cc = (c_);                                                                                           \
+        const int rem = rem_of(cc);                                                                                    \
+        const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc((void*)(ob + cc * chunkb), 0, cc < NC ? kAll : 0, kRsrcFlags); \
+        static_for<16 * (q_), 16 * (q_) + 16>([&](auto I) __attribute__((always_inline)) {                             \
+            constexpr int t = decltype(I)::value;                                                                      \
+            if (t < rem) buf_store<T>(hs[t], ro, voff, (uint32_t)t * rowb);                                            \
+        });                                                                                                            \
+    }
 
-    for (int64_t r = 0; r < rounds; ++r) {
-        const bool mine = (r % NW) == wave && r < NC;
-        const int64_t t0 = r * kCH;
-        if (mine) {
+    if (wave == 0) baton[lane] = (h0 && active) ? h0[bh * D + d] : 0.0f;
+    MMF_LOAD_QUARTER(wave, 0) MMF_LOAD_QUARTER(wave, 1) MMF_LOAD_QUARTER(wave, 2) MMF_LOAD_QUARTER(wave, 3)
+    __syncthreads();
+    for (int i = 0; i < wave; ++i) __syncthreads();              // wave w takes its first turn in round w
+
+    for (int it = 0; it < iters; ++it) {
+        const int c = it * NW + wave;
+        {                                                        // my turn: chunk c, 64 dependent steps
+            const int rem = rem_of(c);
             float h = baton[lane];
-#pragma unroll
-            for (int t = 0; t < kCH; ++t) {
-                if (t0 + t < Tlen) {
-                    h = __fadd_rn(__fmul_rn(Raw<T>::get(gr[t]), h), Raw<T>::get(xr[t]));
-                    hs[t] = h;
-                }
-            }
+            static_for<0, kCH>([&](auto I) __attribute__((always_inline)) {
+                constexpr int t = decltype(I)::value;
+                const float gl = raw_get<T, R>(gr[t]);
+                const float gv = t < rem ? (LOG ? __expf(gl) : gl) : 1.0f;
+                const float xv = t < rem ? raw_get<T, R>(xr[t]) : -0.0f;
+                h = __fadd_rn(__fmul_rn(gv, h), xv);
+                hs[t] = h;
+            });
             baton[lane] = h;
         }
         __syncthreads();
-        if (mine) {
-#pragma unroll
-            for (int t = 0; t < kCH; ++t)
-                if (active && t0 + t < Tlen) store_one<T>(o + base + (t0 + t) * D, hs[t]);
-            if (r + NW < NC) load_chunk(r + NW);
-        }
-    }
-    if (ht && wave == 0 && active) ht[bh * D + d] = baton[lane];
-}
-
-// -------------------------------------------------------------------------- chunk
-template <typename T, int NW>
-__global__ __launch_bounds__(64 * NW) void hgrn_chunk_kernel(const T* __restrict__ x, const T* __restrict__ g,
-                                                             const float* __restrict__ h0, T* __restrict__ o,
-                                                             float* __restrict__ ht, int64_t Tlen, int64_t D, int chunk) {
-    using R = typename Raw<T>::type;
-    __shared__ float sum_h[2][NW][64];
-    __shared__ float sum_g[2][NW][64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t bh = blockIdx.y;
-    const int64_t d = (int64_t)blockIdx.x * 64 + lane;
-    const bool active = d < D;
-    const int64_t base = bh * Tlen * D + d;
-    const R* xr_p = reinterpret_cast<const R*>(x);
-    const R* gr_p = reinterpret_cast<const R*>(g);
-
-    const int64_t NC = (Tlen + chunk - 1) / chunk;
-    const int64_t supers = (NC + NW - 1) / NW;
-
-    R xr[kCH], gr[kCH];
-    float hl[kCH], gc[kCH];
-    float carry = 0.0f;   // fixed-up last output of the chunk before this super-step
-
-    for (int64_t sidx = 0; sidx < supers; ++sidx) {
-        const int64_t c = sidx * NW + wave;
-        const int64_t t0 = c * chunk;
-        const bool have = c < NC;
-        const int pb = (int)(sidx & 1);
-        if (have) {
-#pragma unroll
-            for (int t = 0; t < kCH; ++t)
-                if (active && t < chunk && t0 + t < Tlen) {
-                    xr[t] = xr_p[base + (t0 + t) * D];
-                    gr[t] = gr_p[base + (t0 + t) * D];
-                }
-            float h = (c == 0 && h0 && active) ? h0[bh * D + d] : 0.0f;
-            float a = 0.0f;
-#pragma unroll
-            for (int t = 0; t < kCH; ++t)
-                if (t < chunk && t0 + t < Tlen) {
-                    const float gv = Raw<T>::get(gr[t]);
-                    h = __fadd_rn(__fmul_rn(__expf(gv), h), Raw<T>::get(xr[t]));
-                    a = __fadd_rn(a, gv);
-                    hl[t] = h;
-                    gc[t] = a;
-                }
-            sum_h[pb][wave][lane] = h;
-            sum_g[pb][wave][lane] = a;
-        }
+        MMF_STORE_QUARTER(c, 0) MMF_LOAD_QUARTER(c + NW, 0)
         __syncthreads();
-        // carry chain over the chunks of this super-step that precede this wave's chunk
-        float prev = carry;          // fixed-up last output of chunk sidx*NW - 1
-        float mine_prev = carry;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) {
-            if (w == wave) mine_prev = prev;
-            const int64_t cw = sidx * NW + w;
-            if (cw < NC) {
-                const float hw = sum_h[pb][w][lane], gw = sum_g[pb][w][lane];
-                prev = (cw == 0) ? hw : __fadd_rn(hw, __fmul_rn(__expf(gw), prev));
-            }
-        }
-        carry = prev;
-        if (have) {
-#pragma unroll
-            for (int t = 0; t < kCH; ++t)
-                if (active && t < chunk && t0 + t < Tlen) {
-                    const float v = (c == 0) ? hl[t] : __fadd_rn(hl[t], __fmul_rn(__expf(gc[t]), mine_prev));
-                    store_one<T>(o + base + (t0 + t) * D, v);
-                }
-        }
-        // sum_* buffers alternate between super-steps, so one barrier per super-step is enough
+        MMF_STORE_QUARTER(c, 1) MMF_LOAD_QUARTER(c + NW, 1)
+        __syncthreads();
+        MMF_STORE_QUARTER(c, 2) MMF_LOAD_QUARTER(c + NW, 2)
+        __syncthreads();
+        MMF_STORE_QUARTER(c, 3) MMF_LOAD_QUARTER(c + NW, 3)
+        __syncthreads();
+        __syncthreads();
+        __syncthreads();
+        __syncthreads();
     }
-    if (ht && wave == 0 && active) ht[bh * D + d] = carry;
+    for (int i = wave; i < NW - 1; ++i) __syncthreads();         // every wave passes the same number of barriers
+    __syncthreads();
+    if (ht && wave == 0 && active) ht[bh * D + d] = baton[lane];
+#undef MMF_LOAD_QUARTER
+#undef MMF_STORE_QUARTER
 }
 
 // -------------------------------------------------------------------------- gate math
@@ -232,38 +216,19 @@ __global__ __launch_bounds__(256) void state_init_kernel(const float* __restrict
     if (i < n) ht[i] = h0 ? h0[i] : 0.0f;
 }
 
+// The kernel addresses a 64-step chunk with 32-bit offsets and counts chunks in an int.
 template <typename T>
-int launch_recurrent(const void* x, const void* g, const float* h0, void* o, float* ht, int64_t BH, int64_t Tlen,
-                     int64_t D, hipStream_t s) {
-    dim3 grid((unsigned)mmf_ceil_div(D, 64), (unsigned)BH);
-    const int64_t NC = mmf_ceil_div(Tlen, kCH);
-    if (NC >= 8)
-        hgrn_recurrent_kernel<T, 8><<<grid, 512, 0, s>>>(static_cast<const T*>(x), static_cast<const T*>(g), h0,
-                                                         static_cast<T*>(o), ht, Tlen, D);
-    else if (NC >= 2)
-        hgrn_recurrent_kernel<T, 2><<<grid, 128, 0, s>>>(static_cast<const T*>(x), static_cast<const T*>(g), h0,
-                                                         static_cast<T*>(o), ht, Tlen, D);
-    else
-        hgrn_recurrent_kernel<T, 1><<<grid, 64, 0, s>>>(static_cast<const T*>(x), static_cast<const T*>(g), h0,
-                                                        static_cast<T*>(o), ht, Tlen, D);
-    MMF_CHECK_LAUNCH();
-    return 0;
+bool scan_fits(int64_t Tlen, int64_t D) {
+    return mmf_ceil_div(Tlen, (int64_t)kCH) < (1 << 30) && (int64_t)kCH * D * (int64_t)sizeof(T) < (1ll << 31);
 }
 
-template <typename T>
-int launch_chunk(const void* x, const void* g, const float* h0, void* o, float* ht, int64_t BH, int64_t Tlen,
-                 int64_t D, int chunk, hipStream_t s) {
+template <typename T, bool LOG>
+int launch_scan(const void* x, const void* g, const float* h0, void* o, float* ht, int64_t BH, int64_t Tlen, int64_t D,
+                hipStream_t s) {
+    if (!scan_fits<T>(Tlen, D)) return MMF_ERR_WIDE;
     dim3 grid((unsigned)mmf_ceil_div(D, 64), (unsigned)BH);
-    const int64_t NC = mmf_ceil_div(Tlen, chunk);
-    if (NC >= 8)
-        hgrn_chunk_kernel<T, 8><<<grid, 512, 0, s>>>(static_cast<const T*>(x), static_cast<const T*>(g), h0,
-                                                     static_cast<T*>(o), ht, Tlen, D, chunk);
-    else if (NC >= 2)
-        hgrn_chunk_kernel<T, 2><<<grid, 128, 0, s>>>(static_cast<const T*>(x), static_cast<const T*>(g), h0,
-                                                     static_cast<T*>(o), ht, Tlen, D, chunk);
-    else
-        hgrn_chunk_kernel<T, 1><<<grid, 64, 0, s>>>(static_cast<const T*>(x), static_cast<const T*>(g), h0,
-                                                    static_cast<T*>(o), ht, Tlen, D, chunk);
+    hgrn_recurrent_pipelined_kernel<T, LOG><<<grid, 512, 0, s>>>(static_cast<const T*>(x), static_cast<const T*>(g), h0,
+                                                                 static_cast<T*>(o), ht, Tlen, D);
     MMF_CHECK_LAUNCH();
     return 0;
 }
@@ -302,9 +267,9 @@ int mmf_hgrn_recurrent(const void* x, const void* g, const float* h0, void* o, f
     }
     if (!x || !g || !o) return MMF_ERR_ARG;
     switch (dtype) {
-        case MMF_F32: return launch_recurrent<float>(x, g, h0, o, ht, BH, T, D, stream);
-        case MMF_BF16: return launch_recurrent<bf16_t>(x, g, h0, o, ht, BH, T, D, stream);
-        case MMF_F16: return launch_recurrent<f16_t>(x, g, h0, o, ht, BH, T, D, stream);
+        case MMF_F32: return launch_scan<float, false>(x, g, h0, o, ht, BH, T, D, stream);
+        case MMF_BF16: return launch_scan<bf16_t, false>(x, g, h0, o, ht, BH, T, D, stream);
+        case MMF_F16: return launch_scan<f16_t, false>(x, g, h0, o, ht, BH, T, D, stream);
     }
     return MMF_ERR_ARG;
 }
@@ -323,9 +288,9 @@ int mmf_hgrn_chunk(const void* x, const void* g, const float* h0, void* o, float
     }
     if (!x || !g || !o) return MMF_ERR_ARG;
     switch (dtype) {
-        case MMF_F32: return launch_chunk<float>(x, g, h0, o, ht, BH, T, D, chunk, stream);
-        case MMF_BF16: return launch_chunk<bf16_t>(x, g, h0, o, ht, BH, T, D, chunk, stream);
-        case MMF_F16: return launch_chunk<f16_t>(x, g, h0, o, ht, BH, T, D, chunk, stream);
+        case MMF_F32: return launch_scan<float, true>(x, g, h0, o, ht, BH, T, D, stream);
+        case MMF_BF16: return launch_scan<bf16_t, true>(x, g, h0, o, ht, BH, T, D, stream);
+        case MMF_F16: return launch_scan<f16_t, true>(x, g, h0, o, ht, BH, T, D, stream);
     }
     return MMF_ERR_ARG;
 }
