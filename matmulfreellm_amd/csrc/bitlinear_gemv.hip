@@ -92,7 +92,7 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
     __shared__ int red_q[kGemvWaves];
     __shared__ int part[R][kGemvWaves][32];
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keep it in a scalar register
     const int64_t nb = blockIdx.x, row = blockIdx.y;
     const int64_t K = a.K, Kp = a.Kp, KB = Kp >> 7;
     const int64_t NBseg = (a.N / R + 31) >> 5;                  // n-blocks per stacked segment (R > 1)

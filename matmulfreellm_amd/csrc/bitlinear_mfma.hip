@@ -164,7 +164,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs
     constexpr int NPA = (PIECES + NT - 1) / NT;   // pieces per thread
     extern __shared__ __align__(16) unsigned char smem[];   // 2 x BMB x CH bytes
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keep it in a scalar register
     const int wm = wave / WGN, wn = wave % WGN;
 
     // XCD-aware tile order: hardware deals consecutive workgroup ids round-robin to the 8
@@ -291,7 +291,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_dma_kernel(Mfma
     constexpr int NDMA = (WPIECES + NW - 1) / NW;  // per wave
     extern __shared__ __align__(16) unsigned char smem[];
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keep it in a scalar register
     const int wm = wave / WGN, wn = wave % WGN;
     int64_t wg = blockIdx.x;
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
@@ -418,7 +418,7 @@ template <typename T, int MB>
 __global__ __launch_bounds__(512) void bitlinear_mfma_skinny_kernel(MfmaArgs p) {
     constexpr int NWV = 8, PF = 3, MAXK = 8;            // Kp <= 8 * 8 * 128
     __shared__ int red[NWV][MB][16][64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keep it in a scalar register
     const int64_t nb = blockIdx.x;
     const int64_t KB = p.Kp >> 7, KG = p.Kp >> 4;
     const int64_t MBtot = (p.M + 31) >> 5;
