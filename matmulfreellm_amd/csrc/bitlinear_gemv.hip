@@ -19,7 +19,10 @@
 //                PRO_GATEDNORM  v = T(RMSNorm(x; w1) * aux * sigmoid(aux))     (g_norm)
 //                PRO_SWIGLU     v = T((x * aux) / (1 + exp(-x)))               (MLP activation)
 //              then  y = RMSNorm(v; norm_w, eps),  q = int8 absmax codes of y.
-//              The packed weight loads of the wave are issued before any of it.
+//              A launch costs what its instruction stream and its dependent memory round
+//              trips cost, so every global load of the kernel (row, norm weights, the wave's
+//              packed weight blocks, the epilogue's operands) is issued up front, raw, and
+//              converted only where it is used; a thread owns 4 elements of the row per pass.
 //   main     : wave w takes the 1 KiB weight blocks kb = w, w+8, ... of each of its R n-blocks;
 //              a lane holds 64 weights of one output row, expands each dword to four
 //              byte-wide code dwords (shift + mask) and accumulates with v_dot4_i32_i8
@@ -36,8 +39,9 @@ namespace {
 
 constexpr int kGemvWaves = 8;
 constexpr int kGemvThreads = kGemvWaves * 64;
-constexpr int kGemvMaxBlocksPerWave = 8;                        // Kp <= 8 * 8 * 128 = 8192
-constexpr int64_t kGemvMaxK = (int64_t)kGemvWaves * kGemvMaxBlocksPerWave * 128;
+constexpr int kGemvEl = 4;                                      // elements of x per thread and pass
+constexpr int kGemvMaxNV = 4;                                   // passes: Kp <= 4 * 512 * 4 = 8192
+constexpr int64_t kGemvMaxK = (int64_t)kGemvMaxNV * kGemvThreads * kGemvEl;
 
 enum Pro : int { PRO_PLAIN = 0, PRO_NORM = 1, PRO_RESNORM = 2, PRO_GATEDNORM = 3, PRO_SWIGLU = 4 };
 enum Epi : int { EPI_PLAIN = 0, EPI_STEP = 1, EPI_SWIGLU = 2 };
@@ -56,7 +60,8 @@ struct GemvArgs {
     void* g_out;          // EPI_STEP: raw g projection [M, N/3]
     const float* lb;      // EPI_STEP: lower bound [N/3] or null
     float* state;         // EPI_STEP: recurrent state [M, N/3] fp32, updated in place
-    int64_t K, Kp, N, seg_rows, ldx, ldaux;
+    int64_t ldx, ldaux;
+    int K, Kp, N, seg_rows;                                     // all < 2^31 (checked by the entry point)
     float eps, eps1;
 };
 
@@ -81,9 +86,58 @@ __device__ __forceinline__ float block_max_once(float v, float* slot) {
     return s;
 }
 
-template <typename T, typename TW, int NV, int PRO, int EPI>
+// Four consecutive elements as they sit in memory; unpacked to fp32 only where they are used, so
+// that all of a thread's loads are in flight before the first conversion waits for one.
+template <typename T> struct Raw4 { uint2 v; };
+template <> struct Raw4<float> { float4 v; };
+
+template <typename T, bool VEC>
+__device__ __forceinline__ Raw4<T> raw4_load(const T* p, int k0, int K) {
+    Raw4<T> r;
+    if constexpr (VEC) {
+        const int kk = k0 < K ? k0 : 0;                         // lanes past K re-read the row start; zeroed on unpack
+        r.v = *reinterpret_cast<const decltype(r.v)*>(p + kk);
+    } else {
+        T e[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) e[i] = p[k0 + i < K ? k0 + i : 0];
+        __builtin_memcpy(&r.v, e, sizeof(r.v));
+    }
+    return r;
+}
+template <typename T>
+__device__ __forceinline__ void raw4_unpack(const Raw4<T>& r, float (&f)[4]) {
+    if constexpr (sizeof(T) == 4) {
+        f[0] = r.v.x; f[1] = r.v.y; f[2] = r.v.z; f[3] = r.v.w;
+    } else {
+        T e[4];
+        __builtin_memcpy(e, &r.v, sizeof(r.v));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = mmf_to_float(e[i]);
+    }
+}
+template <typename T, bool VEC>
+__device__ __forceinline__ void raw4_store(T* p, int k0, int K, const float (&f)[4]) {
+    T e[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e[i] = mmf_from_float<T>(f[i]);
+    if constexpr (VEC) {
+        if (k0 < K) __builtin_memcpy(p + k0, e, sizeof(e));
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (k0 + i < K) p[k0 + i] = e[i];
+    }
+}
+
+// NV: passes over the row (Kp <= NV * 2048); a wave then owns at most 2 * NV of the row's 1 KiB
+// weight blocks per n-block.  VEC: K, the row strides and every pointer allow 4-element accesses.
+template <typename T, typename TW, int NV, int PRO, int EPI, bool VEC>
 __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a) {
     constexpr int R = EPI == EPI_STEP ? 3 : EPI == EPI_SWIGLU ? 2 : 1;
+    constexpr int BPW = 2 * NV;
+    constexpr bool HAS_AUX = PRO >= PRO_RESNORM;
+    constexpr bool HAS_W1 = PRO >= PRO_NORM && PRO <= PRO_GATEDNORM;
     extern __shared__ __align__(16) unsigned char smem[];
     int8_t* q_lds = reinterpret_cast<int8_t*>(smem);            // Kp bytes
     // one slot array per reduction, so each costs a single barrier
@@ -92,68 +146,73 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
     __shared__ int red_q[kGemvWaves];
     __shared__ int part[R][kGemvWaves][32];
 
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keep it in a scalar register
-    const int64_t nb = blockIdx.x, row = blockIdx.y;
-    const int64_t K = a.K, Kp = a.Kp, KB = Kp >> 7;
-    const int64_t NBseg = (a.N / R + 31) >> 5;                  // n-blocks per stacked segment (R > 1)
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nb = blockIdx.x, row = blockIdx.y;
+    const int K = a.K, Kp = a.Kp, KB = Kp >> 7;
+    const int Nseg = a.N / R;
+    const int NBseg = (Nseg + 31) >> 5;                         // n-blocks per stacked segment (R > 1)
 
-    // ---- issue this wave's weight loads first (independent of the prologue)
-    uint4 wreg[R][kGemvMaxBlocksPerWave];
+    // ---- every global load of the kernel, back to back: the row first (the prologue's
+    // reductions wait for it), then this wave's packed weights, then the epilogue's operands
+    const T* x = static_cast<const T*>(a.x) + (int64_t)row * a.ldx;
+    const T* aux = static_cast<const T*>(a.aux) + (int64_t)row * a.ldaux;
+    const TW* w1 = static_cast<const TW*>(a.w1);
+    const TW* nw = static_cast<const TW*>(a.norm_w);
+    Raw4<T> xraw[NV], araw[HAS_AUX ? NV : 1];
+    Raw4<TW> w1raw[HAS_W1 ? NV : 1], nwraw[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int k0 = (v * kGemvThreads + (int)threadIdx.x) * kGemvEl;
+        xraw[v] = raw4_load<T, VEC>(x, k0, K);
+        if constexpr (HAS_AUX) araw[v] = raw4_load<T, VEC>(aux, k0, K);
+        if constexpr (HAS_W1) w1raw[v] = raw4_load<TW, VEC>(w1, k0, K);
+        if (nw) nwraw[v] = raw4_load<TW, VEC>(nw, k0, K);
+    }
+    uint4 wreg[R][BPW];
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int i = 0; i < kGemvMaxBlocksPerWave; ++i) {
-            const int64_t kb = wave + (int64_t)i * kGemvWaves;
-            if (kb < KB) wreg[r][i] = a.packed[((nb + r * NBseg) * KB + kb) * 64 + lane];
+        for (int i = 0; i < BPW; ++i) {
+            const int kb = wave + i * kGemvWaves;
+            if (kb < KB) wreg[r][i] = a.packed[((int64_t)(nb + r * NBseg) * KB + kb) * 64 + lane];
         }
-
-    // ---- all other global loads the kernel will need, back to back
-    const bool vec_ok = (K % 8) == 0 && (a.ldx % 8) == 0 && (a.ldaux % 8) == 0;
-    const T* x = static_cast<const T*>(a.x) + row * a.ldx;
-    const T* aux = static_cast<const T*>(a.aux) + row * a.ldaux;
-    const TW* w1 = static_cast<const TW*>(a.w1);
-    const TW* nw = static_cast<const TW*>(a.norm_w);
-    float xv[NV][8], av[PRO >= PRO_RESNORM ? NV : 1][8], w1v[(PRO >= PRO_NORM && PRO <= PRO_GATEDNORM) ? NV : 1][8], wv[NV][8];
-#pragma unroll
-    for (int v = 0; v < NV; ++v) {
-        const int64_t k0 = ((int64_t)v * kGemvThreads + threadIdx.x) * 8;
-        if (k0 < K) {
-            mmf_load8<T>(x, k0, K, vec_ok, xv[v]);
-            if constexpr (PRO >= PRO_RESNORM) mmf_load8<T>(aux, k0, K, vec_ok, av[v]);
-            if constexpr (PRO >= PRO_NORM && PRO <= PRO_GATEDNORM) mmf_load8<TW>(w1, k0, K, vec_ok, w1v[v]);
-            if (nw) mmf_load8<TW>(nw, k0, K, vec_ok, wv[v]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) xv[v][i] = 0.0f;
-        }
-    }
     float ep_wdeq[R], ep_bias = 0.0f, ep_add = 0.0f, ep_lb = 0.0f, ep_state = 0.0f;
-    const int64_t ch = nb * 32 + (threadIdx.x & 31);            // output column / channel of the epilogue lanes
-    const int64_t Nseg = a.N / R;
-    if (threadIdx.x < 32 && ch < Nseg) {
+    const int ch = nb * 32 + (lane & 31);                       // output column / channel of the epilogue lanes
+    const bool ep_lane = wave == 0 && lane < 32 && ch < Nseg;
+    if (wave == 0) {
+        // the 32 outputs of an n-block share a scale (segments are multiples of 32 rows)
 #pragma unroll
-        for (int r = 0; r < R; ++r) ep_wdeq[r] = a.wdeq[(ch + r * NBseg * 32) / a.seg_rows];
-        if constexpr (EPI == EPI_PLAIN) {
-            if (a.bias) ep_bias = mmf_to_float(static_cast<const T*>(a.bias)[ch]);
-            if (a.addend) ep_add = mmf_to_float(static_cast<const T*>(a.addend)[row * a.N + ch]);
-        }
-        if constexpr (EPI == EPI_STEP) {
-            if (a.lb) ep_lb = a.lb[ch];
-            ep_state = a.state[row * Nseg + ch];
+        for (int r = 0; r < R; ++r) ep_wdeq[r] = a.wdeq[(uint32_t)((nb + r * NBseg) * 32) / (uint32_t)a.seg_rows];
+        if (ep_lane) {
+            if constexpr (EPI == EPI_PLAIN) {
+                if (a.bias) ep_bias = mmf_to_float(static_cast<const T*>(a.bias)[ch]);
+                if (a.addend) ep_add = mmf_to_float(static_cast<const T*>(a.addend)[(int64_t)row * a.N + ch]);
+            }
+            if constexpr (EPI == EPI_STEP) {
+                if (a.lb) ep_lb = a.lb[ch];
+                ep_state = a.state[(int64_t)row * Nseg + ch];
+            }
         }
     }
 
     // ---- prologue stage 1: the value the BitLinear sees, v (rounded to T like the tensor it replaces)
+    float xv[NV][4], av[HAS_AUX ? NV : 1][4];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int k0 = (v * kGemvThreads + (int)threadIdx.x) * kGemvEl;
+        raw4_unpack<T>(xraw[v], xv[v]);
+        if constexpr (HAS_AUX) raw4_unpack<T>(araw[v], av[v]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (k0 + i >= K) xv[v][i] = 0.0f;
+    }
     if constexpr (PRO == PRO_RESNORM) {
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
-            const int64_t k0 = ((int64_t)v * kGemvThreads + threadIdx.x) * 8;
-            if (k0 < K) {
+            const int k0 = (v * kGemvThreads + (int)threadIdx.x) * kGemvEl;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) xv[v][i] = __fadd_rn(xv[v][i], av[v][i]);
-                if (a.res_out && blockIdx.x == 0)
-                    mmf_store8<T>(static_cast<T*>(a.res_out) + row * K, k0, K, (K % 8) == 0, xv[v]);
-            }
+            for (int i = 0; i < 4; ++i) xv[v][i] = k0 + i < K ? __fadd_rn(xv[v][i], av[v][i]) : 0.0f;
+            if (a.res_out && blockIdx.x == 0) raw4_store<T, VEC>(static_cast<T*>(a.res_out) + (int64_t)row * K, k0, K, xv[v]);
         }
     }
     if constexpr (PRO == PRO_NORM || PRO == PRO_RESNORM || PRO == PRO_GATEDNORM) {
@@ -161,33 +220,31 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
 #pragma unroll
         for (int v = 0; v < NV; ++v)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) s1 += (double)xv[v][i] * (double)xv[v][i];
+            for (int i = 0; i < 4; ++i) s1 += (double)xv[v][i] * (double)xv[v][i];
         s1 = block_sum_once<kGemvWaves>(s1, red_a);
         const float rstd1 = mmf_rstd(s1, K, a.eps1);
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
-            const int64_t k0 = ((int64_t)v * kGemvThreads + threadIdx.x) * 8;
-            if (k0 < K) {
+            const int k0 = (v * kGemvThreads + (int)threadIdx.x) * kGemvEl;
+            float w1v[4];
+            raw4_unpack<TW>(w1raw[v], w1v);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    float y = __fmul_rn(__fmul_rn(xv[v][i], rstd1), w1v[v][i]);
-                    if constexpr (PRO == PRO_GATEDNORM) y = __fmul_rn(__fmul_rn(y, av[v][i]), mmf_sigmoid(av[v][i]));
-                    xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(y) : 0.0f;
-                }
+            for (int i = 0; i < 4; ++i) {
+                float y = __fmul_rn(__fmul_rn(xv[v][i], rstd1), w1v[i]);
+                if constexpr (PRO == PRO_GATEDNORM) y = __fmul_rn(__fmul_rn(y, av[v][i]), mmf_sigmoid(av[v][i]));
+                xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(y) : 0.0f;
             }
         }
     }
     if constexpr (PRO == PRO_SWIGLU) {
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
-            const int64_t k0 = ((int64_t)v * kGemvThreads + threadIdx.x) * 8;
-            if (k0 < K) {
+            const int k0 = (v * kGemvThreads + (int)threadIdx.x) * kGemvEl;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const float g = xv[v][i];
-                    const float z = __fdiv_rn(__fmul_rn(g, av[v][i]), __fadd_rn(1.0f, mmf_exp(-g)));
-                    xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(z) : 0.0f;
-                }
+            for (int i = 0; i < 4; ++i) {
+                const float g = xv[v][i];
+                const float z = __fdiv_rn(__fmul_rn(g, av[v][i]), __fadd_rn(1.0f, mmf_exp(-g)));
+                xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(z) : 0.0f;
             }
         }
     }
@@ -197,21 +254,20 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
 #pragma unroll
     for (int v = 0; v < NV; ++v)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
+        for (int i = 0; i < 4; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
     ss = block_sum_once<kGemvWaves>(ss, red_b);
     const float rstd = mmf_rstd(ss, K, a.eps);
     float amax = 0.0f;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        const int64_t k0 = ((int64_t)v * kGemvThreads + threadIdx.x) * 8;
-        if (k0 < K) {
+        float wv[4];
+        if (nw) raw4_unpack<TW>(nwraw[v], wv);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                float y = __fmul_rn(xv[v][i], rstd);
-                if (nw) y = __fmul_rn(y, wv[v][i]);
-                xv[v][i] = y;
-                amax = fmaxf(amax, fabsf(y));
-            }
+        for (int i = 0; i < 4; ++i) {
+            float y = __fmul_rn(xv[v][i], rstd);
+            if (nw) y = __fmul_rn(y, wv[i]);
+            xv[v][i] = y;                                       // elements past K are exact zeros and stay so
+            amax = fmaxf(amax, fabsf(y));
         }
     }
     amax = block_max_once<kGemvWaves>(amax, red_f);
@@ -219,17 +275,16 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
     int qs = 0;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        const int64_t k0 = ((int64_t)v * kGemvThreads + threadIdx.x) * 8;
+        const int k0 = (v * kGemvThreads + (int)threadIdx.x) * kGemvEl;
         if (k0 < Kp) {
-            uint32_t lo = 0, hi = 0;
+            uint32_t packed4 = 0;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
+            for (int i = 0; i < 4; ++i) {
                 const int c = (k0 + i < K) ? mmf_code(xv[v][i], scale) : 0;
                 qs += c;
-                const uint32_t b = (uint32_t)(c & 0xff) << (8 * (i & 3));
-                if (i < 4) lo |= b; else hi |= b;
+                packed4 |= (uint32_t)(c & 0xff) << (8 * i);
             }
-            *reinterpret_cast<uint2*>(q_lds + k0) = make_uint2(lo, hi);
+            *reinterpret_cast<uint32_t*>(q_lds + k0) = packed4;
         }
     }
     qs = mmf_wave_sum(qs);
@@ -242,8 +297,8 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = 0;
 #pragma unroll
-    for (int i = 0; i < kGemvMaxBlocksPerWave; ++i) {
-        const int64_t kb = wave + (int64_t)i * kGemvWaves;
+    for (int i = 0; i < BPW; ++i) {
+        const int kb = wave + i * kGemvWaves;
         if (kb < KB) {
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
@@ -265,7 +320,7 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
         if (lane < 32) part[r][wave][lane] = acc[r];
     }
     __syncthreads();
-    if (threadIdx.x < 32 && ch < Nseg) {
+    if (ep_lane) {
         int qtot = 0;
 #pragma unroll
         for (int w = 0; w < kGemvWaves; ++w) qtot += red_q[w];
@@ -275,14 +330,14 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
         for (int r = 0; r < R; ++r) {
             int tot = 0;
 #pragma unroll
-            for (int w = 0; w < kGemvWaves; ++w) tot += part[r][w][threadIdx.x];
+            for (int w = 0; w < kGemvWaves; ++w) tot += part[r][w][lane];
             res[r] = __fmul_rn(__fmul_rn((float)(tot - qtot), deq), ep_wdeq[r]);
         }
         if constexpr (EPI == EPI_PLAIN) {
             float o = res[0];
             if (a.bias) o = __fadd_rn(o, ep_bias);
             if (a.addend) o = __fadd_rn(mmf_round_to<T>(o), ep_add);
-            static_cast<T*>(a.out)[row * a.N + ch] = mmf_from_float<T>(o);
+            static_cast<T*>(a.out)[(int64_t)row * a.N + ch] = mmf_from_float<T>(o);
         } else if constexpr (EPI == EPI_STEP) {
             // res = raw i, f, g projections of channel ch (each rounded to T like the tensors they replace)
             const float iv = mmf_round_to<T>(res[0]), fv = mmf_round_to<T>(res[1]);
@@ -291,59 +346,61 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
             const float go = mmf_round_to<T>(s);
             const float xo = mmf_round_to<T>(__fdiv_rn(__fmul_rn(iv, __fsub_rn(1.0f, go)), __fadd_rn(1.0f, mmf_exp(-iv))));
             const float h = __fadd_rn(__fmul_rn(go, ep_state), xo);
-            a.state[row * Nseg + ch] = h;
-            static_cast<T*>(a.out)[row * Nseg + ch] = mmf_from_float<T>(h);
-            static_cast<T*>(a.g_out)[row * Nseg + ch] = mmf_from_float<T>(res[2]);
+            a.state[(int64_t)row * Nseg + ch] = h;
+            static_cast<T*>(a.out)[(int64_t)row * Nseg + ch] = mmf_from_float<T>(h);
+            static_cast<T*>(a.g_out)[(int64_t)row * Nseg + ch] = mmf_from_float<T>(res[2]);
         } else {
             const float g = mmf_round_to<T>(res[0]), u = mmf_round_to<T>(res[1]);
-            static_cast<T*>(a.out)[row * Nseg + ch] =
+            static_cast<T*>(a.out)[(int64_t)row * Nseg + ch] =
                 mmf_from_float<T>(__fdiv_rn(__fmul_rn(g, u), __fadd_rn(1.0f, mmf_exp(-g))));
         }
     }
 }
 
 template <typename T, typename TW, int PRO, int EPI>
-int launch_gemv(const GemvArgs& a, int64_t M, hipStream_t s) {
+int launch_gemv(const GemvArgs& a, int64_t M, bool vec, hipStream_t s) {
     constexpr int R = EPI == EPI_STEP ? 3 : EPI == EPI_SWIGLU ? 2 : 1;
-    const int64_t nv = mmf_ceil_div(a.Kp, (int64_t)kGemvThreads * 8);
+    const int nv = (int)mmf_ceil_div((int64_t)a.Kp, (int64_t)kGemvThreads * kGemvEl);
     dim3 grid((unsigned)mmf_ceil_div(a.N / R, 32), (unsigned)M), block(kGemvThreads);
     const size_t lds = (size_t)a.Kp;
-    if (nv <= 1) bitlinear_gemv_kernel<T, TW, 1, PRO, EPI><<<grid, block, lds, s>>>(a);
-    else if (nv <= 2) bitlinear_gemv_kernel<T, TW, 2, PRO, EPI><<<grid, block, lds, s>>>(a);
-    else return MMF_ERR_WIDE;
+    if (!vec) bitlinear_gemv_kernel<T, TW, kGemvMaxNV, PRO, EPI, false><<<grid, block, lds, s>>>(a);   // ragged shapes: one generic build
+    else if (nv <= 1) bitlinear_gemv_kernel<T, TW, 1, PRO, EPI, true><<<grid, block, lds, s>>>(a);
+    else if (nv <= 2) bitlinear_gemv_kernel<T, TW, 2, PRO, EPI, true><<<grid, block, lds, s>>>(a);
+    else if (nv <= 3) bitlinear_gemv_kernel<T, TW, 3, PRO, EPI, true><<<grid, block, lds, s>>>(a);
+    else bitlinear_gemv_kernel<T, TW, 4, PRO, EPI, true><<<grid, block, lds, s>>>(a);
     MMF_CHECK_LAUNCH();
     return 0;
 }
 
 template <typename T, typename TW>
-int dispatch_gemv_kind(const GemvArgs& a, int64_t M, int pro, int epi, hipStream_t s) {
+int dispatch_gemv_kind(const GemvArgs& a, int64_t M, int pro, int epi, bool vec, hipStream_t s) {
     // the combinations a decode step uses
     if (epi == EPI_PLAIN) {
         switch (pro) {
-            case PRO_PLAIN: return launch_gemv<T, TW, PRO_PLAIN, EPI_PLAIN>(a, M, s);
-            case PRO_NORM: return launch_gemv<T, TW, PRO_NORM, EPI_PLAIN>(a, M, s);
-            case PRO_RESNORM: return launch_gemv<T, TW, PRO_RESNORM, EPI_PLAIN>(a, M, s);
-            case PRO_GATEDNORM: return launch_gemv<T, TW, PRO_GATEDNORM, EPI_PLAIN>(a, M, s);
-            case PRO_SWIGLU: return launch_gemv<T, TW, PRO_SWIGLU, EPI_PLAIN>(a, M, s);
+            case PRO_PLAIN: return launch_gemv<T, TW, PRO_PLAIN, EPI_PLAIN>(a, M, vec, s);
+            case PRO_NORM: return launch_gemv<T, TW, PRO_NORM, EPI_PLAIN>(a, M, vec, s);
+            case PRO_RESNORM: return launch_gemv<T, TW, PRO_RESNORM, EPI_PLAIN>(a, M, vec, s);
+            case PRO_GATEDNORM: return launch_gemv<T, TW, PRO_GATEDNORM, EPI_PLAIN>(a, M, vec, s);
+            case PRO_SWIGLU: return launch_gemv<T, TW, PRO_SWIGLU, EPI_PLAIN>(a, M, vec, s);
         }
     } else if (epi == EPI_STEP) {
-        if (pro == PRO_NORM) return launch_gemv<T, TW, PRO_NORM, EPI_STEP>(a, M, s);
-        if (pro == PRO_PLAIN) return launch_gemv<T, TW, PRO_PLAIN, EPI_STEP>(a, M, s);
+        if (pro == PRO_NORM) return launch_gemv<T, TW, PRO_NORM, EPI_STEP>(a, M, vec, s);
+        if (pro == PRO_PLAIN) return launch_gemv<T, TW, PRO_PLAIN, EPI_STEP>(a, M, vec, s);
     } else if (epi == EPI_SWIGLU) {
-        if (pro == PRO_RESNORM) return launch_gemv<T, TW, PRO_RESNORM, EPI_SWIGLU>(a, M, s);
-        if (pro == PRO_PLAIN) return launch_gemv<T, TW, PRO_PLAIN, EPI_SWIGLU>(a, M, s);
+        if (pro == PRO_RESNORM) return launch_gemv<T, TW, PRO_RESNORM, EPI_SWIGLU>(a, M, vec, s);
+        if (pro == PRO_PLAIN) return launch_gemv<T, TW, PRO_PLAIN, EPI_SWIGLU>(a, M, vec, s);
     }
     return MMF_ERR_ARG;
 }
 
 template <typename T>
-int dispatch_gemv_w(const GemvArgs& a, int64_t M, int pro, int epi, int x_dtype, int w_dtype, hipStream_t s) {
-    if (w_dtype == MMF_F32) return dispatch_gemv_kind<T, float>(a, M, pro, epi, s);
-    if (w_dtype == x_dtype) return dispatch_gemv_kind<T, T>(a, M, pro, epi, s);
+int dispatch_gemv_w(const GemvArgs& a, int64_t M, int pro, int epi, int x_dtype, int w_dtype, bool vec, hipStream_t s) {
+    if (w_dtype == MMF_F32) return dispatch_gemv_kind<T, float>(a, M, pro, epi, vec, s);
+    if (w_dtype == x_dtype) return dispatch_gemv_kind<T, T>(a, M, pro, epi, vec, s);
     return MMF_ERR_ARG;
 }
 
-bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+bool aligned(const void* p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
 
 }  // namespace
 
@@ -365,22 +422,26 @@ int mmf_bitlinear_gemv_fused(int prologue, int epilogue, const void* x, int64_t 
     if (prologue >= PRO_NORM && prologue <= PRO_GATEDNORM && !w1) return MMF_ERR_ARG;
     if (epilogue == EPI_STEP && (N % 96 != 0 || !g_out || !state || bias || addend)) return MMF_ERR_ARG;
     if (epilogue == EPI_SWIGLU && (N % 64 != 0 || bias || addend)) return MMF_ERR_ARG;
+    if (K > INT32_MAX - 128 || N > INT32_MAX - 96 || seg_rows > INT32_MAX) return MMF_ERR_WIDE;
+    if (seg_rows % 32 != 0 && seg_rows < N) return MMF_ERR_ARG;   // stacked segments are whole n-blocks
     GemvArgs a{};
     a.x = x; a.aux = aux ? aux : x; a.res_out = res_out; a.w1 = w1; a.norm_w = norm_weight;
     a.packed = static_cast<const uint4*>(packed); a.wdeq = wdeq; a.bias = bias; a.addend = addend; a.out = out;
     a.g_out = g_out; a.lb = lower_bound; a.state = state;
-    a.K = K; a.Kp = mmf_round_up(K, 128); a.N = N; a.seg_rows = seg_rows; a.ldx = ldx; a.ldaux = aux ? ldaux : ldx;
+    a.K = (int)K; a.Kp = (int)mmf_round_up(K, 128); a.N = (int)N; a.seg_rows = (int)seg_rows; a.ldx = ldx;
+    a.ldaux = aux ? ldaux : ldx;
     a.eps = eps; a.eps1 = eps1;
     if (a.Kp > kGemvMaxK) return MMF_ERR_WIDE;
-    if (!al16(packed)) return MMF_ERR_ALIGN;
-    if (K % 8 == 0 && ldx % 8 == 0 && a.ldaux % 8 == 0 &&
-        !(al16(x) && al16(a.aux) && al16(w1) && al16(norm_weight) && al16(res_out)))
-        return MMF_ERR_ALIGN;
+    if (!aligned(packed, 16)) return MMF_ERR_ALIGN;
     if (!norm_weight && !w1) weight_dtype = MMF_F32;
+    const size_t xa = 4 * (x_dtype == MMF_F32 ? 4 : 2), wa = 4 * (weight_dtype == MMF_F32 ? 4 : 2);
+    const bool vec = K % 4 == 0 && ldx % 4 == 0 && a.ldaux % 4 == 0;
+    if (vec && !(aligned(x, xa) && aligned(a.aux, xa) && aligned(res_out, xa) && aligned(w1, wa) && aligned(norm_weight, wa)))
+        return MMF_ERR_ALIGN;
     switch (x_dtype) {
-        case MMF_F32: return dispatch_gemv_w<float>(a, M, prologue, epilogue, x_dtype, weight_dtype, stream);
-        case MMF_BF16: return dispatch_gemv_w<bf16_t>(a, M, prologue, epilogue, x_dtype, weight_dtype, stream);
-        case MMF_F16: return dispatch_gemv_w<f16_t>(a, M, prologue, epilogue, x_dtype, weight_dtype, stream);
+        case MMF_F32: return dispatch_gemv_w<float>(a, M, prologue, epilogue, x_dtype, weight_dtype, vec, stream);
+        case MMF_BF16: return dispatch_gemv_w<bf16_t>(a, M, prologue, epilogue, x_dtype, weight_dtype, vec, stream);
+        case MMF_F16: return dispatch_gemv_w<f16_t>(a, M, prologue, epilogue, x_dtype, weight_dtype, vec, stream);
     }
     return MMF_ERR_ARG;
 }

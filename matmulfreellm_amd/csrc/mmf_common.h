@@ -127,21 +127,45 @@ __device__ __forceinline__ float mmf_sigmoid(float x) {
     return __fdiv_rn(1.0f, __fadd_rn(1.0f, mmf_exp(-x)));
 }
 
-// ---------------------------------------------------------------- reductions (wave64 butterfly)
+// ---------------------------------------------------------------- reductions (wave64)
+// Rows of 16 lanes are folded with four DPP moves (quad swaps, half-row mirror, row mirror: a few
+// cycles each, where a generic cross-lane shuffle goes through the LDS crossbar); the four row
+// results are then read as scalars and combined in row order.  Every lane ends with the same bits.
+template <int CTRL>
+__device__ __forceinline__ int mmf_dpp(int v) { return __builtin_amdgcn_mov_dpp(v, CTRL, 0xf, 0xf, true); }
+template <int CTRL>
+__device__ __forceinline__ float mmf_dpp(float v) { return __int_as_float(mmf_dpp<CTRL>(__float_as_int(v))); }
+template <int CTRL>
+__device__ __forceinline__ double mmf_dpp(double v) {
+    return __hiloint2double(mmf_dpp<CTRL>(__double2hiint(v)), mmf_dpp<CTRL>(__double2loint(v)));
+}
+__device__ __forceinline__ int mmf_readlane(int v, int l) { return __builtin_amdgcn_readlane(v, l); }
+__device__ __forceinline__ float mmf_readlane(float v, int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), l)); }
+__device__ __forceinline__ double mmf_readlane(double v, int l) {
+    return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(v), l), __builtin_amdgcn_readlane(__double2loint(v), l));
+}
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140;
+
 __device__ __forceinline__ double mmf_wave_sum(double v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
+    v += mmf_dpp<kDppXor1>(v);
+    v += mmf_dpp<kDppXor2>(v);
+    v += mmf_dpp<kDppHalfMirror>(v);
+    v += mmf_dpp<kDppMirror>(v);
+    return ((mmf_readlane(v, 0) + mmf_readlane(v, 16)) + mmf_readlane(v, 32)) + mmf_readlane(v, 48);
 }
 __device__ __forceinline__ float mmf_wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
+    v = fmaxf(v, mmf_dpp<kDppXor1>(v));
+    v = fmaxf(v, mmf_dpp<kDppXor2>(v));
+    v = fmaxf(v, mmf_dpp<kDppHalfMirror>(v));
+    v = fmaxf(v, mmf_dpp<kDppMirror>(v));
+    return fmaxf(fmaxf(mmf_readlane(v, 0), mmf_readlane(v, 16)), fmaxf(mmf_readlane(v, 32), mmf_readlane(v, 48)));
 }
 __device__ __forceinline__ int mmf_wave_sum(int v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
+    v += mmf_dpp<kDppXor1>(v);
+    v += mmf_dpp<kDppXor2>(v);
+    v += mmf_dpp<kDppHalfMirror>(v);
+    v += mmf_dpp<kDppMirror>(v);
+    return mmf_readlane(v, 0) + mmf_readlane(v, 16) + mmf_readlane(v, 32) + mmf_readlane(v, 48);
 }
 
 // Block-wide reductions for blocks of NW waves; `red` is LDS scratch of >= NW entries
