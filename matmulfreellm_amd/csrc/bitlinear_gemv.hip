@@ -27,8 +27,7 @@
 //              a lane holds 64 weights of one output row, expands each dword to four
 //              byte-wide code dwords (shift + mask) and accumulates with v_dot4_i32_i8
 //              against the broadcast activation bytes read from LDS.
-//   epilogue : halves of the wave are folded with one cross-lane move, the 8 wave partials
-//              through LDS;  r = T(fp32(acc - sum(q)) * deq_row * deq_weight (+ bias)), then
+//   epilogue : the two k-halves of the 8 waves' lanes are summed through LDS;  r = T(fp32(acc - sum(q)) * deq_row * deq_weight (+ bias)), then
 //                EPI_PLAIN   out = r, or T(r + addend)                          (residual add)
 //                EPI_STEP    R = 3 (i, f, g rows of the same 32 channels): gate math, one
 //                            recurrence step on the fp32 state, writes o and g
@@ -63,6 +62,7 @@ struct GemvArgs {
     int64_t ldx, ldaux;
     int K, Kp, N, seg_rows;                                     // all < 2^31 (checked by the entry point)
     float eps, eps1;
+    double inv_K;         // RN(1 / K)
 };
 
 template <int NW>
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
     __shared__ double red_a[kGemvWaves], red_b[kGemvWaves];
     __shared__ float red_f[kGemvWaves];
     __shared__ int red_q[kGemvWaves];
-    __shared__ int part[R][kGemvWaves][32];
+    __shared__ int2 part[R][kGemvWaves][32];                    // .x / .y: the two k-halves of a wave's lanes
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nb = blockIdx.x, row = blockIdx.y;
@@ -222,7 +222,7 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
 #pragma unroll
             for (int i = 0; i < 4; ++i) s1 += (double)xv[v][i] * (double)xv[v][i];
         s1 = block_sum_once<kGemvWaves>(s1, red_a);
-        const float rstd1 = mmf_rstd(s1, K, a.eps1);
+        const float rstd1 = mmf_rstd(s1, K, a.inv_K, a.eps1);
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int k0 = (v * kGemvThreads + (int)threadIdx.x) * kGemvEl;
@@ -256,7 +256,7 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
 #pragma unroll
         for (int i = 0; i < 4; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
     ss = block_sum_once<kGemvWaves>(ss, red_b);
-    const float rstd = mmf_rstd(ss, K, a.eps);
+    const float rstd = mmf_rstd(ss, K, a.inv_K, a.eps);
     float amax = 0.0f;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
@@ -316,8 +316,7 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        acc[r] += __shfl_xor(acc[r], 32, 64);
-        if (lane < 32) part[r][wave][lane] = acc[r];
+        reinterpret_cast<int*>(&part[r][wave][lane & 31])[half] = acc[r];
     }
     __syncthreads();
     if (ep_lane) {
@@ -330,7 +329,10 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
         for (int r = 0; r < R; ++r) {
             int tot = 0;
 #pragma unroll
-            for (int w = 0; w < kGemvWaves; ++w) tot += part[r][w][lane];
+            for (int w = 0; w < kGemvWaves; ++w) {
+                const int2 pr = part[r][w][lane];
+                tot += pr.x + pr.y;
+            }
             res[r] = __fmul_rn(__fmul_rn((float)(tot - qtot), deq), ep_wdeq[r]);
         }
         if constexpr (EPI == EPI_PLAIN) {
@@ -430,7 +432,7 @@ int mmf_bitlinear_gemv_fused(int prologue, int epilogue, const void* x, int64_t 
     a.g_out = g_out; a.lb = lower_bound; a.state = state;
     a.K = (int)K; a.Kp = (int)mmf_round_up(K, 128); a.N = (int)N; a.seg_rows = (int)seg_rows; a.ldx = ldx;
     a.ldaux = aux ? ldaux : ldx;
-    a.eps = eps; a.eps1 = eps1;
+    a.eps = eps; a.eps1 = eps1; a.inv_K = 1.0 / (double)K;
     if (a.Kp > kGemvMaxK) return MMF_ERR_WIDE;
     if (!aligned(packed, 16)) return MMF_ERR_ALIGN;
     if (!norm_weight && !w1) weight_dtype = MMF_F32;

@@ -446,6 +446,28 @@ __global__ __launch_bounds__(512) void bitlinear_mfma_skinny_kernel(MfmaArgs p) 
     };
 #pragma unroll
     for (int st = 0; st < PF; ++st) load_stage(st, wave + (int64_t)st * NWV);
+
+    // the epilogue's operands, requested now so that the end of the kernel waits for nothing
+    const T* bias = static_cast<const T*>(p.bias);
+    const T* addend = static_cast<const T*>(p.addend);
+    T* out = static_cast<T*>(p.out);
+    const int64_t n_ep = nb * 32 + (lane & 31);
+    const bool n_ok = n_ep < p.N;
+    const float ep_wdeq = p.wdeq[(uint32_t)(nb * 32) / (uint32_t)p.seg_rows];   // an n-block never straddles a segment
+    const float ep_bias = (bias && n_ok) ? mmf_to_float(bias[n_ep]) : 0.0f;
+    int ep_qsum[MB * 2];
+    float ep_deq[MB * 2], ep_add[MB * 2];
+#pragma unroll
+    for (int j = 0; j < MB * 2; ++j) {
+        const int e = threadIdx.x + j * 512;             // (mb, r, lane) flattened
+        const int r = (e >> 6) & 15, mb = e >> 10;
+        const int64_t m = (int64_t)mb * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        const int64_t mc = m < p.M ? m : 0;
+        ep_qsum[j] = p.qsum[mc];
+        ep_deq[j] = p.deq[mc];
+        ep_add[j] = (addend && n_ok) ? mmf_to_float(addend[mc * p.ldo + n_ep]) : 0.0f;
+    }
+
 #pragma unroll
     for (int it = 0; it < MAXK; ++it) {
         const int st = it % PF;
@@ -472,23 +494,19 @@ __global__ __launch_bounds__(512) void bitlinear_mfma_skinny_kernel(MfmaArgs p) 
         for (int r = 0; r < 16; ++r) red[wave][i][r][lane] = acc[i][r];
     __syncthreads();
 
-    const T* bias = static_cast<const T*>(p.bias);
-    const T* addend = static_cast<const T*>(p.addend);
-    T* out = static_cast<T*>(p.out);
 #pragma unroll
     for (int j = 0; j < MB * 2; ++j) {
         const int e = threadIdx.x + j * 512;             // (mb, r, lane) flattened
-        const int l = e & 63, r = (e >> 6) & 15, mb = e >> 10;
+        const int r = (e >> 6) & 15, mb = e >> 10;
         int tot = 0;
 #pragma unroll
-        for (int w = 0; w < NWV; ++w) tot += red[w][mb][r][l];
-        const int64_t m = (int64_t)mb * 32 + 8 * (r >> 2) + 4 * (l >> 5) + (r & 3);
-        const int64_t n = nb * 32 + (l & 31);
-        if (m < p.M && n < p.N) {
-            float o = __fmul_rn(__fmul_rn((float)(tot - p.qsum[m]), p.deq[m]), p.wdeq[(uint32_t)n / (uint32_t)p.seg_rows]);
-            if (bias) o = __fadd_rn(o, mmf_to_float(bias[n]));
-            if (addend) o = __fadd_rn(mmf_round_to<T>(o), mmf_to_float(addend[m * p.ldo + n]));
-            out[m * p.ldo + n] = mmf_from_float<T>(o);
+        for (int w = 0; w < NWV; ++w) tot += red[w][mb][r][lane];
+        const int64_t m = (int64_t)mb * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (m < p.M && n_ok) {
+            float o = __fmul_rn(__fmul_rn((float)(tot - ep_qsum[j]), ep_deq[j]), ep_wdeq);
+            if (bias) o = __fadd_rn(o, ep_bias);
+            if (addend) o = __fadd_rn(mmf_round_to<T>(o), ep_add[j]);
+            out[m * p.ldo + n_ep] = mmf_from_float<T>(o);
         }
     }
 }

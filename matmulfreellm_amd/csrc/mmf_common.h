@@ -74,6 +74,40 @@ __device__ __forceinline__ void mmf_load8(const T* __restrict__ p, int64_t k0, i
     }
 }
 
+// The same eight elements as they sit in memory.  Kernels whose cost is latency issue all of
+// their loads as raw vectors first and unpack them where they are used, so that no conversion
+// waits for one load before the next is issued.  Lanes with k0 >= K read the row start (vector
+// path) or zeros (element path); the caller discards them.
+template <typename T> struct Raw8 { uint4 a; };
+template <> struct Raw8<float> { float4 a, b; };
+
+template <typename T>
+__device__ __forceinline__ Raw8<T> mmf_load8_raw(const T* __restrict__ p, int64_t k0, int64_t K, bool vec_ok) {
+    Raw8<T> r;
+    if (vec_ok) {
+        const T* q = p + (k0 < K ? k0 : 0);
+        if constexpr (sizeof(T) == 4) {
+            r.a = reinterpret_cast<const float4*>(q)[0];
+            r.b = reinterpret_cast<const float4*>(q)[1];
+        } else {
+            r.a = *reinterpret_cast<const uint4*>(q);
+        }
+    } else {
+        T e[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) e[i] = p[k0 + i < K ? k0 + i : 0];
+        __builtin_memcpy(&r, e, sizeof(r));
+    }
+    return r;
+}
+template <typename T>
+__device__ __forceinline__ void mmf_unpack8(const Raw8<T>& r, float (&out)[8]) {
+    T e[8];
+    __builtin_memcpy(e, &r, sizeof(r));
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = mmf_to_float(e[i]);
+}
+
 template <typename T>
 __device__ __forceinline__ void mmf_store8(T* __restrict__ p, int64_t k0, int64_t K, bool vec_ok, const float (&in)[8]) {
     if (vec_ok) {
@@ -212,9 +246,17 @@ __device__ __forceinline__ int mmf_block_sum(int v, int* red) {
     return s;
 }
 
-// rstd = 1 / sqrt( fp32(sumsq / K) + eps )
-__device__ __forceinline__ float mmf_rstd(double sumsq, int64_t K, float eps) {
-    float var = (float)(sumsq / (double)K);
+// rstd = 1 / sqrt( fp32(sumsq / K) + eps ).
+// sumsq / K is the correctly rounded fp64 quotient without the division sequence: with
+// inv_K = RN(1 / K) from the host, q0 = sumsq * inv_K is within two ulps, one residual step
+// makes it faithful, and a second one (r exact through the fused multiply-add) lands on the
+// correctly rounded quotient (Markstein's theorem; K is a small integer, 0 <= sumsq < 2^200).
+__device__ __forceinline__ float mmf_rstd(double sumsq, int64_t K, double inv_K, float eps) {
+    const double Kd = (double)K;
+    double q = sumsq * inv_K;
+    q = fma(fma(-q, Kd, sumsq), inv_K, q);
+    q = fma(fma(-q, Kd, sumsq), inv_K, q);
+    const float var = (float)q;
     return __fdiv_rn(1.0f, sqrtf(__fadd_rn(var, eps)));   // sqrtf: correctly rounded (__fsqrt_rn is the native approximation)
 }
 

@@ -27,6 +27,7 @@ struct RowArgs {
     float* deq;             // [M]
     int* qsum;              // [M]
     int64_t M, K, Kp, ldx;   // ldx: row stride of x in elements
+    double inv_K;            // RN(1 / K)
     float eps;
     int q_tiled;            // 0: row-major [M, Kp]; 1: [ceil32(M)/32][Kp/16][32][16]
 };
@@ -80,7 +81,7 @@ __global__ __launch_bounds__(kThreads) void row_kernel(RowArgs a) {
         }
     }
     ss = mmf_block_sum<kWaves>(ss, red_d);
-    const float rstd = mmf_rstd(ss, K, a.eps);
+    const float rstd = mmf_rstd(ss, K, a.inv_K, a.eps);
 
     float amax = 0.0f;
 #pragma unroll
@@ -200,6 +201,7 @@ struct FusedQuantArgs {
     const float* lb; float* state;
     int8_t* q; float* deq; int* qsum;
     int64_t M, K, Kp;
+    double inv_K;            // RN(1 / K)
     float eps1, eps;
 };
 
@@ -216,25 +218,42 @@ __global__ __launch_bounds__(kThreads) void row_quant_fused_kernel(FusedQuantArg
     const TW* w1 = static_cast<const TW*>(a.w1);
     const TW* nw = static_cast<const TW*>(a.norm_w);
 
-    float xv[NV][8], av[PRO >= QPRO_RESNORM ? NV : 1][8], gv[PRO == QPRO_STEP_GATE ? NV : 1][8];
-    float w1v[PRO != QPRO_SWIGLU ? NV : 1][8], wv[NV][8], lbv[PRO == QPRO_STEP_GATE ? NV : 1][8], stv[PRO == QPRO_STEP_GATE ? NV : 1][8];
+    constexpr bool HAS_AUX = PRO >= QPRO_RESNORM, STEP = PRO == QPRO_STEP_GATE, HAS_W1 = PRO != QPRO_SWIGLU;
+    const bool vec_w = (K % 8) == 0;
+    // every load of the kernel first, raw; conversions only after the last one is issued
+    Raw8<T> xraw[NV], araw[HAS_AUX ? NV : 1], graw[STEP ? NV : 1];
+    Raw8<float> straw[STEP ? NV : 1], lbraw[STEP ? NV : 1];
+    Raw8<TW> w1raw[HAS_W1 ? NV : 1], nwraw[NV];
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
         const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
-        if (k0 < K) {
-            mmf_load8<T>(x, k0, K, vec_ok, xv[v]);
-            if constexpr (PRO >= QPRO_RESNORM) mmf_load8<T>(aux, k0, K, vec_ok, av[v]);
-            if constexpr (PRO == QPRO_STEP_GATE) {
-                mmf_load8<T>(aux2, k0, K, vec_ok, gv[v]);
-                mmf_load8<float>(a.state + row * K, k0, K, (K % 8) == 0, stv[v]);
-                if (a.lb) mmf_load8<float>(a.lb, k0, K, (K % 8) == 0, lbv[v]);
-            }
-            if constexpr (PRO != QPRO_SWIGLU) mmf_load8<TW>(w1, k0, K, (K % 8) == 0, w1v[v]);
-            if (nw) mmf_load8<TW>(nw, k0, K, (K % 8) == 0, wv[v]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) xv[v][i] = 0.0f;
+        xraw[v] = mmf_load8_raw<T>(x, k0, K, vec_ok);
+        if constexpr (HAS_AUX) araw[v] = mmf_load8_raw<T>(aux, k0, K, vec_ok);
+        if constexpr (STEP) {
+            graw[v] = mmf_load8_raw<T>(aux2, k0, K, vec_ok);
+            straw[v] = mmf_load8_raw<float>(a.state + row * K, k0, K, vec_w);
+            if (a.lb) lbraw[v] = mmf_load8_raw<float>(a.lb, k0, K, vec_w);
         }
+        if constexpr (HAS_W1) w1raw[v] = mmf_load8_raw<TW>(w1, k0, K, vec_w);
+        if (nw) nwraw[v] = mmf_load8_raw<TW>(nw, k0, K, vec_w);
+    }
+    float xv[NV][8], av[HAS_AUX ? NV : 1][8], gv[STEP ? NV : 1][8];
+    float w1v[HAS_W1 ? NV : 1][8], wv[NV][8], lbv[STEP ? NV : 1][8], stv[STEP ? NV : 1][8];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
+        mmf_unpack8<T>(xraw[v], xv[v]);
+        if constexpr (HAS_AUX) mmf_unpack8<T>(araw[v], av[v]);
+        if constexpr (STEP) {
+            mmf_unpack8<T>(graw[v], gv[v]);
+            mmf_unpack8<float>(straw[v], stv[v]);
+            if (a.lb) mmf_unpack8<float>(lbraw[v], lbv[v]);
+        }
+        if constexpr (HAS_W1) mmf_unpack8<TW>(w1raw[v], w1v[v]);
+        if (nw) mmf_unpack8<TW>(nwraw[v], wv[v]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (k0 + i >= K) xv[v][i] = 0.0f;
     }
     if constexpr (PRO == QPRO_RESNORM) {
 #pragma unroll
@@ -279,7 +298,7 @@ __global__ __launch_bounds__(kThreads) void row_quant_fused_kernel(FusedQuantArg
         if ((threadIdx.x & 63) == 0) red_a[threadIdx.x >> 6] = s1;
         __syncthreads();
         s1 = red_a[0] + red_a[1] + red_a[2] + red_a[3];
-        const float rstd1 = mmf_rstd(s1, K, a.eps1);
+        const float rstd1 = mmf_rstd(s1, K, a.inv_K, a.eps1);
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
@@ -316,7 +335,7 @@ __global__ __launch_bounds__(kThreads) void row_quant_fused_kernel(FusedQuantArg
     if ((threadIdx.x & 63) == 0) red_b[threadIdx.x >> 6] = ss;
     __syncthreads();
     ss = red_b[0] + red_b[1] + red_b[2] + red_b[3];
-    const float rstd = mmf_rstd(ss, K, a.eps);
+    const float rstd = mmf_rstd(ss, K, a.inv_K, a.eps);
     float amax = 0.0f;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
@@ -368,6 +387,7 @@ int launch_fused_quant(const FusedQuantArgs& a, hipStream_t s) {
     dim3 grid((unsigned)a.M), block(kThreads);
     if (nv <= 1) row_quant_fused_kernel<T, TW, 1, PRO><<<grid, block, 0, s>>>(a);
     else if (nv <= 2) row_quant_fused_kernel<T, TW, 2, PRO><<<grid, block, 0, s>>>(a);
+    else if (nv <= 3) row_quant_fused_kernel<T, TW, 3, PRO><<<grid, block, 0, s>>>(a);
     else if (nv <= 4) row_quant_fused_kernel<T, TW, 4, PRO><<<grid, block, 0, s>>>(a);
     else return MMF_ERR_WIDE;
     MMF_CHECK_LAUNCH();
@@ -449,7 +469,7 @@ int mmf_rmsnorm(const void* x, const void* residual, const void* weight, void* y
         return MMF_ERR_ALIGN;
     RowArgs a{};
     a.x = x; a.residual = residual; a.weight = weight; a.y = y; a.residual_out = residual_out;
-    a.M = M; a.K = K; a.Kp = K; a.ldx = K; a.eps = eps;
+    a.M = M; a.K = K; a.inv_K = 1.0 / (double)K; a.Kp = K; a.ldx = K; a.eps = eps;
     return dispatch_x<ROW_NORM>(a, x_dtype, residual_dtype, weight_dtype, stream);
 }
 
@@ -464,7 +484,7 @@ int mmf_rmsnorm_swishgate(const void* x, int64_t ldx, const void* gate, const vo
         return MMF_ERR_ALIGN;
     RowArgs a{};
     a.x = x; a.gate = gate; a.residual = residual; a.weight = weight; a.y = y; a.residual_out = residual_out;
-    a.M = M; a.K = K; a.Kp = K; a.ldx = ldx; a.eps = eps;
+    a.M = M; a.K = K; a.inv_K = 1.0 / (double)K; a.Kp = K; a.ldx = ldx; a.eps = eps;
     return dispatch_x<ROW_GATE>(a, x_dtype, residual_dtype, weight_dtype, stream);
 }
 
@@ -484,7 +504,7 @@ int mmf_rmsnorm_quant(const void* x, const void* residual, const void* weight, i
     RowArgs a{};
     a.x = x; a.residual = residual; a.weight = weight; a.residual_out = residual_out;
     a.q = q; a.deq = deq; a.qsum = qsum;
-    a.M = M; a.K = K; a.Kp = mmf_round_up(K, 128); a.ldx = K; a.eps = eps; a.q_tiled = tiled;
+    a.M = M; a.K = K; a.inv_K = 1.0 / (double)K; a.Kp = mmf_round_up(K, 128); a.ldx = K; a.eps = eps; a.q_tiled = tiled;
     return dispatch_x<ROW_QUANT>(a, x_dtype, residual_dtype, weight_dtype, stream);
 }
 
@@ -503,7 +523,7 @@ int mmf_rmsnorm_quant_fused(int prologue, const void* x, int64_t ldx, const void
     FusedQuantArgs a{};
     a.x = x; a.aux = aux ? aux : x; a.aux2 = aux2 ? aux2 : x; a.ldx = ldx; a.ldaux = aux ? ldaux : ldx;
     a.ldaux2 = aux2 ? ldaux2 : ldx; a.res_out = res_out; a.w1 = w1; a.norm_w = norm_weight; a.lb = lower_bound; a.state = state;
-    a.q = q; a.deq = deq; a.qsum = qsum; a.M = M; a.K = K; a.Kp = mmf_round_up(K, 128); a.eps1 = eps1; a.eps = eps;
+    a.q = q; a.deq = deq; a.qsum = qsum; a.M = M; a.K = K; a.inv_K = 1.0 / (double)K; a.Kp = mmf_round_up(K, 128); a.eps1 = eps1; a.eps = eps;
     if (!aligned16(q)) return MMF_ERR_ALIGN;
     if (K % 8 == 0 && !(aligned16(x) && aligned16(a.aux) && aligned16(a.aux2) && aligned16(res_out) && aligned16(w1) &&
                         aligned16(norm_weight) && aligned16(lower_bound) && aligned16(state)))
