@@ -102,3 +102,24 @@ def test_layer_norm_linear_quant_fn_rejects_unsupported_forms():
         mm.layer_norm_linear_quant_fn(x, torch.ones(64), torch.zeros(64), w, None, is_rms_norm=True)
     with pytest.raises(NotImplementedError):
         mm.HGRNBitAttention(hidden_size=64, num_heads=1, use_short_conv=True)
+
+
+def test_division_free_quotient_is_the_correctly_rounded_one():
+    """The kernels' rstd uses q = s*y; q = fma(fma(-q,K,s), y, q) twice with y = RN(1/K) in place of
+    the fp64 division s / K (csrc/mmf_common.h, mmf_rstd).  Check the sequence against exact
+    rational arithmetic: it must give the correctly rounded quotient, i.e. what `/` gives."""
+    from fractions import Fraction
+    import random
+
+    def fma(a, b, c):
+        return float(Fraction(a) * Fraction(b) + Fraction(c))       # one rounding, like the hardware's
+
+    rng = random.Random(7)
+    for K in (1, 3, 7, 11, 100, 127, 2048, 5632, 8191, 4096, 33, 999, 65537, 100003):
+        y, Kd = 1.0 / K, float(K)
+        for _ in range(1500):
+            s = rng.random() * 10.0 ** rng.randint(-20, 12)
+            q = s * y
+            q = fma(fma(-q, Kd, s), y, q)
+            q = fma(fma(-q, Kd, s), y, q)
+            assert q == s / Kd, (K, s)
