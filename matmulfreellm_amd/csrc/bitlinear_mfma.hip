@@ -154,6 +154,68 @@ __device__ __forceinline__ void mfma_epilogue(const MfmaArgs& p, v16i (&acc)[WM]
     }
 }
 
+// Lean epilogue of the common case (16-byte stores possible, no bias): the accumulators were
+// started at -qsum[m], so a value costs one convert and two multiplies; lane-constant parts of the
+// store addresses are computed once; interior tiles skip the bounds tests.
+template <typename T, int WM, int WN>
+__device__ __forceinline__ void mfma_epilogue_fast(const MfmaArgs& p, v16i (&acc)[WM][WN], const EpiScales<WM, WN>& sc,
+                                                   unsigned char* smem, int lane, int wave, int wm, int64_t mb0, int64_t nb0) {
+    const T* addend = static_cast<const T*>(p.addend);
+    T* out = static_cast<T*>(p.out);
+    constexpr int E = sizeof(T);
+    constexpr int RS = WN * 32 * E + 16;          // LDS row stride of a wave's 32 x (WN*32) staging tile
+    constexpr int CPR = WN * 32 * E / 16;         // 16-byte chunks per row (divides 64)
+    constexpr int RPI = 64 / CPR;                 // rows covered by one 64-lane store
+    unsigned char* stage = smem + wave * (32 * RS);
+    const int half = lane >> 5, mloc = lane & 31;
+    const int cc = lane % CPR, rsub = lane / CPR;
+    const int64_t m_first = (mb0 + wm * WM) * 32, n_first = nb0 * 32;
+    const bool interior = m_first + WM * 32 <= p.M && n_first + WN * 32 <= p.N;
+    const int64_t n = n_first + cc * (16 / E);
+    const int64_t lane_off = (m_first + rsub) * p.ldo + n;         // element offset of this lane's first chunk
+    unsigned char* wr = stage + mloc * RS + 4 * half * E;
+    const unsigned char* rd = stage + rsub * RS + cc * 16;
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+        const float dq = sc.dq[i];
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float o[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) o[t] = __fmul_rn(__fmul_rn((float)acc[i][j][4 * g + t], dq), sc.wdq[j]);
+                unsigned char* w = wr + (j * 32 + 8 * g) * E;
+                if constexpr (E == 2) *reinterpret_cast<uint2*>(w) = make_uint2(pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]));
+                else *reinterpret_cast<float4*>(w) = make_float4(o[0], o[1], o[2], o[3]);
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int r0 = 0; r0 < 32; r0 += RPI) {
+            const int64_t off = lane_off + (int64_t)(i * 32 + r0) * p.ldo;
+            if (interior || (m_first + i * 32 + r0 + rsub < p.M && n < p.N)) {
+                uint4 v = *reinterpret_cast<const uint4*>(rd + r0 * RS);
+                if (addend) {
+                    const uint4 av = *reinterpret_cast<const uint4*>(addend + off);
+                    const T* pe = reinterpret_cast<const T*>(&v);
+                    const T* ae = reinterpret_cast<const T*>(&av);
+                    uint4 ov;
+                    T* oe = reinterpret_cast<T*>(&ov);
+#pragma unroll
+                    for (int e = 0; e < 16 / E; ++e) oe[e] = mmf_from_float<T>(__fadd_rn(mmf_to_float(pe[e]), mmf_to_float(ae[e])));
+                    v = ov;
+                }
+                *reinterpret_cast<uint4*>(out + off) = v;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
 template <typename T, int WGM, int WGN, int WM, int WN, int KSL>
 __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs p) {
     constexpr int NT = 64 * WGM * WGN;
@@ -272,131 +334,150 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs
     mfma_epilogue<T, WM, WN>(p, acc, sc, smem, lane, wave, wm, mb0, nb0);
 }
 
-// ------------------------------------------------------------------------------------------
-// Same tiling, but the A slab goes global -> LDS by DMA (global_load_lds_dwordx4: lane l's 16
-// bytes land at the wave-uniform LDS base + 16*l, which is exactly the fragment-tiled layout),
-// so no VGPRs stage it and no ds_write sits in the instruction stream; B is prefetched one
-// 128-wide k-block ahead in registers whatever the slab depth.  One barrier per slab of
-// KSL*128 inputs.
 typedef __attribute__((address_space(3))) void* mmf_lds_ptr;
 typedef __attribute__((address_space(1))) const void* mmf_glb_ptr;
 
-template <typename T, int WGM, int WGN, int WM, int WN, int KSL>
-__global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_dma_kernel(MfmaArgs p) {
+// ------------------------------------------------------------------------------------------
+// The large-M kernel.  Same tiling, but A goes global -> LDS by DMA (global_load_lds_dwordx4:
+// lane l's 16 bytes land at the wave-uniform LDS base + 16*l, which is exactly the
+// fragment-tiled layout), so no VGPRs stage it and no ds_write sits in the instruction stream.
+// Three A buffers of one 128-wide k-block each and ONE barrier per k-block,
+// placed after the second of its four k-steps.  At that barrier every wave has left the previous
+// k-block, so its buffer is free for the DMA of k-block s+2, and k-block s+1 (issued one k-block
+// earlier, waited for by each wave just before the barrier) is complete for everybody.  K-block
+// boundaries therefore carry no synchronisation: the A fragments of the next k-block's first
+// step are read while the current one's last MFMAs run, and the matrix pipe never drains.
+// FAST (chosen by the launcher): 16-byte stores possible and no bias -> lean epilogue, accumulators start at -qsum.
+template <typename T, int WGM, int WGN, int WM, int WN, bool FAST>
+__global__ __launch_bounds__(64 * WGM * WGN, (WM * WN <= 4 ? 4 : 1))   // small wave tiles: 4 waves per SIMD = two workgroups per CU
+void bitlinear_mfma_dma3_kernel(MfmaArgs p) {
     constexpr int NW = WGM * WGN;
     constexpr int BMB = WGM * WM;
     constexpr int BNB = WGN * WN;
-    constexpr int CH = KSL * 4096;                 // bytes of one m-block's slab
-    constexpr int WPIECES = BMB * CH / 1024;       // 1 KiB wave-loads per slab
+    constexpr int CH = 4096;                       // bytes of one m-block's k-block
+    constexpr int BUF = BMB * CH;
+    constexpr int WPIECES = BMB * CH / 1024;       // 1 KiB wave-loads per k-block
     constexpr int NDMA = (WPIECES + NW - 1) / NW;  // per wave
+    static_assert(WPIECES % NW == 0, "every wave issues the same number of DMA pieces");
     extern __shared__ __align__(16) unsigned char smem[];
 
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keep it in a scalar register
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
     int64_t wg = blockIdx.x;
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
     if (total % 8 == 0) wg = (wg % 8) * (total / 8) + wg / 8;
     const int64_t tile_m = wg / p.tiles_n, tile_n = wg % p.tiles_n;
     const int64_t MB = (p.M + 31) >> 5, NB = (p.N + 31) >> 5;
-    const int64_t KB = p.Kp >> 7, KG = p.Kp >> 4;
+    const int KB = (int)(p.Kp >> 7);
+    const int64_t KG = p.Kp >> 4;
     const int64_t mb0 = tile_m * BMB, nb0 = tile_n * BNB + wn * WN;
     EpiScales<WM, WN> sc;
     mfma_prefetch_scales<WM, WN>(p, sc, lane, wm, mb0, nb0);
 
-    v16i acc[WM][WN];
-#pragma unroll
-    for (int i = 0; i < WM; ++i)
-#pragma unroll
-        for (int j = 0; j < WN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-
-    // wave-load w of a slab: m-block chunk = w / (CH/1024), 1 KiB piece `within` of that chunk's slab
-    auto dma_slab = [&](int64_t kb, int buf) {
+    auto dma_block = [&](int kb, int boff) {                      // k-block kb -> buffer at byte offset boff
 #pragma unroll
         for (int i = 0; i < NDMA; ++i) {
             const int w = i * NW + wave;
-            if (w < WPIECES) {
-                const int chunk = w / (CH / 1024), within = w % (CH / 1024);
-                int64_t mb = mb0 + chunk;
-                if (mb >= MB) mb = MB - 1;                       // rows past M are never stored: any valid data will do
-                int64_t kg = kb * 8 + within * 2;                // 16-input groups; one 1 KiB piece = 2 groups
-                if (kg + 2 > KG) kg = KG - 2;                    // k-blocks past Kp are skipped by the compute loop
-                const unsigned char* g = reinterpret_cast<const unsigned char*>(p.a) + (mb * KG + kg) * 512 + lane * 16;
-                __builtin_amdgcn_global_load_lds((mmf_glb_ptr)g, (mmf_lds_ptr)(smem + buf * (BMB * CH) + w * 1024), 16, 0, 0);
-            }
+            const int chunk = w >> 2, within = w & 3;             // 4 pieces per m-block
+            int64_t mb = mb0 + chunk;
+            if (mb >= MB) mb = MB - 1;                            // rows past M are never stored: any valid data will do
+            const int kbc = kb < KB ? kb : KB - 1;                // past the end: harmless re-read, never consumed
+            const unsigned char* g = reinterpret_cast<const unsigned char*>(p.a) + (mb * KG + kbc * 8 + within * 2) * 512 + lane * 16;
+            __builtin_amdgcn_global_load_lds((mmf_glb_ptr)g, (mmf_lds_ptr)(smem + boff + w * 1024), 16, 0, 0);
         }
     };
-    auto load_b = [&](int64_t kb, uint4 (&dst)[WN]) {
+    auto load_b = [&](int kb, uint4 (&dst)[WN]) {                 // unconditional: the barrier's vmcnt counts on WN loads
 #pragma unroll
         for (int j = 0; j < WN; ++j) {
-            dst[j] = make_uint4(0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u);
-            if (nb0 + j < NB && kb < KB) dst[j] = p.b[((nb0 + j) * KB + kb) * 64 + lane];
+            const int64_t nb = nb0 + j < NB ? nb0 + j : NB - 1;   // columns past N are never stored
+            const int kbc = kb < KB ? kb : KB - 1;                // past the end: never consumed
+            dst[j] = p.b[(nb * KB + kbc) * 64 + lane];
+        }
+    };
+    auto expand_b = [&](const uint4 (&src)[WN], int ks, v4i (&bf)[WN]) {
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+            const uint32_t w = ks == 0 ? src[j].x : ks == 1 ? src[j].y : ks == 2 ? src[j].z : src[j].w;
+            bf[j][0] = (int)(w & 0x03030303u);
+            bf[j][1] = (int)((w >> 2) & 0x03030303u);
+            bf[j][2] = (int)((w >> 4) & 0x03030303u);
+            bf[j][3] = (int)((w >> 6) & 0x03030303u);
         }
     };
 
-    uint4 breg[WN], bnext[WN];
-    dma_slab(0, 0);
+    // B runs two k-blocks ahead: the loads of k-block s+2 are the only vector-memory operations
+    // younger than the DMA of k-block s+1 when the barrier of k-block s waits for that DMA
+    uint4 breg[WN], bnext[WN], bnext2[WN];
+    dma_block(0, 0);
+    dma_block(1, BUF);
     load_b(0, breg);
-    __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): this wave's DMA has landed
+    load_b(1, bnext);
+    __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): this wave's pieces of k-blocks 0 and 1 have landed
     __syncthreads();
 
-    for (int64_t kb0 = 0; kb0 < KB; kb0 += KSL) {
-        const int buf = (int)((kb0 / KSL) & 1);
-        if (kb0 + KSL < KB) dma_slab(kb0 + KSL, buf ^ 1);
-        const unsigned char* abase = smem + buf * (BMB * CH) + (wm * WM) * CH + lane * 16;
+    // a lane's 16 accumulator registers of one tile all belong to output row (lane % 32)
+    v16i acc[WM][WN];
 #pragma unroll
-        for (int q = 0; q < KSL; ++q) {
-            const int64_t kb = kb0 + q;
-            if (kb < KB) {                                       // uniform over the workgroup
-                load_b(kb + 1, bnext);
-                v4i af[2][WM];
+    for (int i = 0; i < WM; ++i) {
+        const int init = FAST ? -sc.qs[i] : 0;
 #pragma unroll
-                for (int i = 0; i < WM; ++i) af[0][i] = *reinterpret_cast<const v4i*>(abase + i * CH + q * 4096);
+        for (int j = 0; j < WN; ++j)
 #pragma unroll
-                for (int ks = 0; ks < 4; ++ks) {
-                    if (ks + 1 < 4) {
-#pragma unroll
-                        for (int i = 0; i < WM; ++i)
-                            af[(ks + 1) & 1][i] = *reinterpret_cast<const v4i*>(abase + i * CH + q * 4096 + (ks + 1) * 1024);
-                    }
-                    v4i bf[WN];
-#pragma unroll
-                    for (int j = 0; j < WN; ++j) {
-                        const uint32_t w = ks == 0 ? breg[j].x : ks == 1 ? breg[j].y : ks == 2 ? breg[j].z : breg[j].w;
-                        bf[j][0] = (int)(w & 0x03030303u);
-                        bf[j][1] = (int)((w >> 2) & 0x03030303u);
-                        bf[j][2] = (int)((w >> 4) & 0x03030303u);
-                        bf[j][3] = (int)((w >> 6) & 0x03030303u);
-                    }
-#pragma unroll
-                    for (int i = 0; i < WM; ++i)
-#pragma unroll
-                        for (int j = 0; j < WN; ++j)
-                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[ks & 1][i], acc[i][j], 0, 0, 0);
-                }
-#pragma unroll
-                for (int j = 0; j < WN; ++j) breg[j] = bnext[j];
-            }
-        }
-        __builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0): next slab's DMA (and B prefetch) complete
-        __syncthreads();
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = init;
     }
-    mfma_epilogue<T, WM, WN>(p, acc, sc, smem, lane, wave, wm, mb0, nb0);
+    const int aoff = (wm * WM) * CH + lane * 16;
+    int cur = 0, nxt = BUF, fre = 2 * BUF;         // byte offsets of the buffers of k-blocks s, s+1, s+2
+    v4i af[2][WM];
+#pragma unroll
+    for (int i = 0; i < WM; ++i) af[0][i] = *reinterpret_cast<const v4i*>(smem + cur + aoff + i * CH);
+
+    for (int kb = 0; kb < KB; ++kb) {
+        load_b(kb + 2, bnext2);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            if (ks == 2) {
+                // DMA of k-block kb+1 (issued one k-block ago) is older than this iteration's B loads
+                __builtin_amdgcn_s_waitcnt(0x0F70 | WN);          // vmcnt(WN)
+                __syncthreads();
+                dma_block(kb + 2, fre);
+            }
+            // next step's A fragments: same k-block, or the first step of the next one
+            const unsigned char* nsrc = ks < 3 ? smem + cur + aoff + (ks + 1) * 1024 : smem + nxt + aoff;
+#pragma unroll
+            for (int i = 0; i < WM; ++i) af[(ks + 1) & 1][i] = *reinterpret_cast<const v4i*>(nsrc + i * CH);
+            __builtin_amdgcn_sched_barrier(0);                    // keep the prefetch ahead of this step's MFMAs
+            v4i bf[WN];
+            expand_b(breg, ks, bf);
+#pragma unroll
+            for (int i = 0; i < WM; ++i)
+#pragma unroll
+                for (int j = 0; j < WN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[ks & 1][i], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < WN; ++j) { breg[j] = bnext[j]; bnext[j] = bnext2[j]; }
+        const int t = cur; cur = nxt; nxt = fre; fre = t;
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);            // the trailing DMA must not land in the epilogue's staging area
+    __syncthreads();
+    if constexpr (FAST) mfma_epilogue_fast<T, WM, WN>(p, acc, sc, smem, lane, wave, wm, mb0, nb0);
+    else mfma_epilogue<T, WM, WN>(p, acc, sc, smem, lane, wave, wm, mb0, nb0);
 }
 
-template <typename T, int WGM, int WGN, int WM, int WN, int KSL>
-int launch_mfma_dma(MfmaArgs a, hipStream_t s) {
+template <typename T, int WGM, int WGN, int WM, int WN>
+int launch_mfma_dma3(MfmaArgs a, hipStream_t s) {
     constexpr int BM = WGM * WM * 32, BN = WGN * WN * 32;
     a.tiles_m = (int)mmf_ceil_div(a.M, BM);
     a.tiles_n = (int)mmf_ceil_div(a.N, BN);
-    size_t lds = 2u * (WGM * WM) * 4096u * KSL;
+    size_t lds = 3u * (WGM * WM) * 4096u;
     const size_t lds_epi = (size_t)(WGM * WGN) * 32u * (WN * 32u * sizeof(T) + 16u);
     if (lds_epi > lds) lds = lds_epi;
     const int per_vec = 16 / (int)sizeof(T);
     a.vec_store = (a.N % per_vec == 0) && (a.ldo % per_vec == 0) && ((reinterpret_cast<uintptr_t>(a.out) & 15u) == 0) &&
                   ((reinterpret_cast<uintptr_t>(a.addend) & 15u) == 0);
-    auto kern = bitlinear_mfma_dma_kernel<T, WGM, WGN, WM, WN, KSL>;
+    const bool fast = a.vec_store && !a.bias;
+    auto kern = fast ? bitlinear_mfma_dma3_kernel<T, WGM, WGN, WM, WN, true> : bitlinear_mfma_dma3_kernel<T, WGM, WGN, WM, WN, false>;
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)lds);
@@ -543,17 +624,14 @@ int launch_mfma(MfmaArgs a, hipStream_t s) {
 template <typename T>
 int dispatch_mfma(const MfmaArgs& a, int config, hipStream_t s) {
     // config < 0: pick by shape.
-    //   5 / 6   decode-sized weight-stream kernel, M <= 32 / M <= 64 (needs Kp <= 8192)
-    //   0 - 4   tiled, A staged through registers: 32x256, 64x256, 128x256, 256x256, 256x256 (2x4 accs per wave)
-    //   10 - 14 tiled, A staged by DMA: 256x256 (slab 256), 128x512 (slab 512), 128x256 (slab 512),
-    //           128x512 (slab 256), 256x256 (slab 128)
+    //   5 / 6    decode-sized weight-stream kernel, M <= 32 / M <= 64 (needs Kp <= 8192)
+    //   0 / 1    32x256 / 64x256 tiles, A staged through registers (M <= 64 with Kp > 8192)
+    //   15 / 16  256x256 / 128x256 tiles, A staged by DMA
     if (config < 0) {
-        const int64_t tiles256 = mmf_ceil_div(a.M, 256) * mmf_ceil_div(a.N, 256);
         if (a.M <= 64 && a.Kp <= 8192) config = a.M <= 32 ? 5 : 6;
         else if (a.M <= 32) config = 0;
         else if (a.M <= 64) config = 1;
-        else if (a.M <= 128 || tiles256 < 512) config = 12;     // few tiles: smaller ones fill the 256 CUs better
-        else config = 14;
+        else config = 16;                                       // measured best from M = 128 to 16384
     }
     if ((config == 5 && a.M > 32) || (config == 6 && a.M > 64) || ((config == 5 || config == 6) && a.Kp > 8192))
         return MMF_ERR_ARG;
@@ -562,14 +640,8 @@ int dispatch_mfma(const MfmaArgs& a, int config, hipStream_t s) {
         case 6: return launch_skinny<T, 2>(a, s);
         case 0: return launch_mfma<T, 1, 8, 1, 1>(a, s);
         case 1: return launch_mfma<T, 1, 8, 2, 1>(a, s);
-        case 2: return launch_mfma<T, 2, 4, 2, 2>(a, s);
-        case 3: return launch_mfma<T, 2, 4, 4, 2>(a, s);
-        case 4: return launch_mfma<T, 4, 2, 2, 4>(a, s);
-        case 10: return launch_mfma_dma<T, 2, 4, 4, 2, 2>(a, s);
-        case 11: return launch_mfma_dma<T, 1, 8, 4, 2, 4>(a, s);
-        case 12: return launch_mfma_dma<T, 2, 4, 2, 2, 4>(a, s);
-        case 13: return launch_mfma_dma<T, 1, 8, 4, 2, 2>(a, s);
-        case 14: return launch_mfma_dma<T, 2, 4, 4, 2, 1>(a, s);
+        case 15: return launch_mfma_dma3<T, 2, 4, 4, 2>(a, s);
+        case 16: return launch_mfma_dma3<T, 2, 4, 2, 2>(a, s);
     }
     return MMF_ERR_ARG;
 }
