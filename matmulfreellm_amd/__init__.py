@@ -26,7 +26,8 @@ __version__ = "0.1"
 
 _LAZY = {"HGRNBitAttention": ".attention", "HGRNBitConfig": ".configuration_hgrn_bit",
          "HGRNBitModel": ".modeling_hgrn_bit", "HGRNBitForCausalLM": ".modeling_hgrn_bit",
-         "HGRNBitBlock": ".modeling_hgrn_bit", "HGRNBitMLP": ".modeling_hgrn_bit", "DecodeEngine": ".decode"}
+         "HGRNBitBlock": ".modeling_hgrn_bit", "HGRNBitMLP": ".modeling_hgrn_bit", "DecodeEngine": ".decode",
+         "save_packed": ".checkpoint", "load_packed": ".checkpoint", "load_pretrained": ".checkpoint", "pack_all": ".checkpoint"}
 
 __all__ = ["swiglu", "BitLinear", "FusedBitLinear", "activation_quant", "weight_quant", "layer_norm_linear_quant_fn",
            "RecurrentCache", "FusedRMSNormSwishGate", "chunk_hgrn", "fused_recurrent_hgrn", "RMSNorm", "rms_norm_fn",

@@ -123,8 +123,8 @@ class HGRNBitAttention(nn.Module):
 
     def init_state(self, batch_size: int) -> Tuple[torch.Tensor]:
         """Zero recurrent state [B, num_heads, head_dim], kept in fp32."""
-        param = next(self.parameters())
-        return (torch.zeros(batch_size, self.num_heads, self.head_dim, dtype=torch.float32, device=param.device),)
+        device = self.g_norm.weight.device       # the projections' latent weights may be absent (packed checkpoints)
+        return (torch.zeros(batch_size, self.num_heads, self.head_dim, dtype=torch.float32, device=device),)
 
     def state_size(self, **kwargs) -> int:
         return self.hidden_size

@@ -27,9 +27,17 @@ class _PackCache:
     """Packed codes of one weight tensor, invalidated when the tensor is written or replaced."""
 
     def __init__(self):
-        self.key, self.pw = None, None
+        self.key, self.pw, self.frozen = None, None, False
+
+    def freeze(self, pw):
+        """Pin codes loaded from a packed checkpoint: there is no latent weight to re-pack from."""
+        self.key, self.pw, self.frozen = None, pw, True
 
     def get(self, weight):
+        if self.frozen:
+            if not weight.is_meta:
+                raise RuntimeError("this BitLinear holds packed codes only; assigning a latent weight to it is not supported")
+            return self.pw
         key = (weight.data_ptr(), weight._version, weight.dtype, weight.device, tuple(weight.shape))
         if key != self.key:
             self.pw = F_.ternarize_pack(weight)

@@ -146,3 +146,44 @@ def test_weight_update_repacks(dev, tiny_bf16):
         lin.weight.mul_(-1.0)
     y1 = lin(x)
     assert torch.equal(y1, -y0)
+
+
+def test_packed_checkpoint_round_trip(dev, tmp_path):
+    """save_packed -> load_packed: no latent weights in memory, same logits and greedy tokens bit for bit,
+    and the file holds 2 bits per BitLinear weight."""
+    import os
+    import matmulfreellm_amd as mm
+    from matmulfreellm_amd import checkpoint as ck
+    cfg = mm.HGRNBitConfig(vocab_size=96, hidden_size=128, num_hidden_layers=2)
+    torch.manual_seed(3)
+    model = mm.HGRNBitForCausalLM(cfg).to(torch.bfloat16).to(dev).eval()
+    with torch.no_grad():
+        model.model.lower_bounds.normal_()
+    ids = torch.randint(0, 96, (2, 9), device=dev)
+    ref_logits = model(input_ids=ids).logits
+    ref_tokens = model.generate(ids, max_new_tokens=6)
+    path = ck.save_packed(model, tmp_path)
+    packed = ck.load_packed(tmp_path, device=dev)
+    bl = [m for m in packed.modules() if isinstance(m, mm.BitLinear)]
+    assert bl and all(m.weight.is_meta for m in bl)
+    assert not any(p.is_meta for n, p in packed.named_parameters() if not n.endswith("_proj.weight") and n != "lm_head.weight")
+    assert torch.equal(packed(input_ids=ids).logits, ref_logits)
+    assert torch.equal(packed.generate(ids, max_new_tokens=6), ref_tokens)
+    n_bit = sum(m.in_features * m.out_features for m in bl)
+    rest = sum(p.numel() * p.element_size() for n, p in model.named_parameters()
+               if not n.endswith("_proj.weight") and n != "lm_head.weight")
+    assert os.path.getsize(path) < n_bit // 4 + rest + 64 * 1024      # K = 128: no padding, 2 bits per weight
+
+
+def test_load_pretrained_packs_at_load(dev, tmp_path):
+    import matmulfreellm_amd as mm
+    from matmulfreellm_amd import checkpoint as ck
+    cfg = mm.HGRNBitConfig(vocab_size=64, hidden_size=64, num_hidden_layers=1)
+    torch.manual_seed(4)
+    m = mm.HGRNBitForCausalLM(cfg)
+    m.save_pretrained(tmp_path)
+    loaded = ck.load_pretrained(tmp_path, device=dev, dtype=torch.bfloat16)
+    assert all(b._pack.pw is not None for b in loaded.modules() if isinstance(b, mm.BitLinear))
+    ids = torch.randint(0, 64, (1, 5), device=dev)
+    want = m.to(torch.bfloat16).to(dev).eval()(input_ids=ids).logits
+    assert torch.equal(loaded(input_ids=ids).logits, want)

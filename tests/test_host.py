@@ -123,3 +123,34 @@ def test_division_free_quotient_is_the_correctly_rounded_one():
             q = fma(fma(-q, Kd, s), y, q)
             q = fma(fma(-q, Kd, s), y, q)
             assert q == s / Kd, (K, s)
+
+
+def test_reference_format_checkpoint_round_trip(tmp_path):
+    """save_pretrained / from_pretrained keep the reference's state-dict keys and values (no GPU needed:
+    nothing is packed until a BitLinear runs)."""
+    import matmulfreellm_amd as mm
+    cfg = mm.HGRNBitConfig(vocab_size=64, hidden_size=64, num_hidden_layers=2)
+    torch.manual_seed(0)
+    m = mm.HGRNBitForCausalLM(cfg)
+    m.save_pretrained(tmp_path)
+    m2 = mm.HGRNBitForCausalLM.from_pretrained(tmp_path)
+    a, b = m.state_dict(), m2.state_dict()
+    assert set(a) == set(b)
+    assert all(torch.equal(a[k], b[k]) for k in a)
+    for key in ("model.embeddings.weight", "model.lower_bounds", "model.layers.0.attn.i_proj.weight",
+                "model.layers.0.attn.i_proj.norm.weight", "model.layers.1.mlp.down_proj.norm.weight", "lm_head.weight"):
+        assert key in a
+
+
+def test_packed_checkpoint_loader_rejects_foreign_files(tmp_path):
+    import matmulfreellm_amd as mm
+    from matmulfreellm_amd import checkpoint as ck
+    from safetensors.torch import save_file
+    cfg = mm.HGRNBitConfig(vocab_size=64, hidden_size=64, num_hidden_layers=1)
+    cfg.save_pretrained(tmp_path)
+    save_file({"x": torch.zeros(1)}, str(tmp_path / ck.PACKED_FILE), metadata={"format": "something-else"})
+    with pytest.raises(ValueError):
+        ck.load_packed(tmp_path, device="cpu")
+    save_file({"x": torch.zeros(1)}, str(tmp_path / ck.PACKED_FILE), metadata={"format": ck.FORMAT})
+    with pytest.raises(KeyError):
+        ck.load_packed(tmp_path, device="cpu")
