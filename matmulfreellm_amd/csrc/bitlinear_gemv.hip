@@ -132,10 +132,17 @@ __device__ __forceinline__ void raw4_store(T* p, int k0, int K, const float (&f)
 
 // NV: passes over the row (Kp <= NV * 2048); a wave then owns at most 2 * NV of the row's 1 KiB
 // weight blocks per n-block.  VEC: K, the row strides and every pointer allow 4-element accesses.
-template <typename T, typename TW, int NV, int PRO, int EPI, bool VEC>
+// S: row split.  S = 1: a workgroup owns whole n-blocks (32 output rows; lane = (k-half, row)).
+// S = 4: it owns 8 of the 32 rows, so that a 2048-row projection fills 256 CUs instead of 64; a
+// lane is (k-block of a group of four, k-half, row of 8), a wave-load covers four k-blocks (two
+// 128-byte runs of each 1 KiB block), and the waves share out the (n-block, k-group) items.
+template <typename T, typename TW, int NV, int PRO, int EPI, bool VEC, int S>
 __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a) {
     constexpr int R = EPI == EPI_STEP ? 3 : EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int BPW = 2 * NV;
+    constexpr int GMAX = 4 * NV;                                // k-groups of four blocks (S = 4)
+    constexpr int ITEMS = (R * GMAX + kGemvWaves - 1) / kGemvWaves;   // (n-block, k-group) items per wave (S = 4)
+    constexpr int CHN = 32 / S;                                 // output channels per workgroup and n-block
     constexpr bool HAS_AUX = PRO >= PRO_RESNORM;
     constexpr bool HAS_W1 = PRO >= PRO_NORM && PRO <= PRO_GATEDNORM;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -144,10 +151,10 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
     __shared__ double red_a[kGemvWaves], red_b[kGemvWaves];
     __shared__ float red_f[kGemvWaves];
     __shared__ int red_q[kGemvWaves];
-    __shared__ int2 part[R][kGemvWaves][32];                    // .x / .y: the two k-halves of a wave's lanes
+    __shared__ int2 part[S == 1 ? R * kGemvWaves * 32 : R * GMAX * 8];   // S = 1: [r][wave][row], S = 4: [item][row8]; .x/.y: lane halves
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int nb = blockIdx.x, row = blockIdx.y;
+    const int nb = blockIdx.x / S, sub = blockIdx.x % S, row = blockIdx.y;
     const int K = a.K, Kp = a.Kp, KB = Kp >> 7;
     const int Nseg = a.N / R;
     const int NBseg = (Nseg + 31) >> 5;                         // n-blocks per stacked segment (R > 1)
@@ -168,17 +175,33 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
         if constexpr (HAS_W1) w1raw[v] = raw4_load<TW, VEC>(w1, k0, K);
         if (nw) nwraw[v] = raw4_load<TW, VEC>(nw, k0, K);
     }
-    uint4 wreg[R][BPW];
+    constexpr int NWREG = S == 1 ? R * BPW : ITEMS;
+    uint4 wreg[NWREG];
+    const int G = (KB + 3) >> 2;                                // k-groups in this row (S = 4)
+    const int kbi = lane >> 4, half = S == 1 ? lane >> 5 : (lane >> 3) & 1;
+    if constexpr (S == 1) {
 #pragma unroll
-    for (int r = 0; r < R; ++r)
+        for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int i = 0; i < BPW; ++i) {
-            const int kb = wave + i * kGemvWaves;
-            if (kb < KB) wreg[r][i] = a.packed[((int64_t)(nb + r * NBseg) * KB + kb) * 64 + lane];
+            for (int i = 0; i < BPW; ++i) {
+                const int kb = wave + i * kGemvWaves;
+                if (kb < KB) wreg[r * BPW + i] = a.packed[((int64_t)(nb + r * NBseg) * KB + kb) * 64 + lane];
+            }
+    } else {
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const int item = wave + i * kGemvWaves;             // wave-uniform
+            wreg[i] = make_uint4(0u, 0u, 0u, 0u);               // code 0 against any activation adds nothing
+            if (item < R * G) {
+                const int r = item / G, kb = (item % G) * 4 + kbi;
+                if (kb < KB)
+                    wreg[i] = a.packed[((int64_t)(nb + r * NBseg) * KB + kb) * 64 + half * 32 + sub * CHN + (lane & 7)];
+            }
         }
+    }
     float ep_wdeq[R], ep_bias = 0.0f, ep_add = 0.0f, ep_lb = 0.0f, ep_state = 0.0f;
-    const int ch = nb * 32 + (lane & 31);                       // output column / channel of the epilogue lanes
-    const bool ep_lane = wave == 0 && lane < 32 && ch < Nseg;
+    const int ch = nb * 32 + sub * CHN + (lane & (CHN - 1));    // output column / channel of the epilogue lanes
+    const bool ep_lane = wave == 0 && lane < CHN && ch < Nseg;
     if (wave == 0) {
         // the 32 outputs of an n-block share a scale (segments are multiples of 32 rows)
 #pragma unroll
@@ -291,32 +314,45 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
     if (lane == 0) red_q[wave] = qs;
     __syncthreads();                                            // publishes q_lds and red_q
 
-    // ---- main: sum_k q[k] * (t[n,k] + 1) for n = (nb + r*NBseg)*32 + lane%32 over this wave's blocks
-    const int half = lane >> 5;
-    int acc[R];
+    // ---- main: sum_k q[k] * (t[n,k] + 1) over this wave's blocks
+    auto dot_block = [&](const uint4& wq, int kb, int acc) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = 0;
+        for (int s4 = 0; s4 < 4; ++s4) {
+            const int4 qv = *reinterpret_cast<const int4*>(q_lds + kb * 128 + s4 * 32 + half * 16);
+            const uint32_t w = s4 == 0 ? wq.x : s4 == 1 ? wq.y : s4 == 2 ? wq.z : wq.w;
+            acc = __builtin_amdgcn_sdot4((int)(w & 0x03030303u), qv.x, acc, false);
+            acc = __builtin_amdgcn_sdot4((int)((w >> 2) & 0x03030303u), qv.y, acc, false);
+            acc = __builtin_amdgcn_sdot4((int)((w >> 4) & 0x03030303u), qv.z, acc, false);
+            acc = __builtin_amdgcn_sdot4((int)((w >> 6) & 0x03030303u), qv.w, acc, false);
+        }
+        return acc;
+    };
+    if constexpr (S == 1) {
+        int acc[R];
 #pragma unroll
-    for (int i = 0; i < BPW; ++i) {
-        const int kb = wave + i * kGemvWaves;
-        if (kb < KB) {
+        for (int r = 0; r < R; ++r) acc[r] = 0;
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const int4 qv = *reinterpret_cast<const int4*>(q_lds + kb * 128 + s * 32 + half * 16);
+        for (int i = 0; i < BPW; ++i) {
+            const int kb = wave + i * kGemvWaves;
+            if (kb < KB) {
 #pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    const uint32_t w = s == 0 ? wreg[r][i].x : s == 1 ? wreg[r][i].y : s == 2 ? wreg[r][i].z : wreg[r][i].w;
-                    acc[r] = __builtin_amdgcn_sdot4((int)(w & 0x03030303u), qv.x, acc[r], false);
-                    acc[r] = __builtin_amdgcn_sdot4((int)((w >> 2) & 0x03030303u), qv.y, acc[r], false);
-                    acc[r] = __builtin_amdgcn_sdot4((int)((w >> 4) & 0x03030303u), qv.z, acc[r], false);
-                    acc[r] = __builtin_amdgcn_sdot4((int)((w >> 6) & 0x03030303u), qv.w, acc[r], false);
-                }
+                for (int r = 0; r < R; ++r) acc[r] = dot_block(wreg[r * BPW + i], kb, acc[r]);
             }
         }
-    }
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        reinterpret_cast<int*>(&part[r][wave][lane & 31])[half] = acc[r];
+        for (int r = 0; r < R; ++r) reinterpret_cast<int*>(&part[(r * kGemvWaves + wave) * 32 + (lane & 31)])[half] = acc[r];
+    } else {
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const int item = wave + i * kGemvWaves;
+            if (item < R * G) {
+                const int kb = (item % G) * 4 + kbi;
+                int acc = dot_block(wreg[i], kb < KB ? kb : 0, 0);   // blocks past the end carry zero codes
+                acc += mmf_dpp<0x128>(acc);                      // row_ror:8 -> the other k-half
+                acc += __builtin_amdgcn_ds_swizzle(acc, 0x401F);   // xor 16 -> the neighbouring k-block
+                if ((lane & 31) < 8) reinterpret_cast<int*>(&part[item * 8 + (lane & 7)])[lane >> 5] = acc;
+            }
+        }
     }
     __syncthreads();
     if (ep_lane) {
@@ -328,10 +364,17 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             int tot = 0;
+            if constexpr (S == 1) {
 #pragma unroll
-            for (int w = 0; w < kGemvWaves; ++w) {
-                const int2 pr = part[r][w][lane];
-                tot += pr.x + pr.y;
+                for (int w = 0; w < kGemvWaves; ++w) {
+                    const int2 pr = part[(r * kGemvWaves + w) * 32 + lane];
+                    tot += pr.x + pr.y;
+                }
+            } else {
+                for (int gi = 0; gi < G; ++gi) {
+                    const int2 pr = part[(r * G + gi) * 8 + lane];
+                    tot += pr.x + pr.y;
+                }
             }
             res[r] = __fmul_rn(__fmul_rn((float)(tot - qtot), deq), ep_wdeq[r]);
         }
@@ -363,13 +406,21 @@ template <typename T, typename TW, int PRO, int EPI>
 int launch_gemv(const GemvArgs& a, int64_t M, bool vec, hipStream_t s) {
     constexpr int R = EPI == EPI_STEP ? 3 : EPI == EPI_SWIGLU ? 2 : 1;
     const int nv = (int)mmf_ceil_div((int64_t)a.Kp, (int64_t)kGemvThreads * kGemvEl);
-    dim3 grid((unsigned)mmf_ceil_div(a.N / R, 32), (unsigned)M), block(kGemvThreads);
+    const int64_t nblocks = mmf_ceil_div(a.N / R, 32);
+    // few n-blocks (a 2048-row projection has 64): give each workgroup 8 rows, not 32, to reach every CU
+    const bool split = vec && nblocks * M <= 96;
+    dim3 grid((unsigned)(nblocks * (split ? 4 : 1)), (unsigned)M), block(kGemvThreads);
     const size_t lds = (size_t)a.Kp;
-    if (!vec) bitlinear_gemv_kernel<T, TW, kGemvMaxNV, PRO, EPI, false><<<grid, block, lds, s>>>(a);   // ragged shapes: one generic build
-    else if (nv <= 1) bitlinear_gemv_kernel<T, TW, 1, PRO, EPI, true><<<grid, block, lds, s>>>(a);
-    else if (nv <= 2) bitlinear_gemv_kernel<T, TW, 2, PRO, EPI, true><<<grid, block, lds, s>>>(a);
-    else if (nv <= 3) bitlinear_gemv_kernel<T, TW, 3, PRO, EPI, true><<<grid, block, lds, s>>>(a);
-    else bitlinear_gemv_kernel<T, TW, 4, PRO, EPI, true><<<grid, block, lds, s>>>(a);
+    if (!vec) bitlinear_gemv_kernel<T, TW, kGemvMaxNV, PRO, EPI, false, 1><<<grid, block, lds, s>>>(a);   // ragged shapes: one generic build
+    else if (split) {
+        if (nv <= 1) bitlinear_gemv_kernel<T, TW, 1, PRO, EPI, true, 4><<<grid, block, lds, s>>>(a);
+        else if (nv <= 2) bitlinear_gemv_kernel<T, TW, 2, PRO, EPI, true, 4><<<grid, block, lds, s>>>(a);
+        else if (nv <= 3) bitlinear_gemv_kernel<T, TW, 3, PRO, EPI, true, 4><<<grid, block, lds, s>>>(a);
+        else bitlinear_gemv_kernel<T, TW, 4, PRO, EPI, true, 4><<<grid, block, lds, s>>>(a);
+    } else if (nv <= 1) bitlinear_gemv_kernel<T, TW, 1, PRO, EPI, true, 1><<<grid, block, lds, s>>>(a);
+    else if (nv <= 2) bitlinear_gemv_kernel<T, TW, 2, PRO, EPI, true, 1><<<grid, block, lds, s>>>(a);
+    else if (nv <= 3) bitlinear_gemv_kernel<T, TW, 3, PRO, EPI, true, 1><<<grid, block, lds, s>>>(a);
+    else bitlinear_gemv_kernel<T, TW, 4, PRO, EPI, true, 1><<<grid, block, lds, s>>>(a);
     MMF_CHECK_LAUNCH();
     return 0;
 }

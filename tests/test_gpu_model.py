@@ -187,3 +187,31 @@ def test_load_pretrained_packs_at_load(dev, tmp_path):
     ids = torch.randint(0, 64, (1, 5), device=dev)
     want = m.to(torch.bfloat16).to(dev).eval()(input_ids=ids).logits
     assert torch.equal(loaded(input_ids=ids).logits, want)
+
+
+@pytest.mark.parametrize("batch", [1, 4])
+def test_fused_decode_matches_per_op_decode_at_width_1024(dev, batch):
+    """At hidden size 1024 the fused GEMV runs with 8 rows per workgroup at batch 1 and with whole
+    32-row blocks at batch 4; both must reproduce the per-op engine (itself pinned to the oracle at
+    small widths) bit for bit, logits and recurrent state."""
+    import matmulfreellm_amd as mm
+    from matmulfreellm_amd.decode import DecodeEngine
+    cfg = mm.HGRNBitConfig(vocab_size=4096, hidden_size=1024, num_hidden_layers=2)
+    torch.manual_seed(5)
+    model = mm.HGRNBitForCausalLM(cfg).to(torch.bfloat16).to(dev).eval()
+    with torch.no_grad():
+        model.model.lower_bounds.normal_()
+    ids = torch.randint(0, 4096, (batch, 16), device=dev)
+    out = model(input_ids=ids, use_cache=True, logits_to_keep=1)
+    states = [c[-1].clone() for c in out.past_key_values]
+    toks = torch.randint(0, 4096, (5, batch), device=dev)
+    results = []
+    for fuse in (True, False):
+        eng = DecodeEngine.for_model(model, batch, use_graph=False, fuse=fuse)
+        eng.load_state(states)
+        logits = [eng.step(toks[t]).clone() for t in range(5)]
+        results.append((logits, [e["state"].clone() for e in eng.layers]))
+    for a, b in zip(results[0][0], results[1][0]):
+        assert torch.equal(a, b)
+    for a, b in zip(results[0][1], results[1][1]):
+        assert torch.equal(a, b)

@@ -188,7 +188,8 @@ def _bitlinear_case(dev, dtype, m, k, n, path, bias=False, seed=7):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("mkn", [(1, 2048, 2048), (1, 512, 3072), (3, 5632, 2048), (1, 300, 70), (2, 6912, 2560)])
+@pytest.mark.parametrize("mkn", [(1, 2048, 2048), (1, 512, 3072), (3, 5632, 2048), (1, 300, 70), (2, 6912, 2560),
+                                 (1, 5632, 2048), (1, 1024, 3200), (1, 8192, 96), (2, 384, 1504)])
 def test_bitlinear_gemv(dev, dtype, mkn):
     _bitlinear_case(dev, dtype, *mkn, path="gemv")
 
