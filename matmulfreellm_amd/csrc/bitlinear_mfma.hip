@@ -489,9 +489,10 @@ int launch_mfma_dma3(MfmaArgs a, hipStream_t s) {
 }
 
 // ------------------------------------------------------------------------------------------
-// Decode-sized M (<= 64): the contraction is a weight stream, not a GEMM, and the enemy is
-// latency, so nothing is staged and nothing waits on a barrier until the very end.
-// One workgroup of 8 waves owns one 32-row n-block; wave w takes the k-blocks w, w+8, ...
+// Small problems (decode batches, short prompts): the contraction is a weight stream, not a
+// GEMM, and the enemy is latency, so nothing is staged and nothing waits on a barrier until the
+// very end.  One workgroup of 8 waves owns MB 32x32 output blocks of one 32-row n-block (grid.y
+// walks M); wave w takes the k-blocks w, w+8, ...
 // A fragments (1 KiB each, L2 resident: the whole A is M x K bytes) and the packed B block
 // are loaded straight into registers, three k-blocks in flight per wave; the 8 partial
 // accumulators meet in LDS and all 512 threads run the epilogue.
@@ -500,7 +501,7 @@ __global__ __launch_bounds__(512) void bitlinear_mfma_skinny_kernel(MfmaArgs p) 
     constexpr int NWV = 8, PF = 3, MAXK = 8;            // Kp <= 8 * 8 * 128
     __shared__ int red[NWV][MB][16][64];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave-uniform: keep it in a scalar register
-    const int64_t nb = blockIdx.x;
+    const int64_t nb = blockIdx.x, mbase = (int64_t)blockIdx.y * MB;   // this workgroup's first m-block
     const int64_t KB = p.Kp >> 7, KG = p.Kp >> 4;
     const int64_t MBtot = (p.M + 31) >> 5;
 
@@ -520,8 +521,8 @@ __global__ __launch_bounds__(512) void bitlinear_mfma_skinny_kernel(MfmaArgs p) 
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks) {
                     areg[st][i][ks] = (v4i){0, 0, 0, 0};
-                    if (i < MBtot)
-                        areg[st][i][ks] = *reinterpret_cast<const v4i*>(p.a + ((int64_t)i * KG + kb * 8 + ks * 2) * 512 + lane * 16);
+                    if (mbase + i < MBtot)
+                        areg[st][i][ks] = *reinterpret_cast<const v4i*>(p.a + ((mbase + i) * KG + kb * 8 + ks * 2) * 512 + lane * 16);
                 }
         }
     };
@@ -542,7 +543,7 @@ __global__ __launch_bounds__(512) void bitlinear_mfma_skinny_kernel(MfmaArgs p) 
     for (int j = 0; j < MB * 2; ++j) {
         const int e = threadIdx.x + j * 512;             // (mb, r, lane) flattened
         const int r = (e >> 6) & 15, mb = e >> 10;
-        const int64_t m = (int64_t)mb * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        const int64_t m = (mbase + mb) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         const int64_t mc = m < p.M ? m : 0;
         ep_qsum[j] = p.qsum[mc];
         ep_deq[j] = p.deq[mc];
@@ -582,7 +583,7 @@ __global__ __launch_bounds__(512) void bitlinear_mfma_skinny_kernel(MfmaArgs p) 
         int tot = 0;
 #pragma unroll
         for (int w = 0; w < NWV; ++w) tot += red[w][mb][r][lane];
-        const int64_t m = (int64_t)mb * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        const int64_t m = (mbase + mb) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         if (m < p.M && n_ok) {
             float o = __fmul_rn(__fmul_rn((float)(tot - ep_qsum[j]), ep_deq[j]), ep_wdeq);
             if (bias) o = __fadd_rn(o, ep_bias);
@@ -594,7 +595,7 @@ __global__ __launch_bounds__(512) void bitlinear_mfma_skinny_kernel(MfmaArgs p) 
 
 template <typename T, int MB>
 int launch_skinny(const MfmaArgs& a, hipStream_t s) {
-    bitlinear_mfma_skinny_kernel<T, MB><<<dim3((unsigned)mmf_ceil_div(a.N, 32)), dim3(512), 0, s>>>(a);
+    bitlinear_mfma_skinny_kernel<T, MB><<<dim3((unsigned)mmf_ceil_div(a.N, 32), (unsigned)mmf_ceil_div(a.M, 32 * MB)), dim3(512), 0, s>>>(a);
     MMF_CHECK_LAUNCH();
     return 0;
 }
@@ -624,20 +625,25 @@ int launch_mfma(MfmaArgs a, hipStream_t s) {
 template <typename T>
 int dispatch_mfma(const MfmaArgs& a, int config, hipStream_t s) {
     // config < 0: pick by shape.
-    //   5 / 6    decode-sized weight-stream kernel, M <= 32 / M <= 64 (needs Kp <= 8192)
-    //   0 / 1    32x256 / 64x256 tiles, A staged through registers (M <= 64 with Kp > 8192)
+    //   5        weight-stream kernel: one 32x32 output block per workgroup, 8 waves split K (needs Kp <= 8192)
+    //   0 / 1    32x256 / 64x256 tiles, A staged through registers (small M with Kp > 8192)
     //   15 / 16  256x256 / 128x256 tiles, A staged by DMA
     if (config < 0) {
-        if (a.M <= 64 && a.Kp <= 8192) config = a.M <= 32 ? 5 : 6;
+        const int64_t KB = a.Kp >> 7;
+        const double wgs = (double)mmf_ceil_div(a.M, 32) * (double)mmf_ceil_div(a.N, 32);
+        const double tiles = (double)mmf_ceil_div(a.M, 128) * (double)mmf_ceil_div(a.N, 256);
+        // measured on MI355X: the stream kernel costs ~3 us + 0.33 ns per (output block x k-block); a round of
+        // tiles of the DMA kernel ~0.9 us per k-block whatever the problem size
+        const double t_stream = 3.0 + wgs * (double)KB * 0.00033;
+        const double t_tiled = (double)KB * 0.9 * (double)mmf_ceil_div((int64_t)tiles, 256);
+        if (a.Kp <= 8192 && (a.M <= 64 || t_stream < t_tiled)) config = 5;
         else if (a.M <= 32) config = 0;
         else if (a.M <= 64) config = 1;
-        else config = 16;                                       // measured best from M = 128 to 16384
+        else config = 16;
     }
-    if ((config == 5 && a.M > 32) || (config == 6 && a.M > 64) || ((config == 5 || config == 6) && a.Kp > 8192))
-        return MMF_ERR_ARG;
+    if (config == 5 && (a.Kp > 8192 || a.M > 65535 * 32)) return MMF_ERR_ARG;
     switch (config) {
         case 5: return launch_skinny<T, 1>(a, s);
-        case 6: return launch_skinny<T, 2>(a, s);
         case 0: return launch_mfma<T, 1, 8, 1, 1>(a, s);
         case 1: return launch_mfma<T, 1, 8, 2, 1>(a, s);
         case 15: return launch_mfma_dma3<T, 2, 4, 4, 2>(a, s);

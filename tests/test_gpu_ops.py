@@ -207,13 +207,13 @@ def test_bitlinear_bias_and_known_answers(dev):
 
 
 @pytest.mark.parametrize("config,m,k,n", [(0, 300, 1024, 640), (1, 300, 1024, 640), (0, 20, 2048, 512), (1, 64, 2048, 512),
-                                          (5, 32, 2048, 640), (5, 7, 5632, 2048), (5, 1, 300, 70), (6, 64, 2048, 6144),
-                                          (6, 40, 5632, 2048), (6, 64, 8192, 96), (6, 33, 6912, 2560),
+                                          (5, 32, 2048, 640), (5, 7, 5632, 2048), (5, 1, 300, 70), (5, 64, 2048, 6144),
+                                          (5, 40, 5632, 2048), (5, 64, 8192, 96), (5, 33, 6912, 2560), (5, 300, 1024, 648),
                                           (15, 520, 2048, 1032), (15, 300, 128, 640), (15, 300, 256, 648), (16, 300, 1152, 640),
                                           (15, 4096, 2048, 1024), (16, 70, 384, 100), (15, 300, 1024, 644), (16, 300, 1024, 648),
                                           (16, 200, 128, 520), (-1, 4096, 512, 2048), (-1, 100, 512, 256), (-1, 40, 8320, 96)])
 def test_bitlinear_mfma_all_tile_configs(dev, config, m, k, n):
-    """Every tile shape of the matrix-core contraction (0/1 register-staged, 5/6 the decode-sized stream kernel,
+    """Every tile shape of the matrix-core contraction (0/1 register-staged, 5 the weight-stream kernel,
     15/16 DMA-staged; ragged M, K, N; one and two k-blocks)."""
     torch.manual_seed(8)
     x = torch.randn(m, k).bfloat16()
