@@ -86,50 +86,6 @@ __device__ __forceinline__ float block_max_once(float v, float* slot) {
     return s;
 }
 
-// Four consecutive elements as they sit in memory; unpacked to fp32 only where they are used, so
-// that all of a thread's loads are in flight before the first conversion waits for one.
-template <typename T> struct Raw4 { uint2 v; };
-template <> struct Raw4<float> { float4 v; };
-
-template <typename T, bool VEC>
-__device__ __forceinline__ Raw4<T> raw4_load(const T* p, int k0, int K) {
-    Raw4<T> r;
-    if constexpr (VEC) {
-        const int kk = k0 < K ? k0 : 0;                         // lanes past K re-read the row start; zeroed on unpack
-        r.v = *reinterpret_cast<const decltype(r.v)*>(p + kk);
-    } else {
-        T e[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) e[i] = p[k0 + i < K ? k0 + i : 0];
-        __builtin_memcpy(&r.v, e, sizeof(r.v));
-    }
-    return r;
-}
-template <typename T>
-__device__ __forceinline__ void raw4_unpack(const Raw4<T>& r, float (&f)[4]) {
-    if constexpr (sizeof(T) == 4) {
-        f[0] = r.v.x; f[1] = r.v.y; f[2] = r.v.z; f[3] = r.v.w;
-    } else {
-        T e[4];
-        __builtin_memcpy(e, &r.v, sizeof(r.v));
-#pragma unroll
-        for (int i = 0; i < 4; ++i) f[i] = mmf_to_float(e[i]);
-    }
-}
-template <typename T, bool VEC>
-__device__ __forceinline__ void raw4_store(T* p, int k0, int K, const float (&f)[4]) {
-    T e[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) e[i] = mmf_from_float<T>(f[i]);
-    if constexpr (VEC) {
-        if (k0 < K) __builtin_memcpy(p + k0, e, sizeof(e));
-    } else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (k0 + i < K) p[k0 + i] = e[i];
-    }
-}
-
 // NV: passes over the row (Kp <= NV * 2048); a wave then owns at most 2 * NV of the row's 1 KiB
 // weight blocks per n-block.  VEC: K, the row strides and every pointer allow 4-element accesses.
 // S: row split.  S = 1: a workgroup owns whole n-blocks (32 output rows; lane = (k-half, row)).

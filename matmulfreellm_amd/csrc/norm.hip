@@ -205,123 +205,119 @@ struct FusedQuantArgs {
     float eps1, eps;
 };
 
-template <typename T, typename TW, int NV, int PRO>
-__global__ __launch_bounds__(kThreads) void row_quant_fused_kernel(FusedQuantArgs a) {
-    __shared__ double red_a[kWaves], red_b[kWaves];
-    __shared__ float red_f[kWaves];
-    __shared__ int red_i[kWaves];
-    const int64_t row = blockIdx.x, K = a.K, Kp = a.Kp;
-    const bool vec_ok = (K % 8) == 0 && (a.ldx % 8) == 0 && (a.ldaux % 8) == 0 && (a.ldaux2 % 8) == 0;
+constexpr int kQWaves = 8, kQThreads = kQWaves * 64;            // a row of 2048 = 4 elements per thread
+
+// NV passes of 2048 elements.  VEC: K, the strides and every pointer allow 4-element accesses.
+template <typename T, typename TW, int NV, int PRO, bool VEC>
+__global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantArgs a) {
+    __shared__ double red_a[kQWaves], red_b[kQWaves];
+    __shared__ float red_f[kQWaves];
+    __shared__ int red_i[kQWaves];
+    constexpr bool HAS_AUX = PRO >= QPRO_RESNORM, STEP = PRO == QPRO_STEP_GATE, HAS_W1 = PRO != QPRO_SWIGLU;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t row = blockIdx.x;
+    const int K = (int)a.K, Kp = (int)a.Kp;
     const T* x = static_cast<const T*>(a.x) + row * a.ldx;
     const T* aux = static_cast<const T*>(a.aux) + row * a.ldaux;
     const T* aux2 = static_cast<const T*>(a.aux2) + row * a.ldaux2;
     const TW* w1 = static_cast<const TW*>(a.w1);
     const TW* nw = static_cast<const TW*>(a.norm_w);
+    float* st = a.state + row * K;
 
-    constexpr bool HAS_AUX = PRO >= QPRO_RESNORM, STEP = PRO == QPRO_STEP_GATE, HAS_W1 = PRO != QPRO_SWIGLU;
-    const bool vec_w = (K % 8) == 0;
     // every load of the kernel first, raw; conversions only after the last one is issued
-    Raw8<T> xraw[NV], araw[HAS_AUX ? NV : 1], graw[STEP ? NV : 1];
-    Raw8<float> straw[STEP ? NV : 1], lbraw[STEP ? NV : 1];
-    Raw8<TW> w1raw[HAS_W1 ? NV : 1], nwraw[NV];
+    Raw4<T> xraw[NV], araw[HAS_AUX ? NV : 1], graw[STEP ? NV : 1];
+    Raw4<float> straw[STEP ? NV : 1], lbraw[STEP ? NV : 1];
+    Raw4<TW> w1raw[HAS_W1 ? NV : 1], nwraw[NV];
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
-        xraw[v] = mmf_load8_raw<T>(x, k0, K, vec_ok);
-        if constexpr (HAS_AUX) araw[v] = mmf_load8_raw<T>(aux, k0, K, vec_ok);
+        const int k0 = (v * kQThreads + (int)threadIdx.x) * 4;
+        xraw[v] = raw4_load<T, VEC>(x, k0, K);
+        if constexpr (HAS_AUX) araw[v] = raw4_load<T, VEC>(aux, k0, K);
         if constexpr (STEP) {
-            graw[v] = mmf_load8_raw<T>(aux2, k0, K, vec_ok);
-            straw[v] = mmf_load8_raw<float>(a.state + row * K, k0, K, vec_w);
-            if (a.lb) lbraw[v] = mmf_load8_raw<float>(a.lb, k0, K, vec_w);
+            graw[v] = raw4_load<T, VEC>(aux2, k0, K);
+            straw[v] = raw4_load<float, VEC>(st, k0, K);
+            if (a.lb) lbraw[v] = raw4_load<float, VEC>(a.lb, k0, K);
         }
-        if constexpr (HAS_W1) w1raw[v] = mmf_load8_raw<TW>(w1, k0, K, vec_w);
-        if (nw) nwraw[v] = mmf_load8_raw<TW>(nw, k0, K, vec_w);
+        if constexpr (HAS_W1) w1raw[v] = raw4_load<TW, VEC>(w1, k0, K);
+        if (nw) nwraw[v] = raw4_load<TW, VEC>(nw, k0, K);
     }
-    float xv[NV][8], av[HAS_AUX ? NV : 1][8], gv[STEP ? NV : 1][8];
-    float w1v[HAS_W1 ? NV : 1][8], wv[NV][8], lbv[STEP ? NV : 1][8], stv[STEP ? NV : 1][8];
+    float xv[NV][4], av[HAS_AUX ? NV : 1][4];
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
-        mmf_unpack8<T>(xraw[v], xv[v]);
-        if constexpr (HAS_AUX) mmf_unpack8<T>(araw[v], av[v]);
-        if constexpr (STEP) {
-            mmf_unpack8<T>(graw[v], gv[v]);
-            mmf_unpack8<float>(straw[v], stv[v]);
-            if (a.lb) mmf_unpack8<float>(lbraw[v], lbv[v]);
-        }
-        if constexpr (HAS_W1) mmf_unpack8<TW>(w1raw[v], w1v[v]);
-        if (nw) mmf_unpack8<TW>(nwraw[v], wv[v]);
+        const int k0 = (v * kQThreads + (int)threadIdx.x) * 4;
+        raw4_unpack<T>(xraw[v], xv[v]);
+        if constexpr (HAS_AUX) raw4_unpack<T>(araw[v], av[v]);
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+        for (int i = 0; i < 4; ++i)
             if (k0 + i >= K) xv[v][i] = 0.0f;
     }
     if constexpr (PRO == QPRO_RESNORM) {
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
-            const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
-            if (k0 < K) {
+            const int k0 = (v * kQThreads + (int)threadIdx.x) * 4;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) xv[v][i] = __fadd_rn(xv[v][i], av[v][i]);
-                if (a.res_out) mmf_store8<T>(static_cast<T*>(a.res_out) + row * K, k0, K, (K % 8) == 0, xv[v]);
-            }
+            for (int i = 0; i < 4; ++i) xv[v][i] = k0 + i < K ? __fadd_rn(xv[v][i], av[v][i]) : 0.0f;
+            if (a.res_out) raw4_store<T, VEC>(static_cast<T*>(a.res_out) + row * K, k0, K, xv[v]);
         }
     }
-    if constexpr (PRO == QPRO_STEP_GATE) {
+    if constexpr (STEP) {
         // gate math + one recurrence step per channel; xv becomes the raw g projection, av the new o
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
-            const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
-            if (k0 < K) {
+            const int k0 = (v * kQThreads + (int)threadIdx.x) * 4;
+            float gv[4], stv[4], lbv[4];
+            raw4_unpack<T>(graw[v], gv);
+            raw4_unpack<float>(straw[v], stv);
+            if (a.lb) raw4_unpack<float>(lbraw[v], lbv);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const float iv = xv[v][i], fv = av[v][i];
-                    float s = mmf_sigmoid(fv);
-                    if (a.lb) s = __fadd_rn(lbv[v][i], __fmul_rn(__fsub_rn(1.0f, lbv[v][i]), s));
-                    const float go = mmf_round_to<T>(s);
-                    const float xo = mmf_round_to<T>(__fdiv_rn(__fmul_rn(iv, __fsub_rn(1.0f, go)), __fadd_rn(1.0f, mmf_exp(-iv))));
-                    const float h = __fadd_rn(__fmul_rn(go, stv[v][i]), xo);
-                    stv[v][i] = h;
-                    av[v][i] = mmf_round_to<T>(h);      // o, the swish gate of the gated norm
-                    xv[v][i] = gv[v][i];                // the gated norm normalises the g projection
-                }
-                mmf_store8<float>(a.state + row * K, k0, K, (K % 8) == 0, stv[v]);
+            for (int i = 0; i < 4; ++i) {
+                const float iv = xv[v][i], fv = av[v][i];
+                float s = mmf_sigmoid(fv);
+                if (a.lb) s = __fadd_rn(lbv[i], __fmul_rn(__fsub_rn(1.0f, lbv[i]), s));
+                const float go = mmf_round_to<T>(s);
+                const float xo = mmf_round_to<T>(__fdiv_rn(__fmul_rn(iv, __fsub_rn(1.0f, go)), __fadd_rn(1.0f, mmf_exp(-iv))));
+                const float h = __fadd_rn(__fmul_rn(go, stv[i]), xo);
+                stv[i] = h;
+                av[v][i] = mmf_round_to<T>(h);          // o, the swish gate of the gated norm
+                xv[v][i] = k0 + i < K ? gv[i] : 0.0f;   // the gated norm normalises the g projection
             }
+            raw4_store<float, VEC>(st, k0, K, stv);
         }
     }
-    if constexpr (PRO != QPRO_SWIGLU) {
+    if constexpr (HAS_W1) {
         double s1 = 0.0;
 #pragma unroll
         for (int v = 0; v < NV; ++v)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) s1 += (double)xv[v][i] * (double)xv[v][i];
+            for (int i = 0; i < 4; ++i) s1 += (double)xv[v][i] * (double)xv[v][i];
         s1 = mmf_wave_sum(s1);
-        if ((threadIdx.x & 63) == 0) red_a[threadIdx.x >> 6] = s1;
+        if ((threadIdx.x & 63) == 0) red_a[wave] = s1;
         __syncthreads();
-        s1 = red_a[0] + red_a[1] + red_a[2] + red_a[3];
+        s1 = red_a[0];
+#pragma unroll
+        for (int w = 1; w < kQWaves; ++w) s1 += red_a[w];
         const float rstd1 = mmf_rstd(s1, K, a.inv_K, a.eps1);
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
-            const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
-            if (k0 < K) {
+            const int k0 = (v * kQThreads + (int)threadIdx.x) * 4;
+            float w1v[4];
+            raw4_unpack<TW>(w1raw[v], w1v);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    float y = __fmul_rn(__fmul_rn(xv[v][i], rstd1), w1v[v][i]);
-                    if constexpr (PRO == QPRO_STEP_GATE) y = __fmul_rn(__fmul_rn(y, av[v][i]), mmf_sigmoid(av[v][i]));
-                    xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(y) : 0.0f;
-                }
+            for (int i = 0; i < 4; ++i) {
+                float y = __fmul_rn(__fmul_rn(xv[v][i], rstd1), w1v[i]);
+                if constexpr (STEP) y = __fmul_rn(__fmul_rn(y, av[v][i]), mmf_sigmoid(av[v][i]));
+                xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(y) : 0.0f;
             }
         }
     } else {
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
-            const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
-            if (k0 < K) {
+            const int k0 = (v * kQThreads + (int)threadIdx.x) * 4;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const float g = xv[v][i];
-                    const float z = __fdiv_rn(__fmul_rn(g, av[v][i]), __fadd_rn(1.0f, mmf_exp(-g)));
-                    xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(z) : 0.0f;
-                }
+            for (int i = 0; i < 4; ++i) {
+                const float g = xv[v][i];
+                const float z = __fdiv_rn(__fmul_rn(g, av[v][i]), __fadd_rn(1.0f, mmf_exp(-g)));
+                xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(z) : 0.0f;
             }
         }
     }
@@ -330,77 +326,84 @@ __global__ __launch_bounds__(kThreads) void row_quant_fused_kernel(FusedQuantArg
 #pragma unroll
     for (int v = 0; v < NV; ++v)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
+        for (int i = 0; i < 4; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
     ss = mmf_wave_sum(ss);
-    if ((threadIdx.x & 63) == 0) red_b[threadIdx.x >> 6] = ss;
+    if ((threadIdx.x & 63) == 0) red_b[wave] = ss;
     __syncthreads();
-    ss = red_b[0] + red_b[1] + red_b[2] + red_b[3];
+    ss = red_b[0];
+#pragma unroll
+    for (int w = 1; w < kQWaves; ++w) ss += red_b[w];
     const float rstd = mmf_rstd(ss, K, a.inv_K, a.eps);
     float amax = 0.0f;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
-        if (k0 < K) {
+        float wv[4];
+        if (nw) raw4_unpack<TW>(nwraw[v], wv);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                float y = __fmul_rn(xv[v][i], rstd);
-                if (nw) y = __fmul_rn(y, wv[v][i]);
-                xv[v][i] = y;
-                amax = fmaxf(amax, fabsf(y));
-            }
+        for (int i = 0; i < 4; ++i) {
+            float y = __fmul_rn(xv[v][i], rstd);
+            if (nw) y = __fmul_rn(y, wv[i]);
+            xv[v][i] = y;                                       // elements past K are exact zeros and stay so
+            amax = fmaxf(amax, fabsf(y));
         }
     }
     amax = mmf_wave_max(amax);
-    if ((threadIdx.x & 63) == 0) red_f[threadIdx.x >> 6] = amax;
+    if ((threadIdx.x & 63) == 0) red_f[wave] = amax;
     __syncthreads();
-    amax = fmaxf(fmaxf(red_f[0], red_f[1]), fmaxf(red_f[2], red_f[3]));
+    amax = red_f[0];
+#pragma unroll
+    for (int w = 1; w < kQWaves; ++w) amax = fmaxf(amax, red_f[w]);
     const float scale = __fdiv_rn(127.0f, fmaxf(amax, 1e-5f));
     int qs = 0;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
+        const int k0 = (v * kQThreads + (int)threadIdx.x) * 4;
         if (k0 < Kp) {
-            uint32_t lo = 0, hi = 0;
+            uint32_t packed4 = 0;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
+            for (int i = 0; i < 4; ++i) {
                 const int c = (k0 + i < K) ? mmf_code(xv[v][i], scale) : 0;
                 qs += c;
-                const uint32_t b = (uint32_t)(c & 0xff) << (8 * (i & 3));
-                if (i < 4) lo |= b; else hi |= b;
+                packed4 |= (uint32_t)(c & 0xff) << (8 * i);
             }
             const int64_t off = ((row >> 5) * (Kp >> 4) + (k0 >> 4)) * 512 + (row & 31) * 16 + (k0 & 15);
-            *reinterpret_cast<uint2*>(a.q + off) = make_uint2(lo, hi);
+            *reinterpret_cast<uint32_t*>(a.q + off) = packed4;
         }
     }
     qs = mmf_wave_sum(qs);
-    if ((threadIdx.x & 63) == 0) red_i[threadIdx.x >> 6] = qs;
+    if ((threadIdx.x & 63) == 0) red_i[wave] = qs;
     __syncthreads();
     if (threadIdx.x == 0) {
+        int qt = 0;
+#pragma unroll
+        for (int w = 0; w < kQWaves; ++w) qt += red_i[w];
         a.deq[row] = __fdiv_rn(1.0f, scale);
-        a.qsum[row] = red_i[0] + red_i[1] + red_i[2] + red_i[3];
+        a.qsum[row] = qt;
     }
 }
 
 template <typename T, typename TW, int PRO>
-int launch_fused_quant(const FusedQuantArgs& a, hipStream_t s) {
-    const int64_t nv = mmf_ceil_div(a.Kp, (int64_t)kThreads * 8);
-    dim3 grid((unsigned)a.M), block(kThreads);
-    if (nv <= 1) row_quant_fused_kernel<T, TW, 1, PRO><<<grid, block, 0, s>>>(a);
-    else if (nv <= 2) row_quant_fused_kernel<T, TW, 2, PRO><<<grid, block, 0, s>>>(a);
-    else if (nv <= 3) row_quant_fused_kernel<T, TW, 3, PRO><<<grid, block, 0, s>>>(a);
-    else if (nv <= 4) row_quant_fused_kernel<T, TW, 4, PRO><<<grid, block, 0, s>>>(a);
-    else return MMF_ERR_WIDE;
+int launch_fused_quant(const FusedQuantArgs& a, bool vec, hipStream_t s) {
+    const int64_t nv = mmf_ceil_div(a.Kp, (int64_t)kQThreads * 4);
+    dim3 grid((unsigned)a.M), block(kQThreads);
+    if (nv > 8) return MMF_ERR_WIDE;
+    if (!vec) row_quant_fused_kernel<T, TW, 8, PRO, false><<<grid, block, 0, s>>>(a);      // ragged rows: one generic build
+    else if (nv <= 1) row_quant_fused_kernel<T, TW, 1, PRO, true><<<grid, block, 0, s>>>(a);
+    else if (nv <= 2) row_quant_fused_kernel<T, TW, 2, PRO, true><<<grid, block, 0, s>>>(a);
+    else if (nv <= 3) row_quant_fused_kernel<T, TW, 3, PRO, true><<<grid, block, 0, s>>>(a);
+    else if (nv <= 4) row_quant_fused_kernel<T, TW, 4, PRO, true><<<grid, block, 0, s>>>(a);
+    else row_quant_fused_kernel<T, TW, 8, PRO, true><<<grid, block, 0, s>>>(a);
     MMF_CHECK_LAUNCH();
     return 0;
 }
 
 template <typename T, typename TW>
-int dispatch_fused_quant(const FusedQuantArgs& a, int pro, hipStream_t s) {
+int dispatch_fused_quant(const FusedQuantArgs& a, int pro, bool vec, hipStream_t s) {
     switch (pro) {
-        case QPRO_NORM: return launch_fused_quant<T, TW, QPRO_NORM>(a, s);
-        case QPRO_RESNORM: return launch_fused_quant<T, TW, QPRO_RESNORM>(a, s);
-        case QPRO_STEP_GATE: return launch_fused_quant<T, TW, QPRO_STEP_GATE>(a, s);
-        case QPRO_SWIGLU: return launch_fused_quant<T, TW, QPRO_SWIGLU>(a, s);
+        case QPRO_NORM: return launch_fused_quant<T, TW, QPRO_NORM>(a, vec, s);
+        case QPRO_RESNORM: return launch_fused_quant<T, TW, QPRO_RESNORM>(a, vec, s);
+        case QPRO_STEP_GATE: return launch_fused_quant<T, TW, QPRO_STEP_GATE>(a, vec, s);
+        case QPRO_SWIGLU: return launch_fused_quant<T, TW, QPRO_SWIGLU>(a, vec, s);
     }
     return MMF_ERR_ARG;
 }
@@ -525,18 +528,21 @@ int mmf_rmsnorm_quant_fused(int prologue, const void* x, int64_t ldx, const void
     a.ldaux2 = aux2 ? ldaux2 : ldx; a.res_out = res_out; a.w1 = w1; a.norm_w = norm_weight; a.lb = lower_bound; a.state = state;
     a.q = q; a.deq = deq; a.qsum = qsum; a.M = M; a.K = K; a.inv_K = 1.0 / (double)K; a.Kp = mmf_round_up(K, 128); a.eps1 = eps1; a.eps = eps;
     if (!aligned16(q)) return MMF_ERR_ALIGN;
-    if (K % 8 == 0 && !(aligned16(x) && aligned16(a.aux) && aligned16(a.aux2) && aligned16(res_out) && aligned16(w1) &&
-                        aligned16(norm_weight) && aligned16(lower_bound) && aligned16(state)))
-        return MMF_ERR_ALIGN;
     if (!norm_weight && !w1) weight_dtype = MMF_F32;
+    const uintptr_t xa = 4 * (x_dtype == MMF_F32 ? 4 : 2), wa = 4 * (weight_dtype == MMF_F32 ? 4 : 2);
+    auto al = [](const void* ptr, uintptr_t n) { return (reinterpret_cast<uintptr_t>(ptr) % n) == 0; };
+    const bool vec = K % 4 == 0 && ldx % 4 == 0 && a.ldaux % 4 == 0 && a.ldaux2 % 4 == 0;
+    if (vec && !(al(x, xa) && al(a.aux, xa) && al(a.aux2, xa) && al(res_out, xa) && al(w1, wa) && al(norm_weight, wa) &&
+                 al(lower_bound, 16) && al(state, 16)))
+        return MMF_ERR_ALIGN;
     const bool wf32 = weight_dtype == MMF_F32;
     if (!wf32 && weight_dtype != x_dtype) return MMF_ERR_ARG;
     switch (x_dtype) {
-        case MMF_F32: return dispatch_fused_quant<float, float>(a, prologue, stream);
-        case MMF_BF16: return wf32 ? dispatch_fused_quant<bf16_t, float>(a, prologue, stream)
-                                   : dispatch_fused_quant<bf16_t, bf16_t>(a, prologue, stream);
-        case MMF_F16: return wf32 ? dispatch_fused_quant<f16_t, float>(a, prologue, stream)
-                                  : dispatch_fused_quant<f16_t, f16_t>(a, prologue, stream);
+        case MMF_F32: return dispatch_fused_quant<float, float>(a, prologue, vec, stream);
+        case MMF_BF16: return wf32 ? dispatch_fused_quant<bf16_t, float>(a, prologue, vec, stream)
+                                   : dispatch_fused_quant<bf16_t, bf16_t>(a, prologue, vec, stream);
+        case MMF_F16: return wf32 ? dispatch_fused_quant<f16_t, float>(a, prologue, vec, stream)
+                                  : dispatch_fused_quant<f16_t, f16_t>(a, prologue, vec, stream);
     }
     return MMF_ERR_ARG;
 }
