@@ -323,3 +323,36 @@ def test_embedding_and_argmax(dev):
     for r in range(2, 5):
         row = logits[r].float()
         assert am[r].item() == int((row == row.max()).nonzero()[0])
+
+
+@pytest.mark.parametrize("k", [2048, 301, 5632, 9000])
+@pytest.mark.parametrize("pro", [1, 2, 4])
+def test_fused_quantiser_equals_the_separate_ops(dev, k, pro):
+    """mmf_rmsnorm_quant_fused through the C ABI (vector and ragged-row builds, 1 to 5 passes per row)
+    against the chain of separately validated ops it replaces: identical codes, scales, code sums."""
+    import matmulfreellm_amd._lib as L_
+    lib = L_.load()
+    torch.manual_seed(20 + pro)
+    m, dt = 5, torch.bfloat16
+    x = torch.randn(m, k).to(dt).to(dev)
+    aux = torch.randn(m, k).to(dt).to(dev)
+    w1 = (1 + 0.1 * torch.randn(k)).to(dt).to(dev)
+    nw = (1 + 0.1 * torch.randn(k)).to(dt).to(dev)
+    if pro == 1:
+        v = F().rmsnorm(x, w1, eps=1e-6)
+    elif pro == 2:
+        v, res = F().rmsnorm(x, w1, residual=aux, eps=1e-6, prenorm=True)
+    else:
+        v = F().swiglu(x, aux)
+    q_ref, deq_ref, qsum_ref = F().rmsnorm_quant(v, nw, eps=1e-8, tiled=True)
+    q = torch.empty_like(q_ref)
+    deq, qsum = torch.empty_like(deq_ref), torch.empty_like(qsum_ref)
+    res_out = torch.empty_like(x)
+    rc = lib.mmf_rmsnorm_quant_fused(pro, x.data_ptr(), k, aux.data_ptr(), k, None, 0, res_out.data_ptr() if pro == 2 else None,
+                                     w1.data_ptr() if pro != 4 else None, 1e-6, nw.data_ptr(), 1e-8, None, None, q.data_ptr(),
+                                     deq.data_ptr(), qsum.data_ptr(), m, k, L_.dtype_id(dt), L_.dtype_id(dt), L_.stream())
+    assert rc == 0
+    assert torch.equal(F().codes_tiled_to_rowmajor(q, m, k), F().codes_tiled_to_rowmajor(q_ref, m, k))
+    assert torch.equal(deq, deq_ref) and torch.equal(qsum, qsum_ref)
+    if pro == 2:
+        assert torch.equal(res_out, res)
