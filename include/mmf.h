@@ -99,6 +99,7 @@ int mmf_rmsnorm_quant(const void* x, const void* residual, const void* weight, i
  *                step on state[M, K] (fp32, in place) as mmf_hgrn_step, then
  *                v = RMSNorm(g; w1, eps1) * o * sigmoid(o)                  layers/hgrn_bit.py:113-139
  *   4 SWIGLU     v = (x * aux) / (1 + exp(-x))                             modeling_hgrn_bit.py:58
+ *   5 GATEDNORM  v = RMSNorm(x; w1, eps1) * aux * sigmoid(aux)             layers/hgrn_bit.py:138 (any number of tokens)
  * v is rounded to the activation dtype like the tensor it replaces; then q = codes of RMSNorm(v; norm_weight, eps). */
 int mmf_rmsnorm_quant_fused(int prologue, const void* x, int64_t ldx, const void* aux, int64_t ldaux, const void* aux2,
                             int64_t ldaux2, void* res_out, const void* w1, float eps1, const void* norm_weight, float eps,

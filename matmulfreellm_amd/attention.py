@@ -82,7 +82,9 @@ class HGRNBitAttention(nn.Module):
 
     def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
                 past_key_values=None, use_cache: Optional[bool] = False, output_attentions: Optional[bool] = False,
-                lower_bound: Optional[torch.Tensor] = None, **kwargs) -> Tuple[torch.Tensor, None, object]:
+                lower_bound: Optional[torch.Tensor] = None, input_norm=None, **kwargs) -> Tuple[torch.Tensor, None, object]:
+        """``input_norm``: the block's RMSNorm in front of this layer; given here, it is folded into the
+        stacked i/f/g projection instead of running as a launch of its own."""
         B, T, _ = hidden_states.shape
         D = self.input_dim
         last_state = past_key_values[self.layer_idx] if use_cache else None
@@ -91,9 +93,12 @@ class HGRNBitAttention(nn.Module):
         if stacked is not None:
             p = self.i_proj
             eps = p.norm.eps if p.fused_eps is None else p.fused_eps
-            ifg = F_.bitlinear(hidden_states, p.norm.weight, stacked, eps=eps)
+            pro = ("norm", input_norm.weight, input_norm.eps) if input_norm is not None else None
+            ifg = F_.bitlinear(hidden_states, p.norm.weight, stacked, eps=eps, prologue=pro)
             i, f, g = ifg[..., :D], ifg[..., D:2 * D], ifg[..., 2 * D:]
         else:
+            if input_norm is not None:
+                hidden_states = input_norm(hidden_states)
             i, f, g = self.i_proj(hidden_states), self.f_proj(hidden_states), self.g_proj(hidden_states)
 
         lb = lower_bound if (lower_bound is not None and self.layer_idx > 0) else None
@@ -117,8 +122,8 @@ class HGRNBitAttention(nn.Module):
         if past_key_values is not None:
             past_key_values.update((recurrent_state,), self.layer_idx, T)
 
-        o = self.g_norm(g, o)
-        o = self.o_proj(o)
+        # g_norm (layers/hgrn_bit.py:138) folded into o_proj
+        o = self.o_proj.forward_fused(g, ("gatednorm", o.reshape(g.shape), self.g_norm.weight, self.g_norm.eps))
         return o, None, past_key_values
 
     def init_state(self, batch_size: int) -> Tuple[torch.Tensor]:

@@ -73,6 +73,17 @@ class BitLinear(nn.Linear):
     def packed_weight(self):
         return self._pack.get(self.weight)
 
+    def run_eps(self):
+        """eps of the inner norm as forward() uses it (FusedBitLinear may override it)."""
+        fe = getattr(self, "fused_eps", None)
+        return self.norm.eps if fe is None else fe
+
+    def forward_fused(self, x, prologue, addend=None):
+        """forward() with the elementwise op that produces x folded into the same launch(es);
+        ``prologue`` as functional.bitlinear takes it."""
+        return F_.bitlinear(x, self.norm.weight, self.packed_weight(), bias=self.bias, eps=self.run_eps(), addend=addend,
+                            prologue=prologue)
+
     def forward(self, x):
         return layer_norm_linear_quant_fn(x, self.norm.weight, self.norm.bias, self.weight, self.bias,
                                           eps=self.norm.eps, is_rms_norm=True, packed=self.packed_weight())

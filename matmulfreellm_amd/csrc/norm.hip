@@ -190,8 +190,9 @@ int dispatch_x(const RowArgs& a, int x_dtype, int r_dtype, int w_dtype, hipStrea
 //   QPRO_STEP_GATE  i = x, f = aux, g = aux2 (raw projections of one token): gate math, one recurrence
 //                   step on the fp32 state (in place), o = T(h); v = T(RMSNorm(g; w1, eps1) * o * sigmoid(o))
 //   QPRO_SWIGLU     v = T((x * aux) / (1 + exp(-x)))                       (MLP activation)
+//   QPRO_GATEDNORM  v = T(RMSNorm(x; w1, eps1) * aux * sigmoid(aux))       (g_norm in front of o_proj, any T)
 // then  y = RMSNorm(v; norm_w, eps),  q = int8 absmax codes of y  (tiled operand layout).
-enum QPro : int { QPRO_NORM = 1, QPRO_RESNORM = 2, QPRO_STEP_GATE = 3, QPRO_SWIGLU = 4 };
+enum QPro : int { QPRO_NORM = 1, QPRO_RESNORM = 2, QPRO_STEP_GATE = 3, QPRO_SWIGLU = 4, QPRO_GATEDNORM = 5 };
 
 struct FusedQuantArgs {
     const void* x; const void* aux; const void* aux2;
@@ -305,7 +306,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 float y = __fmul_rn(__fmul_rn(xv[v][i], rstd1), w1v[i]);
-                if constexpr (STEP) y = __fmul_rn(__fmul_rn(y, av[v][i]), mmf_sigmoid(av[v][i]));
+                if constexpr (STEP || PRO == QPRO_GATEDNORM) y = __fmul_rn(__fmul_rn(y, av[v][i]), mmf_sigmoid(av[v][i]));
                 xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(y) : 0.0f;
             }
         }
@@ -404,6 +405,7 @@ int dispatch_fused_quant(const FusedQuantArgs& a, int pro, bool vec, hipStream_t
         case QPRO_RESNORM: return launch_fused_quant<T, TW, QPRO_RESNORM>(a, vec, s);
         case QPRO_STEP_GATE: return launch_fused_quant<T, TW, QPRO_STEP_GATE>(a, vec, s);
         case QPRO_SWIGLU: return launch_fused_quant<T, TW, QPRO_SWIGLU>(a, vec, s);
+        case QPRO_GATEDNORM: return launch_fused_quant<T, TW, QPRO_GATEDNORM>(a, vec, s);
     }
     return MMF_ERR_ARG;
 }
@@ -519,7 +521,7 @@ int mmf_rmsnorm_quant_fused(int prologue, const void* x, int64_t ldx, const void
     if (M < 0 || K <= 0 || ldx < K) return MMF_ERR_ARG;
     if (M == 0) return 0;
     if (!x || !q || !deq || !qsum) return MMF_ERR_ARG;
-    if (prologue < QPRO_NORM || prologue > QPRO_SWIGLU) return MMF_ERR_ARG;
+    if (prologue < QPRO_NORM || prologue > QPRO_GATEDNORM) return MMF_ERR_ARG;
     if (prologue >= QPRO_RESNORM && (!aux || ldaux < K)) return MMF_ERR_ARG;
     if (prologue == QPRO_STEP_GATE && (!aux2 || ldaux2 < K || !state)) return MMF_ERR_ARG;
     if (prologue != QPRO_SWIGLU && !w1) return MMF_ERR_ARG;

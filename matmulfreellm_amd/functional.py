@@ -228,12 +228,80 @@ def bitlinear_gemv(x2, norm_weight, pw, eps, bias=None, addend=None):
     return out
 
 
+# prologue kinds -> (GEMV prologue id, fused-quantiser prologue id), include/mmf.h
+_PROLOGUES = {"norm": (1, 1), "resnorm": (2, 2), "gatednorm": (3, 5), "swiglu": (4, 4)}
+
+
+def _bitlinear_prologue(x, norm_weight, pw, bias, eps, addend, prologue):
+    """BitLinear with the op in front of it folded into the same launch (M <= 4) or into the quantiser
+    (larger M).  prologue: ("norm", w1, eps1) | ("resnorm", residual, w1, eps1) | ("gatednorm", gate, w1, eps1)
+    | ("swiglu", up).  x and the second operand may be column slices of a wider tensor.
+    Returns out, or (out, summed_residual) for "resnorm"."""
+    lib = L.load()
+    kind = prologue[0]
+    gid, qid = _PROLOGUES[kind]
+    aux = prologue[1] if kind != "norm" else None
+    w1 = prologue[-2] if kind != "swiglu" else None
+    eps1 = float(prologue[-1]) if kind != "swiglu" else 0.0
+    dev = L.require_gpu(x, aux, norm_weight, w1, pw.packed, bias)
+    shp = x.shape
+    k = shp[-1]
+    if k != pw.k:
+        raise ValueError(f"input features {k} != weight in_features {pw.k}")
+
+    def rows(t):                                                # [M, K] view; column slices keep their row stride
+        t2 = t.reshape(-1, k)
+        return t2 if t2.stride(-1) == 1 else t2.contiguous()
+
+    x2 = rows(x)
+    a2 = rows(aux) if aux is not None else None
+    m = x2.shape[0]
+    if a2 is not None and (a2.shape != x2.shape or a2.dtype != x2.dtype):
+        raise ValueError("the prologue operand must match x in shape and dtype")
+    nw = norm_weight.detach().contiguous() if norm_weight is not None else None
+    w1c = w1.detach().contiguous() if w1 is not None else None
+    wdt = nw.dtype if nw is not None else (w1c.dtype if w1c is not None else torch.float32)
+    if w1c is not None and nw is not None and w1c.dtype != nw.dtype:
+        raise ValueError("the two norm weights must share a dtype")
+    res_out = torch.empty(m, k, dtype=x2.dtype, device=dev) if kind == "resnorm" else None
+    out = torch.empty(m, pw.n, dtype=x2.dtype, device=dev)
+    if bias is not None:
+        bias = bias.detach().to(x2.dtype).contiguous()
+    if addend is not None:
+        addend = addend.reshape(m, pw.n)
+        if addend.dtype != x2.dtype or not addend.is_contiguous():
+            raise ValueError("addend must be a contiguous [M, N] tensor of the input dtype")
+    ldx = x2.stride(0) if m > 1 else k
+    lda = (a2.stride(0) if m > 1 else k) if a2 is not None else 0
+    with torch.cuda.device(dev):
+        if m <= GEMV_MAX_M and k <= lib.mmf_bitlinear_gemv_max_k():
+            L.check(lib.mmf_bitlinear_gemv_fused(gid, 0, x2.data_ptr(), ldx, L.ptr(a2), lda, L.ptr(res_out), L.ptr(w1c), eps1,
+                                                 L.ptr(nw), eps, pw.packed.data_ptr(), pw.wdeq.data_ptr(), pw.seg_rows,
+                                                 L.ptr(bias), L.ptr(addend), out.data_ptr(), None, None, None, m, k, pw.n,
+                                                 L.dtype_id(x2.dtype), L.dtype_id(wdt), L.stream()), "mmf_bitlinear_gemv_fused")
+        else:
+            q = torch.empty(lib.mmf_codes_bytes(m, k, 1), dtype=torch.int8, device=dev)
+            deq = torch.empty(m, dtype=torch.float32, device=dev)
+            qsum = torch.empty(m, dtype=torch.int32, device=dev)
+            L.check(lib.mmf_rmsnorm_quant_fused(qid, x2.data_ptr(), ldx, L.ptr(a2), lda, None, 0, L.ptr(res_out), L.ptr(w1c), eps1,
+                                                L.ptr(nw), eps, None, None, q.data_ptr(), deq.data_ptr(), qsum.data_ptr(), m, k,
+                                                L.dtype_id(x2.dtype), L.dtype_id(wdt), L.stream()), "mmf_rmsnorm_quant_fused")
+            bitlinear_mfma(q, deq, qsum, pw, m, x2.dtype, bias, out=out, addend=addend)
+    out = out.reshape(*shp[:-1], pw.n)
+    return (out, res_out.reshape(shp)) if kind == "resnorm" else out
+
+
 def bitlinear(x, norm_weight, pw, bias=None, eps=1e-8, residual=None, prenorm=False, residual_in_fp32=False,
-              path=None, addend=None):
+              path=None, addend=None, prologue=None):
     """Fused BitLinear forward on x [..., K] -> [..., N] (x.dtype).
 
     path: None (by M), "gemv" or "mfma".  With a residual (or prenorm) the two-launch path is used.
+    prologue: see _bitlinear_prologue (the elementwise op that produces this BitLinear's input, fused).
     """
+    if prologue is not None:
+        if residual is not None or prenorm or path is not None:
+            raise ValueError("prologue= excludes residual=, prenorm= and path=")
+        return _bitlinear_prologue(x, norm_weight, pw, bias, eps, addend, prologue)
     lib = L.load()
     L.require_gpu(x)
     shp = x.shape

@@ -59,17 +59,19 @@ class HGRNBitMLP(nn.Module):
         self.gate_proj = BitLinear(self.hidden_size, self.intermediate_size * 2, bias=False)
         self.down_proj = BitLinear(self.intermediate_size, self.hidden_size, bias=False)
 
-    def forward(self, x, residual=None):
-        """down_proj(swiglu(gate, y)); with ``residual`` the block's closing add is fused into
-        the contraction's epilogue."""
-        y = self.gate_proj(x)
-        gate, y = y.chunk(2, -1)
-        z = swiglu(gate, y)
-        if residual is None:
-            return self.down_proj(z)
-        p = self.down_proj
-        eps = p.norm.eps if p.fused_eps is None else p.fused_eps
-        return F_.bitlinear(z, p.norm.weight, p.packed_weight(), bias=p.bias, eps=eps, addend=residual.contiguous())
+    def forward(self, x, residual=None, pre_norm=None):
+        """down_proj(swiglu(gate, y)) as mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py:55-59.
+
+        The swiglu is folded into down_proj's quantiser.  With ``residual`` the block's closing add is
+        fused into down_proj's epilogue; with ``pre_norm`` (the block's mlp_norm) x is the attention
+        output and the residual add + RMSNorm in front of gate_proj (:107) is folded into gate_proj."""
+        inter = self.intermediate_size
+        if pre_norm is not None:
+            y, residual = self.gate_proj.forward_fused(x, ("resnorm", residual, pre_norm.weight, pre_norm.eps))
+        else:
+            y = self.gate_proj(x)
+        addend = residual.contiguous() if residual is not None else None
+        return self.down_proj.forward_fused(y[..., :inter], ("swiglu", y[..., inter:]), addend=addend)
 
 
 class HGRNBitBlock(nn.Module):
@@ -89,13 +91,12 @@ class HGRNBitBlock(nn.Module):
     def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
                 past_key_values=None, use_cache: Optional[bool] = False, output_attentions: Optional[bool] = False,
                 lower_bound: Optional[torch.Tensor] = None, **kwargs):
+        # the reference's op sequence (:97-111) with every norm folded into the BitLinear that consumes it
         residual = hidden_states
-        hidden_states = self.attn_norm(hidden_states)
         hidden_states, attentions, past_key_values = self.attn(
             hidden_states=hidden_states, attention_mask=attention_mask, past_key_values=past_key_values,
-            use_cache=use_cache, output_attentions=output_attentions, lower_bound=lower_bound)
-        hidden_states, residual = self.mlp_norm(hidden_states, residual, True)
-        hidden_states = self.mlp(hidden_states, residual=residual)      # = residual + mlp(hidden_states)
+            use_cache=use_cache, output_attentions=output_attentions, lower_bound=lower_bound, input_norm=self.attn_norm)
+        hidden_states = self.mlp(hidden_states, residual=residual, pre_norm=self.mlp_norm)   # = residual' + mlp(norm(residual'))
         return hidden_states, attentions, past_key_values
 
 
