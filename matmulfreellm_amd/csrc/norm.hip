@@ -206,17 +206,27 @@ struct FusedQuantArgs {
     float eps1, eps;
 };
 
-constexpr int kQWaves = 8, kQThreads = kQWaves * 64;            // a row of 2048 = 4 elements per thread
+constexpr int kQWaves = 8, kQThreads = kQWaves * 64;
 
-// NV passes of 2048 elements.  VEC: K, the strides and every pointer allow 4-element accesses.
-template <typename T, typename TW, int NV, int PRO, bool VEC>
+// RPW rows per workgroup, 512 / RPW threads per row, NV passes of (512 / RPW) * 4 elements.
+//   RPW = 1 : a decode batch has few rows and each launch is a step of a dependent chain, so all
+//             8 waves share one row (shortest latency);
+//   RPW = 8 : prefill has thousands of rows and the kernel should stream: one wave per row, whose
+//             reductions are DPP folds only - no LDS exchange and no barrier anywhere.
+// VEC: K, the strides and every pointer allow 4-element accesses.
+template <typename T, typename TW, int NV, int PRO, bool VEC, int RPW>
 __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantArgs a) {
+    constexpr int TPR = kQThreads / RPW, WPR = TPR / 64;        // threads / waves per row
     __shared__ double red_a[kQWaves], red_b[kQWaves];
     __shared__ float red_f[kQWaves];
     __shared__ int red_i[kQWaves];
     constexpr bool HAS_AUX = PRO >= QPRO_RESNORM, STEP = PRO == QPRO_STEP_GATE, HAS_W1 = PRO != QPRO_SWIGLU;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int64_t row = blockIdx.x;
+    const int w0 = (wave / WPR) * WPR;                          // first wave of this row
+    const int tr = (int)threadIdx.x % TPR;                      // thread within the row
+    const int64_t row_raw = (int64_t)blockIdx.x * RPW + (int)threadIdx.x / TPR;
+    const bool live = row_raw < a.M;                            // rows past M compute on row M-1 and store nothing
+    const int64_t row = live ? row_raw : a.M - 1;
     const int K = (int)a.K, Kp = (int)a.Kp;
     const T* x = static_cast<const T*>(a.x) + row * a.ldx;
     const T* aux = static_cast<const T*>(a.aux) + row * a.ldaux;
@@ -231,7 +241,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
     Raw4<TW> w1raw[HAS_W1 ? NV : 1], nwraw[NV];
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        const int k0 = (v * kQThreads + (int)threadIdx.x) * 4;
+        const int k0 = (v * TPR + tr) * 4;
         xraw[v] = raw4_load<T, VEC>(x, k0, K);
         if constexpr (HAS_AUX) araw[v] = raw4_load<T, VEC>(aux, k0, K);
         if constexpr (STEP) {
@@ -245,7 +255,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
     float xv[NV][4], av[HAS_AUX ? NV : 1][4];
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        const int k0 = (v * kQThreads + (int)threadIdx.x) * 4;
+        const int k0 = (v * TPR + tr) * 4;
         raw4_unpack<T>(xraw[v], xv[v]);
         if constexpr (HAS_AUX) raw4_unpack<T>(araw[v], av[v]);
 #pragma unroll
@@ -255,17 +265,17 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
     if constexpr (PRO == QPRO_RESNORM) {
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
-            const int k0 = (v * kQThreads + (int)threadIdx.x) * 4;
+            const int k0 = (v * TPR + tr) * 4;
 #pragma unroll
             for (int i = 0; i < 4; ++i) xv[v][i] = k0 + i < K ? __fadd_rn(xv[v][i], av[v][i]) : 0.0f;
-            if (a.res_out) raw4_store<T, VEC>(static_cast<T*>(a.res_out) + row * K, k0, K, xv[v]);
+            if (a.res_out && live) raw4_store<T, VEC>(static_cast<T*>(a.res_out) + row * K, k0, K, xv[v]);
         }
     }
     if constexpr (STEP) {
         // gate math + one recurrence step per channel; xv becomes the raw g projection, av the new o
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
-            const int k0 = (v * kQThreads + (int)threadIdx.x) * 4;
+            const int k0 = (v * TPR + tr) * 4;
             float gv[4], stv[4], lbv[4];
             raw4_unpack<T>(graw[v], gv);
             raw4_unpack<float>(straw[v], stv);
@@ -282,7 +292,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
                 av[v][i] = mmf_round_to<T>(h);          // o, the swish gate of the gated norm
                 xv[v][i] = k0 + i < K ? gv[i] : 0.0f;   // the gated norm normalises the g projection
             }
-            raw4_store<float, VEC>(st, k0, K, stv);
+            if (live) raw4_store<float, VEC>(st, k0, K, stv);
         }
     }
     if constexpr (HAS_W1) {
@@ -292,15 +302,17 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
 #pragma unroll
             for (int i = 0; i < 4; ++i) s1 += (double)xv[v][i] * (double)xv[v][i];
         s1 = mmf_wave_sum(s1);
-        if ((threadIdx.x & 63) == 0) red_a[wave] = s1;
-        __syncthreads();
-        s1 = red_a[0];
+        if constexpr (WPR > 1) {
+            if ((threadIdx.x & 63) == 0) red_a[wave] = s1;
+            __syncthreads();
+            s1 = red_a[w0];
 #pragma unroll
-        for (int w = 1; w < kQWaves; ++w) s1 += red_a[w];
+            for (int w = 1; w < WPR; ++w) s1 += red_a[w0 + w];
+        }
         const float rstd1 = mmf_rstd(s1, K, a.inv_K, a.eps1);
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
-            const int k0 = (v * kQThreads + (int)threadIdx.x) * 4;
+            const int k0 = (v * TPR + tr) * 4;
             float w1v[4];
             raw4_unpack<TW>(w1raw[v], w1v);
 #pragma unroll
@@ -313,7 +325,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
     } else {
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
-            const int k0 = (v * kQThreads + (int)threadIdx.x) * 4;
+            const int k0 = (v * TPR + tr) * 4;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const float g = xv[v][i];
@@ -329,11 +341,13 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
 #pragma unroll
         for (int i = 0; i < 4; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
     ss = mmf_wave_sum(ss);
-    if ((threadIdx.x & 63) == 0) red_b[wave] = ss;
-    __syncthreads();
-    ss = red_b[0];
+    if constexpr (WPR > 1) {
+        if ((threadIdx.x & 63) == 0) red_b[wave] = ss;
+        __syncthreads();
+        ss = red_b[w0];
 #pragma unroll
-    for (int w = 1; w < kQWaves; ++w) ss += red_b[w];
+        for (int w = 1; w < WPR; ++w) ss += red_b[w0 + w];
+    }
     const float rstd = mmf_rstd(ss, K, a.inv_K, a.eps);
     float amax = 0.0f;
 #pragma unroll
@@ -349,16 +363,18 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
         }
     }
     amax = mmf_wave_max(amax);
-    if ((threadIdx.x & 63) == 0) red_f[wave] = amax;
-    __syncthreads();
-    amax = red_f[0];
+    if constexpr (WPR > 1) {
+        if ((threadIdx.x & 63) == 0) red_f[wave] = amax;
+        __syncthreads();
+        amax = red_f[w0];
 #pragma unroll
-    for (int w = 1; w < kQWaves; ++w) amax = fmaxf(amax, red_f[w]);
+        for (int w = 1; w < WPR; ++w) amax = fmaxf(amax, red_f[w0 + w]);
+    }
     const float scale = __fdiv_rn(127.0f, fmaxf(amax, 1e-5f));
     int qs = 0;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        const int k0 = (v * kQThreads + (int)threadIdx.x) * 4;
+        const int k0 = (v * TPR + tr) * 4;
         if (k0 < Kp) {
             uint32_t packed4 = 0;
 #pragma unroll
@@ -368,34 +384,53 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
                 packed4 |= (uint32_t)(c & 0xff) << (8 * i);
             }
             const int64_t off = ((row >> 5) * (Kp >> 4) + (k0 >> 4)) * 512 + (row & 31) * 16 + (k0 & 15);
-            *reinterpret_cast<uint32_t*>(a.q + off) = packed4;
+            if (live) *reinterpret_cast<uint32_t*>(a.q + off) = packed4;
         }
     }
     qs = mmf_wave_sum(qs);
-    if ((threadIdx.x & 63) == 0) red_i[wave] = qs;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int qt = 0;
+    if constexpr (WPR > 1) {
+        if ((threadIdx.x & 63) == 0) red_i[wave] = qs;
+        __syncthreads();
+        qs = 0;
 #pragma unroll
-        for (int w = 0; w < kQWaves; ++w) qt += red_i[w];
-        a.deq[row] = __fdiv_rn(1.0f, scale);
-        a.qsum[row] = qt;
+        for (int w = 0; w < WPR; ++w) qs += red_i[w0 + w];
     }
+    if (tr == 0 && live) {
+        a.deq[row] = __fdiv_rn(1.0f, scale);
+        a.qsum[row] = qs;
+    }
+}
+
+template <typename T, typename TW, int PRO, int RPW>
+int launch_fused_quant_rpw(const FusedQuantArgs& a, hipStream_t s) {
+    constexpr int TPR = kQThreads / RPW;
+    const int64_t nv = mmf_ceil_div(a.Kp, (int64_t)TPR * 4);
+    dim3 grid((unsigned)mmf_ceil_div(a.M, (int64_t)RPW)), block(kQThreads);
+    if (nv <= 1) row_quant_fused_kernel<T, TW, 1, PRO, true, RPW><<<grid, block, 0, s>>>(a);
+    else if (nv <= 2) row_quant_fused_kernel<T, TW, 2, PRO, true, RPW><<<grid, block, 0, s>>>(a);
+    else if (nv <= 3) row_quant_fused_kernel<T, TW, 3, PRO, true, RPW><<<grid, block, 0, s>>>(a);
+    else if (nv <= 4) row_quant_fused_kernel<T, TW, 4, PRO, true, RPW><<<grid, block, 0, s>>>(a);
+    else if (nv <= 6) row_quant_fused_kernel<T, TW, 6, PRO, true, RPW><<<grid, block, 0, s>>>(a);
+    else if (nv <= 8) row_quant_fused_kernel<T, TW, 8, PRO, true, RPW><<<grid, block, 0, s>>>(a);
+    else return MMF_ERR_WIDE;
+    MMF_CHECK_LAUNCH();
+    return 0;
 }
 
 template <typename T, typename TW, int PRO>
 int launch_fused_quant(const FusedQuantArgs& a, bool vec, hipStream_t s) {
-    const int64_t nv = mmf_ceil_div(a.Kp, (int64_t)kQThreads * 4);
-    dim3 grid((unsigned)a.M), block(kQThreads);
-    if (nv > 8) return MMF_ERR_WIDE;
-    if (!vec) row_quant_fused_kernel<T, TW, 8, PRO, false><<<grid, block, 0, s>>>(a);      // ragged rows: one generic build
-    else if (nv <= 1) row_quant_fused_kernel<T, TW, 1, PRO, true><<<grid, block, 0, s>>>(a);
-    else if (nv <= 2) row_quant_fused_kernel<T, TW, 2, PRO, true><<<grid, block, 0, s>>>(a);
-    else if (nv <= 3) row_quant_fused_kernel<T, TW, 3, PRO, true><<<grid, block, 0, s>>>(a);
-    else if (nv <= 4) row_quant_fused_kernel<T, TW, 4, PRO, true><<<grid, block, 0, s>>>(a);
-    else row_quant_fused_kernel<T, TW, 8, PRO, true><<<grid, block, 0, s>>>(a);
-    MMF_CHECK_LAUNCH();
-    return 0;
+    if (mmf_ceil_div(a.Kp, (int64_t)kQThreads * 4) > 8) return MMF_ERR_WIDE;
+    if (!vec) {                                                 // ragged rows: one generic build
+        row_quant_fused_kernel<T, TW, 8, PRO, false, 1><<<dim3((unsigned)a.M), dim3(kQThreads), 0, s>>>(a);
+        MMF_CHECK_LAUNCH();
+        return 0;
+    }
+    if (a.M <= 256) return launch_fused_quant_rpw<T, TW, PRO, 1>(a, s);      // decode: latency
+    // prefill: as many rows per workgroup as 8 passes of 4 elements per thread allow
+    if (a.Kp <= 64 * 4 * 8) return launch_fused_quant_rpw<T, TW, PRO, 8>(a, s);
+    if (a.Kp <= 128 * 4 * 8) return launch_fused_quant_rpw<T, TW, PRO, 4>(a, s);
+    if (a.Kp <= 256 * 4 * 8) return launch_fused_quant_rpw<T, TW, PRO, 2>(a, s);
+    return launch_fused_quant_rpw<T, TW, PRO, 1>(a, s);
 }
 
 template <typename T, typename TW>

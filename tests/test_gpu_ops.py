@@ -325,15 +325,17 @@ def test_embedding_and_argmax(dev):
         assert am[r].item() == int((row == row.max()).nonzero()[0])
 
 
-@pytest.mark.parametrize("k", [2048, 301, 5632, 9000])
-@pytest.mark.parametrize("pro", [1, 2, 4])
-def test_fused_quantiser_equals_the_separate_ops(dev, k, pro):
-    """mmf_rmsnorm_quant_fused through the C ABI (vector and ragged-row builds, 1 to 5 passes per row)
-    against the chain of separately validated ops it replaces: identical codes, scales, code sums."""
+@pytest.mark.parametrize("m", [5, 300])
+@pytest.mark.parametrize("k", [2048, 301, 5632, 9000, 3072])
+@pytest.mark.parametrize("pro", [1, 2, 4, 5])
+def test_fused_quantiser_equals_the_separate_ops(dev, m, k, pro):
+    """mmf_rmsnorm_quant_fused through the C ABI (vector and ragged-row builds; one row per workgroup for
+    decode-sized M, 2 / 4 / 8 rows per workgroup above 256 rows) against the chain of separately validated
+    ops it replaces: identical codes, scales, code sums."""
     import matmulfreellm_amd._lib as L_
     lib = L_.load()
     torch.manual_seed(20 + pro)
-    m, dt = 5, torch.bfloat16
+    dt = torch.bfloat16
     x = torch.randn(m, k).to(dt).to(dev)
     aux = torch.randn(m, k).to(dt).to(dev)
     w1 = (1 + 0.1 * torch.randn(k)).to(dt).to(dev)
@@ -342,8 +344,10 @@ def test_fused_quantiser_equals_the_separate_ops(dev, k, pro):
         v = F().rmsnorm(x, w1, eps=1e-6)
     elif pro == 2:
         v, res = F().rmsnorm(x, w1, residual=aux, eps=1e-6, prenorm=True)
-    else:
+    elif pro == 4:
         v = F().swiglu(x, aux)
+    else:
+        v = F().rmsnorm_swishgate(x, aux, w1, eps=1e-6)
     q_ref, deq_ref, qsum_ref = F().rmsnorm_quant(v, nw, eps=1e-8, tiled=True)
     q = torch.empty_like(q_ref)
     deq, qsum = torch.empty_like(deq_ref), torch.empty_like(qsum_ref)
