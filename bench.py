@@ -14,8 +14,8 @@ inputs resident in HBM.  Prints ONE JSON line:
   cpu_baseline the reference's PyTorch formulation (oracle, literal mode, weights
                re-quantised per call as the reference does) timed on this host's cores on a
                bounded sample (2 of the 24 layers + head, scaled to 24)
-  extra        batch-64 decode, prefill-sized BitLinear on the int8 matrix cores (TOP/s and
-               fraction of 5.0 POP/s), HGRN scan and norm bandwidths.
+  extra        batch-64 decode, prompt prefill (8 x 512 tokens), prefill-sized BitLinear on the int8
+               matrix cores (TOP/s and fraction of 5.0 POP/s), HGRN scan and norm bandwidths.
 Synthetic data: random-init N(0, 0.02) weights, uniform random token ids.
 """
 import argparse
@@ -156,6 +156,15 @@ def scan_bench(dev, b=8, t=2048, d=2048, iters=10):
             "chunk64_ms": round(ms_c, 4), "chunk64_GBs": round(nbytes / ms_c / 1e6, 1)}
 
 
+def prefill_bench(model, dev, batch=8, seq=512, iters=5):
+    """Module-path forward over a prompt batch (state cache kept, last-position logits only)."""
+    g = torch.Generator(device=dev).manual_seed(5)
+    ids = torch.randint(0, model.config.vocab_size, (batch, seq), generator=g, device=dev)
+    with torch.no_grad():
+        ms = timed(lambda: model(input_ids=ids, use_cache=True, logits_to_keep=1), iters)
+    return {"batch": batch, "seq_len": seq, "ms": round(ms, 3), "tok_s": round(batch * seq / ms * 1e3)}
+
+
 def norm_bench(dev, m=16384, k=2048, iters=20):
     import matmulfreellm_amd.functional as F_
     g = torch.Generator(device=dev).manual_seed(4)
@@ -265,6 +274,7 @@ def main():
         ms_o, _ = decode_bench(model, other, args.steps, args.warmup, dev)
         extra[f"decode_bs{other}_tok_s"] = round(other * 1e3 / ms_o, 1)
         extra[f"decode_bs{other}_ms_per_step"] = round(ms_o, 4)
+        extra["prefill_8x512"] = prefill_bench(model, dev, 8, 512)
         extra["bitlinear_mfma_gate_proj"] = mfma_bench(dev, 4096, 2048, 11264)
         extra["bitlinear_mfma_down_proj"] = mfma_bench(dev, 4096, 5632, 2048)
         extra["hgrn_scan"] = scan_bench(dev)

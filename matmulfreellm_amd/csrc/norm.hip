@@ -425,11 +425,14 @@ int launch_fused_quant(const FusedQuantArgs& a, bool vec, hipStream_t s) {
         MMF_CHECK_LAUNCH();
         return 0;
     }
-    if (a.M <= 256) return launch_fused_quant_rpw<T, TW, PRO, 1>(a, s);      // decode: latency
+    // decode: latency (the recurrence-step prologue only exists there: one token per row)
+    if (a.M <= 256 || PRO == QPRO_STEP_GATE) return launch_fused_quant_rpw<T, TW, PRO, 1>(a, s);
     // prefill: as many rows per workgroup as 8 passes of 4 elements per thread allow
-    if (a.Kp <= 64 * 4 * 8) return launch_fused_quant_rpw<T, TW, PRO, 8>(a, s);
-    if (a.Kp <= 128 * 4 * 8) return launch_fused_quant_rpw<T, TW, PRO, 4>(a, s);
-    if (a.Kp <= 256 * 4 * 8) return launch_fused_quant_rpw<T, TW, PRO, 2>(a, s);
+    if constexpr (PRO != QPRO_STEP_GATE) {
+        if (a.Kp <= 64 * 4 * 8) return launch_fused_quant_rpw<T, TW, PRO, 8>(a, s);
+        if (a.Kp <= 128 * 4 * 8) return launch_fused_quant_rpw<T, TW, PRO, 4>(a, s);
+        if (a.Kp <= 256 * 4 * 8) return launch_fused_quant_rpw<T, TW, PRO, 2>(a, s);
+    }
     return launch_fused_quant_rpw<T, TW, PRO, 1>(a, s);
 }
 
