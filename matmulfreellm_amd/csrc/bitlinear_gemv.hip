@@ -36,11 +36,8 @@
 
 namespace {
 
-constexpr int kGemvWaves = 8;
-constexpr int kGemvThreads = kGemvWaves * 64;
 constexpr int kGemvEl = 4;                                      // elements of x per thread and pass
-constexpr int kGemvMaxNV = 4;                                   // passes: Kp <= 4 * 512 * 4 = 8192
-constexpr int64_t kGemvMaxK = (int64_t)kGemvMaxNV * kGemvThreads * kGemvEl;
+constexpr int64_t kGemvMaxK = 8192;                             // 16 waves x 2 passes (or 8 waves x 4)
 
 enum Pro : int { PRO_PLAIN = 0, PRO_NORM = 1, PRO_RESNORM = 2, PRO_GATEDNORM = 3, PRO_SWIGLU = 4 };
 enum Epi : int { EPI_PLAIN = 0, EPI_STEP = 1, EPI_SWIGLU = 2 };
@@ -86,17 +83,19 @@ __device__ __forceinline__ float block_max_once(float v, float* slot) {
     return s;
 }
 
-// NV: passes over the row (Kp <= NV * 2048); a wave then owns at most 2 * NV of the row's 1 KiB
-// weight blocks per n-block.  VEC: K, the row strides and every pointer allow 4-element accesses.
+// NW waves per workgroup, NV passes over the row (Kp <= NV * NW * 256); a wave then owns at most
+// 2 * NV of the row's 1 KiB weight blocks per n-block.  The launcher takes the fewest passes, then
+// the fewest waves, that cover K: a thread's instruction stream, not bandwidth, sets the time.  VEC: K, the row strides and every pointer allow 4-element accesses.
 // S: row split.  S = 1: a workgroup owns whole n-blocks (32 output rows; lane = (k-half, row)).
 // S = 4: it owns 8 of the 32 rows, so that a 2048-row projection fills 256 CUs instead of 64; a
 // lane is (k-block of a group of four, k-half, row of 8), a wave-load covers four k-blocks (two
 // 128-byte runs of each 1 KiB block), and the waves share out the (n-block, k-group) items.
-template <typename T, typename TW, int NV, int PRO, int EPI, bool VEC, int S>
-__global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a) {
+template <typename T, typename TW, int NW, int NV, int PRO, int EPI, bool VEC, int S>
+__global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
+    constexpr int kGemvWaves = NW, kGemvThreads = 64 * NW;
     constexpr int R = EPI == EPI_STEP ? 3 : EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int BPW = 2 * NV;
-    constexpr int GMAX = 4 * NV;                                // k-groups of four blocks (S = 4)
+    constexpr int GMAX = NV * NW / 2;                           // k-groups of four blocks (S = 4)
     constexpr int ITEMS = (R * GMAX + kGemvWaves - 1) / kGemvWaves;   // (n-block, k-group) items per wave (S = 4)
     constexpr int CHN = 32 / S;                                 // output channels per workgroup and n-block
     constexpr bool HAS_AUX = PRO >= PRO_RESNORM;
@@ -358,25 +357,25 @@ __global__ __launch_bounds__(kGemvThreads) void bitlinear_gemv_kernel(GemvArgs a
     }
 }
 
+template <typename T, typename TW, int PRO, int EPI, int NW, int NV>
+void launch_gemv_shape(const GemvArgs& a, dim3 grid, bool split, hipStream_t s) {
+    if (split) bitlinear_gemv_kernel<T, TW, NW, NV, PRO, EPI, true, 4><<<grid, dim3(64 * NW), (size_t)a.Kp, s>>>(a);
+    else bitlinear_gemv_kernel<T, TW, NW, NV, PRO, EPI, true, 1><<<grid, dim3(64 * NW), (size_t)a.Kp, s>>>(a);
+}
+
 template <typename T, typename TW, int PRO, int EPI>
 int launch_gemv(const GemvArgs& a, int64_t M, bool vec, hipStream_t s) {
     constexpr int R = EPI == EPI_STEP ? 3 : EPI == EPI_SWIGLU ? 2 : 1;
-    const int nv = (int)mmf_ceil_div((int64_t)a.Kp, (int64_t)kGemvThreads * kGemvEl);
     const int64_t nblocks = mmf_ceil_div(a.N / R, 32);
     // few n-blocks (a 2048-row projection has 64): give each workgroup 8 rows, not 32, to reach every CU
-    const bool split = vec && nblocks * M <= 96;
-    dim3 grid((unsigned)(nblocks * (split ? 4 : 1)), (unsigned)M), block(kGemvThreads);
-    const size_t lds = (size_t)a.Kp;
-    if (!vec) bitlinear_gemv_kernel<T, TW, kGemvMaxNV, PRO, EPI, false, 1><<<grid, block, lds, s>>>(a);   // ragged shapes: one generic build
-    else if (split) {
-        if (nv <= 1) bitlinear_gemv_kernel<T, TW, 1, PRO, EPI, true, 4><<<grid, block, lds, s>>>(a);
-        else if (nv <= 2) bitlinear_gemv_kernel<T, TW, 2, PRO, EPI, true, 4><<<grid, block, lds, s>>>(a);
-        else if (nv <= 3) bitlinear_gemv_kernel<T, TW, 3, PRO, EPI, true, 4><<<grid, block, lds, s>>>(a);
-        else bitlinear_gemv_kernel<T, TW, 4, PRO, EPI, true, 4><<<grid, block, lds, s>>>(a);
-    } else if (nv <= 1) bitlinear_gemv_kernel<T, TW, 1, PRO, EPI, true, 1><<<grid, block, lds, s>>>(a);
-    else if (nv <= 2) bitlinear_gemv_kernel<T, TW, 2, PRO, EPI, true, 1><<<grid, block, lds, s>>>(a);
-    else if (nv <= 3) bitlinear_gemv_kernel<T, TW, 3, PRO, EPI, true, 1><<<grid, block, lds, s>>>(a);
-    else bitlinear_gemv_kernel<T, TW, 4, PRO, EPI, true, 1><<<grid, block, lds, s>>>(a);
+    const bool split = vec && nblocks * M <= 64;             // at most 256 workgroups after the split: one per CU
+    dim3 grid((unsigned)(nblocks * (split ? 4 : 1)), (unsigned)M);
+    if (!vec) bitlinear_gemv_kernel<T, TW, 8, 4, PRO, EPI, false, 1><<<grid, dim3(512), (size_t)a.Kp, s>>>(a);   // ragged shapes: one generic build
+    else if (a.Kp <= 2048) launch_gemv_shape<T, TW, PRO, EPI, 8, 1>(a, grid, split, s);
+    else if (a.Kp <= 3072) launch_gemv_shape<T, TW, PRO, EPI, 12, 1>(a, grid, split, s);
+    else if (a.Kp <= 4096) launch_gemv_shape<T, TW, PRO, EPI, 16, 1>(a, grid, split, s);
+    else if (a.Kp <= 6144) launch_gemv_shape<T, TW, PRO, EPI, 12, 2>(a, grid, split, s);
+    else launch_gemv_shape<T, TW, PRO, EPI, 16, 2>(a, grid, split, s);
     MMF_CHECK_LAUNCH();
     return 0;
 }
