@@ -3,7 +3,8 @@ import torch
 
 from . import _lib as L
 
-GEMV_MAX_M = 4      # rows handled by the fused norm+quant+GEMV launch; above: quantise, then matrix cores
+GEMV_MAX_M = 8      # rows handled by the fused norm+quant+GEMV launch (every workgroup redoes the row's prologue,
+                    # which stops paying off around 8 rows); above: quantise once per row, then the matrix cores
 
 _workspaces = {}
 
@@ -233,7 +234,7 @@ _PROLOGUES = {"norm": (1, 1), "resnorm": (2, 2), "gatednorm": (3, 5), "swiglu": 
 
 
 def _bitlinear_prologue(x, norm_weight, pw, bias, eps, addend, prologue):
-    """BitLinear with the op in front of it folded into the same launch (M <= 4) or into the quantiser
+    """BitLinear with the op in front of it folded into the same launch (M <= GEMV_MAX_M) or into the quantiser
     (larger M).  prologue: ("norm", w1, eps1) | ("resnorm", residual, w1, eps1) | ("gatednorm", gate, w1, eps1)
     | ("swiglu", up).  x and the second operand may be column slices of a wider tensor.
     Returns out, or (out, summed_residual) for "resnorm"."""

@@ -49,7 +49,7 @@ def test_config1_logits_and_greedy_ids_fp32(dev, tiny_fp32):
 
 
 @pytest.mark.parametrize("dtype_name", ["bf16", "fp32"])
-@pytest.mark.parametrize("batch", [1, 3, 8])
+@pytest.mark.parametrize("batch", [1, 3, 8, 12])
 def test_prefill_then_greedy_decode(dev, tiny_fp32, tiny_bf16, dtype_name, batch):
     params, dtype = (tiny_bf16, torch.bfloat16) if dtype_name == "bf16" else (tiny_fp32, torch.float32)
     torch.manual_seed(2)
@@ -70,7 +70,8 @@ def test_prefill_then_greedy_decode(dev, tiny_fp32, tiny_bf16, dtype_name, batch
     assert torch.equal(out.logits[:, -1].cpu(), ref_logits[0])
     for use_graph, fuse in ((False, True), (True, True), (False, False), (True, False)):
         eng = DecodeEngine.for_model(model, batch, use_graph=use_graph, fuse=fuse)
-        assert eng.fused == (fuse and batch <= 4) and eng.fused_mfma == (fuse and batch > 4)
+        from matmulfreellm_amd.functional import GEMV_MAX_M
+        assert eng.fused == (fuse and batch <= GEMV_MAX_M) and eng.fused_mfma == (fuse and batch > GEMV_MAX_M)
         eng.load_state([c[-1] for c in out.past_key_values])
         for t in range(1, 6):
             lg = eng.step(ref_toks[:, t - 1].to(dev)).cpu()
