@@ -216,3 +216,21 @@ def test_fused_decode_matches_per_op_decode_at_width_1024(dev, batch):
         assert torch.equal(a, b)
     for a, b in zip(results[0][1], results[1][1]):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("name", ["fp32", "bf16"])
+def test_model_reproduces_the_committed_golden_vectors(dev, tiny_fp32, tiny_bf16, name):
+    """The HIP path against tests/golden/config1_*.npz: greedy choice at every prompt position, logit bit
+    patterns at 64 fixed vocabulary indices of all 128 positions, and a 12-token greedy continuation."""
+    import os
+    import numpy as np
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", f"config1_{name}.npz"))
+    params, dtype = (tiny_fp32, torch.float32) if name == "fp32" else (tiny_bf16, torch.bfloat16)
+    model = build(params, dtype, dev)
+    ids = torch.from_numpy(g["prompt"]).reshape(1, -1).to(dev)
+    logits = model(input_ids=ids, use_cache=False).logits[0].float().cpu()
+    assert np.array_equal(om.argmax_lowest(logits).numpy(), g["argmax"])
+    probe = torch.from_numpy(g["probe_idx"])
+    assert np.array_equal(logits[:, probe].contiguous().numpy().view(np.uint32), g["probe_bits"])
+    out = model.generate(ids, max_new_tokens=len(g["greedy"])).cpu()
+    assert np.array_equal(out[0, ids.shape[1]:].numpy(), g["greedy"])

@@ -1,5 +1,6 @@
 """Structural invariants that pin the oracle's model wiring (reference: modeling_hgrn_bit.py:55-59, 87-113,
 182-278, 356-409; layers/hgrn_bit.py:83-142) and the statistical agreement of spec and literal arithmetic."""
+import pytest
 import torch
 
 from oracle import model as om
@@ -74,3 +75,19 @@ def test_spec_tracks_literal_statistically():
     cos = torch.nn.functional.cosine_similarity(ls.flatten(), ll.flatten(), dim=0).item()
     agree = (ls.argmax(-1) == ll.argmax(-1)).float().mean().item()
     assert cos > 0.995 and agree > 0.8, (cos, agree)
+
+
+@pytest.mark.parametrize("name", ["fp32", "bf16"])
+def test_oracle_reproduces_the_committed_golden_vectors(name):
+    """tests/golden/config1_*.npz (written by tests/golden/make_golden.py) pin the spec oracle against drift."""
+    import os
+    import importlib.util
+    import numpy as np
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(here, "make_golden.py"))
+    mg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mg)
+    want = np.load(os.path.join(here, f"config1_{name}.npz"))
+    got = mg.vectors(torch.float32 if name == "fp32" else torch.bfloat16)
+    for key in ("prompt", "argmax", "probe_idx", "probe_bits", "greedy"):
+        assert np.array_equal(got[key], want[key]), key
