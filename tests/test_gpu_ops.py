@@ -189,7 +189,7 @@ def _bitlinear_case(dev, dtype, m, k, n, path, bias=False, seed=7):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("mkn", [(1, 2048, 2048), (1, 512, 3072), (3, 5632, 2048), (1, 300, 70), (2, 6912, 2560),
-                                 (1, 5632, 2048), (1, 1024, 3200), (1, 8192, 96), (2, 384, 1504)])
+                                 (1, 5632, 2048), (1, 1024, 3200), (1, 8192, 96), (2, 384, 1504), (1, 301, 70), (2, 6913, 64)])
 def test_bitlinear_gemv(dev, dtype, mkn):
     _bitlinear_case(dev, dtype, *mkn, path="gemv")
 
@@ -360,3 +360,36 @@ def test_fused_quantiser_equals_the_separate_ops(dev, m, k, pro):
     assert torch.equal(deq, deq_ref) and torch.equal(qsum, qsum_ref)
     if pro == 2:
         assert torch.equal(res_out, res)
+
+
+@pytest.mark.parametrize("m", [3, 40])
+@pytest.mark.parametrize("k", [512, 300])
+@pytest.mark.parametrize("kind", ["norm", "resnorm", "gatednorm", "swiglu"])
+def test_bitlinear_prologue_equals_the_separate_ops(dev, m, k, kind):
+    """functional.bitlinear(..., prologue=...) — fused GEMV launch for M <= 8, fused quantiser + matrix cores
+    above — against the separately validated op followed by a plain BitLinear; operands are column slices of
+    wider tensors as in the model (stacked projections), with and without a fused residual add."""
+    torch.manual_seed(31)
+    dt, n = torch.bfloat16, 96
+    wide = torch.randn(m, 2 * k + 8).to(dt).to(dev)
+    x, aux = wide[:, :k], wide[:, k + 8:2 * k + 8]              # row stride 2k+8, second operand offset by 8 elements
+    w1 = (1 + 0.1 * torch.randn(k)).to(dt).to(dev)
+    nw = (1 + 0.1 * torch.randn(k)).to(dt).to(dev)
+    pw = F().ternarize_pack((torch.randn(n, k) * 0.02).to(dt).to(dev))
+    addend = torch.randn(m, n).to(dt).to(dev)
+    if kind == "norm":
+        v, pro = F().rmsnorm(x.contiguous(), w1, eps=1e-6), ("norm", w1, 1e-6)
+    elif kind == "resnorm":
+        v, res = F().rmsnorm(x.contiguous(), w1, residual=aux.contiguous(), eps=1e-6, prenorm=True)
+        pro = ("resnorm", aux, w1, 1e-6)
+    elif kind == "gatednorm":
+        v, pro = F().rmsnorm_swishgate(x.contiguous(), aux.contiguous(), w1, eps=1e-6), ("gatednorm", aux, w1, 1e-6)
+    else:
+        v, pro = F().swiglu(x, aux), ("swiglu", aux)
+    for add in (None, addend):
+        want = F().bitlinear(v, nw, pw, eps=1e-8, addend=add)
+        got = F().bitlinear(x, nw, pw, eps=1e-8, addend=add, prologue=pro)
+        if kind == "resnorm":
+            got, res_got = got
+            assert torch.equal(res_got, res)
+        assert torch.equal(got, want), f"{kind} M={m} K={k} addend={'yes' if add is not None else 'no'}"
