@@ -10,7 +10,8 @@
 // A decode step is a chain of dependent launches whose cost is latency, not bandwidth, so
 // every elementwise op is folded into the GEMV that consumes or produces it.
 //
-// Grid = (row groups of 32 outputs, M).  A workgroup of 8 waves owns R n-blocks of one row of x.
+// Grid = (groups of 32 - or, for small launches, 8 - output rows, M).  A workgroup of 8 to 16 waves owns R
+// n-blocks (or 8 rows of each) of one row of x.
 //   prologue : every workgroup recomputes the row's input itself (the row is <= 16 KiB and L2
 //              resident) and leaves the int8 codes in LDS:
 //                PRO_PLAIN      v = x
@@ -23,11 +24,13 @@
 //              trips cost, so every global load of the kernel (row, norm weights, the wave's
 //              packed weight blocks, the epilogue's operands) is issued up front, raw, and
 //              converted only where it is used; a thread owns 4 elements of the row per pass.
-//   main     : wave w takes the 1 KiB weight blocks kb = w, w+8, ... of each of its R n-blocks;
+//   main     : wave w takes the 1 KiB weight blocks kb = w, w+NW, ... of each of its R n-blocks
+//              (8-row mode: groups of four k-blocks, two 128-byte runs of each);
 //              a lane holds 64 weights of one output row, expands each dword to four
 //              byte-wide code dwords (shift + mask) and accumulates with v_dot4_i32_i8
 //              against the broadcast activation bytes read from LDS.
-//   epilogue : the two k-halves of the 8 waves' lanes are summed through LDS;  r = T(fp32(acc - sum(q)) * deq_row * deq_weight (+ bias)), then
+//   epilogue : the lanes' partial sums (k-halves, waves or k-groups) meet in LDS;
+//              r = T(fp32(acc - sum(q)) * deq_row * deq_weight (+ bias)), then
 //                EPI_PLAIN   out = r, or T(r + addend)                          (residual add)
 //                EPI_STEP    R = 3 (i, f, g rows of the same 32 channels): gate math, one
 //                            recurrence step on the fp32 state, writes o and g

@@ -15,10 +15,14 @@
 //      straight from global memory (they are 16x smaller than the int8 tile they become).
 //   The stored code is t+1 in {0,1,2}; the epilogue subtracts sum_k q[m,k] (qsum).
 //
-// Tiling: a workgroup of WGM x WGN waves computes a (WGM*WM*32) x (WGN*WN*32) tile; each
-// wave owns WM x WN accumulators of 32x32 (16 VGPRs each).  A is staged through LDS in
-// K-slabs of 128, double buffered, one barrier per slab; global loads for slab kb+1 are in
-// flight while slab kb is multiplied.
+// Three kernels, chosen by a measured cost model (dispatch_mfma):
+//   large problems : a workgroup of WGM x WGN waves computes a (WGM*WM*32) x (WGN*WN*32) tile; each
+//                    wave owns WM x WN accumulators of 32x32 (16 VGPRs each); A is staged through
+//                    LDS by DMA in k-blocks of 128, three buffers, one barrier per k-block
+//                    (bitlinear_mfma_dma3_kernel);
+//   small problems : one 32x32 output block per workgroup, 8 waves split K, operands straight
+//                    into registers (bitlinear_mfma_skinny_kernel);
+//   small M with K > 8192 : A staged through registers, double buffered (bitlinear_mfma_kernel).
 #include "mmf_common.h"
 #include "../../include/mmf.h"
 
