@@ -288,7 +288,9 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel):
         """Greedy (default) or top-p sampling; returns [B, T + new] token ids like HF's generate.
 
         Prefill runs the module path with last-position logits only; decode runs the captured
-        whole-step HIP graph of DecodeEngine when use_graph is set (greedy, no padding mask)."""
+        whole-step HIP graph of DecodeEngine when use_graph is set (sampling draws from the graph's logits and
+        feeds the drawn token back; the logits are bit-identical to the module path's, so a seeded generator
+        gives the same tokens either way)."""
         if max_new_tokens is None:
             max_new_tokens = (max_length - input_ids.shape[1]) if max_length is not None else 20
         B = input_ids.shape[0]
@@ -298,7 +300,7 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel):
         tokens = [input_ids]
         finished = torch.zeros(B, dtype=torch.bool, device=input_ids.device)
         engine = None
-        if use_graph and not do_sample and max_new_tokens > 1:
+        if use_graph and max_new_tokens > 1:
             from .decode import DecodeEngine
             engine = DecodeEngine.for_model(self, B)
             engine.load_state([c[-1] for c in cache])

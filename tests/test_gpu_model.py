@@ -234,3 +234,17 @@ def test_model_reproduces_the_committed_golden_vectors(dev, tiny_fp32, tiny_bf16
     assert np.array_equal(logits[:, probe].contiguous().numpy().view(np.uint32), g["probe_bits"])
     out = model.generate(ids, max_new_tokens=len(g["greedy"])).cpu()
     assert np.array_equal(out[0, ids.shape[1]:].numpy(), g["greedy"])
+
+
+def test_top_p_sampling_is_the_same_through_the_decode_graph(dev, tiny_bf16):
+    """generate(do_sample=True, top_p, temperature) as mmfreelm's generate.py calls it: the graph-replayed decode
+    and the module path see bit-identical logits, so equal generator seeds draw equal tokens."""
+    model = build(tiny_bf16, torch.bfloat16, dev)
+    torch.manual_seed(9)
+    ids = torch.randint(0, V, (2, 10), device=dev)
+    outs = []
+    for use_graph in (True, False):
+        g = torch.Generator(device=dev).manual_seed(123)
+        outs.append(model.generate(ids, max_length=26, do_sample=True, top_p=0.4, temperature=0.6, use_graph=use_graph, generator=g))
+    assert outs[0].shape == (2, 26)
+    assert torch.equal(outs[0], outs[1])
