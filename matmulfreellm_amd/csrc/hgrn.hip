@@ -179,35 +179,41 @@ __device__ __forceinline__ void gate_math(float iv, float fv, bool has_lb, float
     xo = mmf_round_to<T>(__fdiv_rn(__fmul_rn(iv, u), __fadd_rn(1.0f, mmf_exp(-iv))));
 }
 
-template <typename T>
+// One kernel for both forms: STEP = false writes (x, g); STEP = true runs one recurrence step on the
+// fp32 state in place and writes o.  grid = (ceil(D / 1024), rows): a thread owns 4 consecutive
+// channels of one row, so there is no index division and the loads are 8- / 16-byte vectors
+// (VEC: D, the row strides and every pointer allow that; otherwise element accesses).
+template <typename T, bool STEP, bool VEC>
 __global__ __launch_bounds__(256) void hgrn_gate_kernel(const T* __restrict__ i_in, int64_t ldi, const T* __restrict__ f_in,
                                                         int64_t ldf, const float* __restrict__ lb,
-                                                        const uint8_t* __restrict__ mask, T* __restrict__ x_out,
-                                                        T* __restrict__ g_out, int64_t rows, int64_t D) {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= rows * D) return;
-    const int64_t r = idx / D, d = idx % D;
-    float xo, go;
-    gate_math<T>(mmf_to_float(i_in[r * ldi + d]), mmf_to_float(f_in[r * ldf + d]), lb != nullptr, lb ? lb[d] : 0.0f, xo, go);
-    if (mask && mask[r] == 0) xo = 0.0f;
-    x_out[idx] = mmf_from_float<T>(xo);
-    g_out[idx] = mmf_from_float<T>(go);
-}
-
-template <typename T>
-__global__ __launch_bounds__(256) void hgrn_step_kernel(const T* __restrict__ i_in, int64_t ldi, const T* __restrict__ f_in,
-                                                        int64_t ldf, const float* __restrict__ lb,
                                                         const uint8_t* __restrict__ mask, float* __restrict__ state,
-                                                        T* __restrict__ o, int64_t rows, int64_t D) {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= rows * D) return;
-    const int64_t r = idx / D, d = idx % D;
-    float xo, go;
-    gate_math<T>(mmf_to_float(i_in[r * ldi + d]), mmf_to_float(f_in[r * ldf + d]), lb != nullptr, lb ? lb[d] : 0.0f, xo, go);
-    if (mask && mask[r] == 0) xo = 0.0f;
-    const float h = __fadd_rn(__fmul_rn(go, state[idx]), xo);
-    state[idx] = h;
-    o[idx] = mmf_from_float<T>(h);
+                                                        T* __restrict__ x_out, T* __restrict__ g_out, int D) {
+    const int64_t r = blockIdx.y;
+    const int d0 = ((int)blockIdx.x * 256 + (int)threadIdx.x) * 4;
+    if (d0 >= D) return;
+    const Raw4<T> iraw = raw4_load<T, VEC>(i_in + r * ldi, d0, D);
+    const Raw4<T> fraw = raw4_load<T, VEC>(f_in + r * ldf, d0, D);
+    Raw4<float> lbraw, straw;
+    if (lb) lbraw = raw4_load<float, VEC>(lb, d0, D);
+    if constexpr (STEP) straw = raw4_load<float, VEC>(state + r * D, d0, D);
+    const bool keep = !(mask && mask[r] == 0);
+    float iv[4], fv[4], lbv[4] = {0.0f, 0.0f, 0.0f, 0.0f}, stv[4], xo[4], go[4];
+    raw4_unpack<T>(iraw, iv);
+    raw4_unpack<T>(fraw, fv);
+    if (lb) raw4_unpack<float>(lbraw, lbv);
+    if constexpr (STEP) raw4_unpack<float>(straw, stv);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        gate_math<T>(iv[e], fv[e], lb != nullptr, lbv[e], xo[e], go[e]);
+        if (!keep) xo[e] = 0.0f;
+        if constexpr (STEP) {
+            stv[e] = __fadd_rn(__fmul_rn(go[e], stv[e]), xo[e]);
+            xo[e] = stv[e];                                     // o = T(h)
+        }
+    }
+    if constexpr (STEP) raw4_store<float, VEC>(state + r * D, d0, D, stv);
+    raw4_store<T, VEC>(x_out + r * D, d0, D, xo);
+    if constexpr (!STEP) raw4_store<T, VEC>(g_out + r * D, d0, D, go);
 }
 
 // ht = h0 (or zeros) for an empty sequence; a kernel, not a memset, so it can be graph captured.
@@ -236,16 +242,36 @@ int launch_scan(const void* x, const void* g, const float* h0, void* o, float* h
 template <typename T>
 int launch_gate(const void* i_in, int64_t ldi, const void* f_in, int64_t ldf, const float* lb, const uint8_t* mask,
                 void* x_out, void* g_out, float* state, int64_t rows, int64_t D, bool step, hipStream_t s) {
-    const int64_t n = rows * D;
-    if (n == 0) return 0;
-    const unsigned blocks = (unsigned)mmf_ceil_div(n, 256);
-    if (step)
-        hgrn_step_kernel<T><<<blocks, 256, 0, s>>>(static_cast<const T*>(i_in), ldi, static_cast<const T*>(f_in), ldf, lb,
-                                                   mask, state, static_cast<T*>(x_out), rows, D);
-    else
-        hgrn_gate_kernel<T><<<blocks, 256, 0, s>>>(static_cast<const T*>(i_in), ldi, static_cast<const T*>(f_in), ldf, lb,
-                                                   mask, static_cast<T*>(x_out), static_cast<T*>(g_out), rows, D);
-    MMF_CHECK_LAUNCH();
+    if (rows * D == 0) return 0;
+    if (rows > 65535 * (int64_t)32768 || D > INT32_MAX - 4) return MMF_ERR_WIDE;
+    auto al = [](const void* p, uintptr_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; };
+    const uintptr_t ea = 4 * sizeof(T);
+    const bool vec = D % 4 == 0 && ldi % 4 == 0 && ldf % 4 == 0 && al(i_in, ea) && al(f_in, ea) && al(x_out, ea) &&
+                     al(g_out, ea) && al(lb, 16) && al(state, 16);
+    const T* ip = static_cast<const T*>(i_in);
+    const T* fp = static_cast<const T*>(f_in);
+    T* xp = static_cast<T*>(x_out);
+    T* gp = static_cast<T*>(g_out);
+    const unsigned gx = (unsigned)mmf_ceil_div(D, (int64_t)1024);
+    // rows go on grid.y (<= 65535 per launch)
+    for (int64_t r0 = 0; r0 < rows; r0 += 65535) {
+        const int64_t nr = rows - r0 < 65535 ? rows - r0 : 65535;
+        dim3 grid(gx, (unsigned)nr);
+        const T* ipr = ip + r0 * ldi;
+        const T* fpr = fp + r0 * ldf;
+        const uint8_t* mk = mask ? mask + r0 : nullptr;
+        float* st = state ? state + r0 * D : nullptr;
+        T* xpr = xp + r0 * D;
+        T* gpr = gp ? gp + r0 * D : nullptr;
+        if (step) {
+            if (vec) hgrn_gate_kernel<T, true, true><<<grid, 256, 0, s>>>(ipr, ldi, fpr, ldf, lb, mk, st, xpr, gpr, (int)D);
+            else hgrn_gate_kernel<T, true, false><<<grid, 256, 0, s>>>(ipr, ldi, fpr, ldf, lb, mk, st, xpr, gpr, (int)D);
+        } else {
+            if (vec) hgrn_gate_kernel<T, false, true><<<grid, 256, 0, s>>>(ipr, ldi, fpr, ldf, lb, mk, st, xpr, gpr, (int)D);
+            else hgrn_gate_kernel<T, false, false><<<grid, 256, 0, s>>>(ipr, ldi, fpr, ldf, lb, mk, st, xpr, gpr, (int)D);
+        }
+        MMF_CHECK_LAUNCH();
+    }
     return 0;
 }
 
