@@ -73,12 +73,16 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 // Requires (checked by the launcher): 64 rows of D elements span < 2^31 bytes, Tlen / 64 < 2^30.
 // LOG: g holds log decays (the chunked entry point's convention); the step uses exp(g).
-template <typename T, bool LOG>
-__global__ __launch_bounds__(512) void hgrn_recurrent_pipelined_kernel(const T* __restrict__ x, const T* __restrict__ g,
+// NW waves per workgroup: 8 for long sequences (the schedule above); 4 or 2 when the sequence has
+// at most 4 or 2 chunks, where more waves would only idle through the barriers - the memory
+// rounds then carry two or all four quarters each.
+template <typename T, bool LOG, int NW>
+__global__ __launch_bounds__(64 * NW) void hgrn_recurrent_pipelined_kernel(const T* __restrict__ x, const T* __restrict__ g,
                                                                        const float* __restrict__ h0, T* __restrict__ o,
                                                                        float* __restrict__ ht, int64_t Tlen, int64_t D) {
     using R = typename std::conditional<sizeof(T) == 4, float, uint16_t>::type;
-    constexpr int NW = 8;
+    constexpr int MR = NW >= 8 ? 4 : NW / 2;                    // memory rounds per iteration
+    constexpr int QPR = 4 / MR;                                 // quarters per memory round
     constexpr int kRsrcFlags = 0x00020000;                      // raw buffer, 32-bit data format, no swizzle
     constexpr int kAll = 0x7fffffff;
     __shared__ float baton[64];
@@ -148,17 +152,15 @@ __global__ __launch_bounds__(512) void hgrn_recurrent_pipelined_kernel(const T* 
             baton[lane] = h;
         }
         __syncthreads();
-        MMF_STORE_QUARTER(c, 0) MMF_LOAD_QUARTER(c + NW, 0)
-        __syncthreads();
-        MMF_STORE_QUARTER(c, 1) MMF_LOAD_QUARTER(c + NW, 1)
-        __syncthreads();
-        MMF_STORE_QUARTER(c, 2) MMF_LOAD_QUARTER(c + NW, 2)
-        __syncthreads();
-        MMF_STORE_QUARTER(c, 3) MMF_LOAD_QUARTER(c + NW, 3)
-        __syncthreads();
-        __syncthreads();
-        __syncthreads();
-        __syncthreads();
+        static_for<0, MR>([&](auto RI) __attribute__((always_inline)) {
+            static_for<0, QPR>([&](auto QI) __attribute__((always_inline)) {
+                constexpr int q = decltype(RI)::value * QPR + decltype(QI)::value;
+                MMF_STORE_QUARTER(c, q) MMF_LOAD_QUARTER(c + NW, q)
+            });
+            __syncthreads();
+        });
+#pragma unroll
+        for (int i = 0; i < NW - 1 - MR; ++i) __syncthreads();   // idle rounds
     }
     for (int i = wave; i < NW - 1; ++i) __syncthreads();         // every wave passes the same number of barriers
     __syncthreads();
@@ -233,8 +235,13 @@ int launch_scan(const void* x, const void* g, const float* h0, void* o, float* h
                 hipStream_t s) {
     if (!scan_fits<T>(Tlen, D)) return MMF_ERR_WIDE;
     dim3 grid((unsigned)mmf_ceil_div(D, 64), (unsigned)BH);
-    hgrn_recurrent_pipelined_kernel<T, LOG><<<grid, 512, 0, s>>>(static_cast<const T*>(x), static_cast<const T*>(g), h0,
-                                                                 static_cast<T*>(o), ht, Tlen, D);
+    const int64_t NC = mmf_ceil_div(Tlen, (int64_t)kCH);
+    const T* xp = static_cast<const T*>(x);
+    const T* gp = static_cast<const T*>(g);
+    T* op = static_cast<T*>(o);
+    if (NC <= 2) hgrn_recurrent_pipelined_kernel<T, LOG, 2><<<grid, 128, 0, s>>>(xp, gp, h0, op, ht, Tlen, D);
+    else if (NC <= 4) hgrn_recurrent_pipelined_kernel<T, LOG, 4><<<grid, 256, 0, s>>>(xp, gp, h0, op, ht, Tlen, D);
+    else hgrn_recurrent_pipelined_kernel<T, LOG, 8><<<grid, 512, 0, s>>>(xp, gp, h0, op, ht, Tlen, D);
     MMF_CHECK_LAUNCH();
     return 0;
 }
