@@ -141,14 +141,23 @@ __global__ __launch_bounds__(64 * NW) void hgrn_recurrent_pipelined_kernel(const
         {                                                        // my turn: chunk c, 64 dependent steps
             const int rem = rem_of(c);
             float h = baton[lane];
-            static_for<0, kCH>([&](auto I) __attribute__((always_inline)) {
-                constexpr int t = decltype(I)::value;
-                const float gl = raw_get<T, R>(gr[t]);
-                const float gv = t < rem ? (LOG ? __expf(gl) : gl) : 1.0f;
-                const float xv = t < rem ? raw_get<T, R>(xr[t]) : -0.0f;
-                h = __fadd_rn(__fmul_rn(gv, h), xv);
-                hs[t] = h;
-            });
+            if (rem == kCH) {                                    // full chunk: no selects on the serial chain's inputs
+                static_for<0, kCH>([&](auto I) __attribute__((always_inline)) {
+                    constexpr int t = decltype(I)::value;
+                    const float gl = raw_get<T, R>(gr[t]);
+                    h = __fadd_rn(__fmul_rn(LOG ? __expf(gl) : gl, h), raw_get<T, R>(xr[t]));
+                    hs[t] = h;
+                });
+            } else {
+                static_for<0, kCH>([&](auto I) __attribute__((always_inline)) {
+                    constexpr int t = decltype(I)::value;
+                    const float gl = raw_get<T, R>(gr[t]);
+                    const float gv = t < rem ? (LOG ? __expf(gl) : gl) : 1.0f;
+                    const float xv = t < rem ? raw_get<T, R>(xr[t]) : -0.0f;
+                    h = __fadd_rn(__fmul_rn(gv, h), xv);
+                    hs[t] = h;
+                });
+            }
             baton[lane] = h;
         }
         __syncthreads();
