@@ -154,3 +154,38 @@ def test_packed_checkpoint_loader_rejects_foreign_files(tmp_path):
     save_file({"x": torch.zeros(1)}, str(tmp_path / ck.PACKED_FILE), metadata={"format": ck.FORMAT})
     with pytest.raises(KeyError):
         ck.load_packed(tmp_path, device="cpu")
+
+
+def test_rejected_shapes_and_pointers_return_their_code_before_any_launch():
+    """MMF_ERR_ARG -1, MMF_ERR_WIDE -2, MMF_ERR_ALIGN -3 (include/mmf.h): every check below sits in front of the
+    first kernel launch, so the calls are safe without a GPU (the fake non-null pointers are never dereferenced)."""
+    from matmulfreellm_amd import _lib
+    lib = _lib.load()
+    P = 4096                                                    # a non-null, 16-byte aligned stand-in
+    # fused GEMV: row too wide for one workgroup's passes; misaligned packed weights; bad prologue / epilogue ids
+    gemv = lambda pro, epi, k, packed=P, n=32, ldx=None: lib.mmf_bitlinear_gemv_fused(
+        pro, epi, P, ldx if ldx is not None else k, None, 0, None, None, 0.0, P, 1e-8, packed, P, 32, None, None, P, None, None,
+        None, 1, k, n, 1, 1, None)
+    assert gemv(0, 0, 9000) == -2
+    assert gemv(0, 0, 2048, packed=P + 8) == -3
+    assert gemv(7, 0, 2048) == -1 and gemv(0, 3, 2048) == -1
+    assert gemv(2, 0, 2048) == -1                               # residual prologue without its second operand
+    assert gemv(0, 0, 2048, ldx=100) == -1                      # row stride shorter than the row
+    assert gemv(0, 1, 2048, n=100) == -1                        # the recurrence-step epilogue wants N = 3 * 32 * j
+    assert lib.mmf_bitlinear_gemv_fused(0, 0, P, 64, None, 0, None, None, 0.0, P, 1e-8, P, P, 32, None, None, P, None, None,
+                                        None, 0, 64, 32, 1, 1, None) == 0      # no rows: nothing to do
+    # fused quantiser
+    fq = lambda pro, k: lib.mmf_rmsnorm_quant_fused(pro, P, k, P, k, None, 0, None, P, 1e-6, P, 1e-8, None, None, P, P, P, 3, k,
+                                                    1, 1, None)
+    assert fq(9, 2048) == -1 and fq(0, 2048) == -1
+    assert fq(1, 20000) == -2
+    assert lib.mmf_rmsnorm_quant_fused(1, P + 2, 2048, None, 0, None, 0, None, P, 1e-6, P, 1e-8, None, None, P, P, P, 3, 2048,
+                                       1, 1, None) == -3
+    # matrix cores: segments must be whole 32-row blocks
+    assert lib.mmf_bitlinear_mfma(P, P, P, P, P, 33, None, None, P, 64, 8, 128, 64, 1, -1, None) == -1
+    # scans: too many (batch, head) pairs for one grid; a 64-step chunk that does not fit 32-bit offsets
+    assert lib.mmf_hgrn_recurrent(P, P, None, P, None, 70000, 4, 64, 1, None) == -1
+    assert lib.mmf_hgrn_recurrent(P, P, None, P, None, 1, 4, 1 << 24, 1, None) == -2
+    assert lib.mmf_hgrn_recurrent(None, None, None, None, None, 0, 4, 64, 1, None) == 0
+    # gate math: row stride shorter than the row
+    assert lib.mmf_hgrn_gate(P, 32, P, 64, None, None, P, P, 2, 64, 1, None) == -1
