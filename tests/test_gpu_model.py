@@ -248,3 +248,23 @@ def test_top_p_sampling_is_the_same_through_the_decode_graph(dev, tiny_bf16):
         outs.append(model.generate(ids, max_length=26, do_sample=True, top_p=0.4, temperature=0.6, use_graph=use_graph, generator=g))
     assert outs[0].shape == (2, 26)
     assert torch.equal(outs[0], outs[1])
+
+
+def test_half_precision_model_as_the_reference_script_runs_it(dev):
+    """mmfreelm's generate.py runs the model with .cuda().half(): fp16 parameters and activations end to end.
+    Prefill logits, greedy tokens and graph-replayed decode logits against the oracle's spec arithmetic in fp16."""
+    from matmulfreellm_amd.decode import DecodeEngine
+    params = om.init_params(2048, 256, 2, seed=4, dtype=torch.float16)
+    torch.manual_seed(6)
+    ids = torch.randint(0, 2048, (2, 24))
+    ref, _ = om.forward(params, ids, 2, mode="spec")
+    toks, step_logits = om.greedy(params, ids, 2, 6, mode="spec")
+    model = build(params, torch.float16, dev)
+    out = model(input_ids=ids.to(dev), use_cache=True)
+    assert torch.equal(out.logits.cpu(), ref)
+    got = model.generate(ids.to(dev), max_new_tokens=6).cpu()
+    assert torch.equal(got[:, 24:], toks)
+    eng = DecodeEngine.for_model(model, 2, use_graph=True)
+    eng.load_state([c[-1] for c in out.past_key_values])
+    for t in range(1, 4):
+        assert torch.equal(eng.step(toks[:, t - 1].to(dev)).cpu(), step_logits[t])
