@@ -65,15 +65,22 @@ struct GemvArgs {
     double inv_K;         // RN(1 / K)
 };
 
+// Pairwise combination of the NW per-wave slots: log2(NW) dependent additions instead of NW - 1
+// (the kernel's time is its longest dependent chain).  Every thread adds in the same order.
+template <int N>
+__device__ __forceinline__ double tree_sum(const double* v) {
+    if constexpr (N == 1) return v[0];
+    else return tree_sum<N / 2>(v) + tree_sum<N - N / 2>(v + N / 2);
+}
 template <int NW>
 __device__ __forceinline__ double block_sum_once(double v, double* slot) {
     v = mmf_wave_sum(v);
     if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = v;
     __syncthreads();
-    double s = slot[0];
+    double t[NW];
 #pragma unroll
-    for (int i = 1; i < NW; ++i) s += slot[i];
-    return s;
+    for (int i = 0; i < NW; ++i) t[i] = slot[i];
+    return tree_sum<NW>(t);
 }
 template <int NW>
 __device__ __forceinline__ float block_max_once(float v, float* slot) {

@@ -229,7 +229,7 @@ __device__ __forceinline__ double mmf_wave_sum(double v) {
     v += mmf_dpp<kDppXor2>(v);
     v += mmf_dpp<kDppHalfMirror>(v);
     v += mmf_dpp<kDppMirror>(v);
-    return ((mmf_readlane(v, 0) + mmf_readlane(v, 16)) + mmf_readlane(v, 32)) + mmf_readlane(v, 48);
+    return (mmf_readlane(v, 0) + mmf_readlane(v, 16)) + (mmf_readlane(v, 32) + mmf_readlane(v, 48));
 }
 __device__ __forceinline__ float mmf_wave_max(float v) {
     v = fmaxf(v, mmf_dpp<kDppXor1>(v));
