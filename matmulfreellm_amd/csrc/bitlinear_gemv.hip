@@ -275,9 +275,11 @@ __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
             *reinterpret_cast<uint32_t*>(q_lds + k0) = packed4;
         }
     }
+    __syncthreads();                                            // publishes q_lds
+    // the code sum is only needed by the epilogue: fold it after the barrier, off the critical path
+    // (red_q is read behind the next barrier)
     qs = mmf_wave_sum(qs);
     if (lane == 0) red_q[wave] = qs;
-    __syncthreads();                                            // publishes q_lds and red_q
 
     // ---- main: sum_k q[k] * (t[n,k] + 1) over this wave's blocks
     auto dot_block = [&](const uint4& wq, int kb, int acc) {
