@@ -99,7 +99,7 @@ def decode_bench(model, batch, steps, warmup, dev, prompt_len=128):
 
 # HBM bytes per GEMV launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain copy of
 # known size); see profiles/bitlinear_gemv_decode_bs1_hbm_traffic.txt for the runs and the scale factors.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3629134
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3629386
 
 
 def gemv_roofline(eng, iters=20):
