@@ -367,10 +367,22 @@ void bitlinear_mfma_dma3_kernel(MfmaArgs p) {
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
+    // Workgroup ids are dealt round-robin to the 8 XCDs.  When the tile rows divide by 8, XCD x owns rows
+    // [x*R, (x+1)*R) and walks the columns with the rows running fastest: the R workgroups that share a weight
+    // tile run together, and the R activation panels stay in that XCD's L2 for the whole walk.
     int64_t wg = blockIdx.x;
     const int64_t total = (int64_t)p.tiles_m * p.tiles_n;
-    if (total % 8 == 0) wg = (wg % 8) * (total / 8) + wg / 8;
-    const int64_t tile_m = wg / p.tiles_n, tile_n = wg % p.tiles_n;
+    int64_t tile_m, tile_n;
+    if (p.tiles_m % 8 == 0) {
+        const int R = p.tiles_m >> 3, x = (int)(wg & 7);
+        const int64_t l = wg >> 3;
+        tile_m = x * R + l % R;
+        tile_n = l / R;
+    } else {
+        if (total % 8 == 0) wg = (wg % 8) * (total / 8) + wg / 8;
+        tile_m = wg / p.tiles_n;
+        tile_n = wg % p.tiles_n;
+    }
     const int64_t MB = (p.M + 31) >> 5, NB = (p.N + 31) >> 5;
     const int KB = (int)(p.Kp >> 7);
     const int64_t KG = p.Kp >> 4;
@@ -631,7 +643,8 @@ int dispatch_mfma(const MfmaArgs& a, int config, hipStream_t s) {
     // config < 0: pick by shape.
     //   5        weight-stream kernel: one 32x32 output block per workgroup, 8 waves split K (needs Kp <= 8192)
     //   0 / 1    32x256 / 64x256 tiles, A staged through registers (small M with Kp > 8192)
-    //   15 / 16  256x256 / 128x256 tiles, A staged by DMA
+    //   15 / 16 / 17  256x256 / 128x256 / 64x512 tiles, A staged by DMA (17: every wave reads the whole activation
+    //            tile from LDS and owns its own weight columns, so no weight block is fetched twice)
     if (config < 0) {
         const int64_t KB = a.Kp >> 7;
         const double wgs = (double)mmf_ceil_div(a.M, 32) * (double)mmf_ceil_div(a.N, 32);
@@ -643,7 +656,7 @@ int dispatch_mfma(const MfmaArgs& a, int config, hipStream_t s) {
         if (a.Kp <= 8192 && (a.M <= 64 || t_stream < t_tiled)) config = 5;
         else if (a.M <= 32) config = 0;
         else if (a.M <= 64) config = 1;
-        else config = 16;
+        else config = a.N >= 512 ? 17 : 16;
     }
     if (config == 5 && (a.Kp > 8192 || a.M > 65535 * 32)) return MMF_ERR_ARG;
     switch (config) {
@@ -652,6 +665,7 @@ int dispatch_mfma(const MfmaArgs& a, int config, hipStream_t s) {
         case 1: return launch_mfma<T, 1, 8, 2, 1>(a, s);
         case 15: return launch_mfma_dma3<T, 2, 4, 4, 2>(a, s);
         case 16: return launch_mfma_dma3<T, 2, 4, 2, 2>(a, s);
+        case 17: return launch_mfma_dma3<T, 1, 8, 2, 2>(a, s);
     }
     return MMF_ERR_ARG;
 }

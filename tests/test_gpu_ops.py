@@ -211,10 +211,13 @@ def test_bitlinear_bias_and_known_answers(dev):
                                           (5, 40, 5632, 2048), (5, 64, 8192, 96), (5, 33, 6912, 2560), (5, 300, 1024, 648),
                                           (15, 520, 2048, 1032), (15, 300, 128, 640), (15, 300, 256, 648), (16, 300, 1152, 640),
                                           (15, 4096, 2048, 1024), (16, 70, 384, 100), (15, 300, 1024, 644), (16, 300, 1024, 648),
-                                          (16, 200, 128, 520), (-1, 4096, 512, 2048), (-1, 100, 512, 256), (-1, 40, 8320, 96)])
+                                          (16, 200, 128, 520), (-1, 4096, 512, 2048), (-1, 100, 512, 256), (-1, 40, 8320, 96),
+                                          (17, 300, 1152, 640), (17, 520, 2048, 1032), (17, 4096, 2048, 1024), (17, 512, 256, 648),
+                                          (17, 70, 384, 100), (16, 1024, 256, 520), (15, 2048, 256, 300), (17, 1000, 128, 1600)])
 def test_bitlinear_mfma_all_tile_configs(dev, config, m, k, n):
     """Every tile shape of the matrix-core contraction (0/1 register-staged, 5 the weight-stream kernel,
-    15/16 DMA-staged; ragged M, K, N; one and two k-blocks)."""
+    15/16/17 DMA-staged; ragged M, K, N; one and two k-blocks; tile-row counts that do and do not divide by the
+    8 XCDs, which selects the tile order)."""
     torch.manual_seed(8)
     x = torch.randn(m, k).bfloat16()
     w = (torch.randn(n, k) * 0.02).bfloat16()
