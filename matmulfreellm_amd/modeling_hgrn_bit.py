@@ -4,8 +4,10 @@ Same module tree, parameter names and forward semantics as
 mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py (MLP :29-59, Block :62-113, PreTrainedModel
 :116-156, Model :159-278, ForCausalLM :281-409), so a checkpoint's state dict loads as is.
 Differences, all on the host side:
-  * the recurrent state cache is this package's RecurrentCache, and generation is a plain
-    greedy / top-p loop owned by the class (transformers >= 5 no longer gives
+  * the recurrent state cache is this package's RecurrentCache; ``generate()`` runs a greedy / top-p loop
+    owned by the class on the captured decode graph for the arguments the reference's generate.py uses, and
+    hands every other call (beams, logits processors, stopping criteria, streamers, a GenerationConfig) to
+    transformers' GenerationMixin, which the class inherits explicitly (transformers >= 5 no longer gives
     PreTrainedModel a generate());
   * ``logits_to_keep`` lets a caller ask for the last positions' logits only (the
     reference projects all T positions through the 32000-wide head);
@@ -19,6 +21,7 @@ from typing import List, Optional, Tuple, Union
 
 import torch
 import torch.nn as nn
+from transformers.generation import GenerationMixin
 from transformers.modeling_outputs import BaseModelOutputWithPast, CausalLMOutputWithPast
 from transformers.modeling_utils import PreTrainedModel
 
@@ -210,8 +213,15 @@ class HGRNBitModel(HGRNBitPreTrainedModel):
                                        hidden_states=all_hidden_states, attentions=None)
 
 
-class HGRNBitForCausalLM(HGRNBitPreTrainedModel):
+class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
     _tied_weights_keys = {}
+    # the recurrent state cannot be rolled back to an earlier position: GenerationMixin refuses assisted decoding
+    _is_stateful = True
+
+    @classmethod
+    def _supports_default_dynamic_cache(cls) -> bool:
+        """GenerationMixin must not build a key/value cache: the first forward creates the RecurrentCache."""
+        return False
 
     def __init__(self, config):
         super().__init__(config)
@@ -240,20 +250,34 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel):
 
     def prepare_inputs_for_generation(self, input_ids: torch.LongTensor = None, past_key_values=None,
                                       attention_mask: Optional[torch.Tensor] = None,
-                                      inputs_embeds: Optional[torch.Tensor] = None, **kwargs):
-        """modeling_hgrn_bit.py:326-354: keep only the last token once a cache exists."""
-        if past_key_values is not None:
+                                      inputs_embeds: Optional[torch.Tensor] = None,
+                                      next_sequence_length: Optional[int] = None,
+                                      is_first_iteration: Optional[bool] = None, **kwargs):
+        """modeling_hgrn_bit.py:326-354: once a cache holds state, only the new tokens are fed.
+
+        Called by GenerationMixin with the whole sequence so far and a mask of the same length.
+        ``next_sequence_length`` (transformers >= 5) says how many trailing tokens are new; older
+        releases do not pass it and always mean one."""
+        has_state = past_key_values is not None and len(past_key_values) > 0
+        if has_state:
             if not isinstance(past_key_values, RecurrentCache):
                 past_key_values = RecurrentCache.from_legacy_cache(past_key_values, input_ids.shape[1] - 1)
-            input_ids = input_ids[:, -1:]
+            n_new = next_sequence_length if next_sequence_length is not None else 1
+            input_ids = input_ids[:, -n_new:]
             if attention_mask is not None:
-                attention_mask = attention_mask[:, -1:]
-        if inputs_embeds is not None and past_key_values is None:
+                attention_mask = attention_mask[:, -n_new:]
+        elif next_sequence_length is not None:
+            input_ids = input_ids[:, -next_sequence_length:]
+            if attention_mask is not None:
+                attention_mask = attention_mask[:, -next_sequence_length:]
+        if inputs_embeds is not None and not has_state:
             model_inputs = {"inputs_embeds": inputs_embeds}
         else:
             model_inputs = {"input_ids": input_ids.contiguous()}
         model_inputs.update({"past_key_values": past_key_values, "use_cache": kwargs.get("use_cache"),
                              "attention_mask": attention_mask})
+        if kwargs.get("logits_to_keep") is not None:
+            model_inputs["logits_to_keep"] = kwargs["logits_to_keep"]
         return model_inputs
 
     @torch.no_grad()
@@ -281,16 +305,32 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel):
 
     # ------------------------------------------------------------------ generation
     @torch.no_grad()
-    def generate(self, input_ids: torch.LongTensor, attention_mask: Optional[torch.Tensor] = None,
+    def generate(self, input_ids: Optional[torch.LongTensor] = None, attention_mask: Optional[torch.Tensor] = None,
                  max_new_tokens: Optional[int] = None, max_length: Optional[int] = None, do_sample: bool = False,
                  top_p: float = 1.0, temperature: float = 1.0, eos_token_id: Optional[int] = None,
-                 use_graph: bool = True, generator: Optional[torch.Generator] = None, **kwargs) -> torch.LongTensor:
+                 pad_token_id: Optional[int] = None, use_graph: bool = True,
+                 generator: Optional[torch.Generator] = None, **kwargs) -> torch.LongTensor:
         """Greedy (default) or top-p sampling; returns [B, T + new] token ids like HF's generate.
 
-        Prefill runs the module path with last-position logits only; decode runs the captured
-        whole-step HIP graph of DecodeEngine when use_graph is set (sampling draws from the graph's logits and
-        feeds the drawn token back; the logits are bit-identical to the module path's, so a seeded generator
-        gives the same tokens either way)."""
+        With the arguments above (what the reference's generate.py passes), prefill runs the module path with
+        last-position logits only and decode runs the captured whole-step HIP graph of DecodeEngine when
+        use_graph is set (sampling draws from the graph's logits and feeds the drawn token back; the logits are
+        bit-identical to the module path's, so a seeded generator gives the same tokens either way). Rows that
+        have produced eos_token_id are filled with pad_token_id (eos_token_id when not given).
+
+        Any further keyword (num_beams, repetition_penalty, logits_processor, stopping_criteria, streamer,
+        generation_config, top_k, return_dict_in_generate, ...) sends the whole call to
+        transformers' GenerationMixin.generate, which steps the module path through
+        prepare_inputs_for_generation and the RecurrentCache."""
+        if kwargs or input_ids is None or not isinstance(eos_token_id, (int, type(None))):
+            hf = dict(kwargs)
+            for name, value, default in (("attention_mask", attention_mask, None), ("max_new_tokens", max_new_tokens, None),
+                                         ("max_length", max_length, None), ("top_p", top_p, 1.0),
+                                         ("temperature", temperature, 1.0), ("eos_token_id", eos_token_id, None),
+                                         ("pad_token_id", pad_token_id, None)):
+                if value is not None and not (isinstance(default, float) and value == default):
+                    hf[name] = value
+            return GenerationMixin.generate(self, input_ids, do_sample=do_sample, **hf)
         if max_new_tokens is None:
             max_new_tokens = (max_length - input_ids.shape[1]) if max_length is not None else 20
         B = input_ids.shape[0]
@@ -310,7 +350,7 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel):
             else:
                 nxt = F_.argmax(logits)
             if eos_token_id is not None:
-                nxt = torch.where(finished, torch.full_like(nxt, eos_token_id), nxt)
+                nxt = torch.where(finished, torch.full_like(nxt, eos_token_id if pad_token_id is None else pad_token_id), nxt)
                 finished |= nxt == eos_token_id
             tokens.append(nxt.view(B, 1))
             if step == max_new_tokens - 1 or (eos_token_id is not None and bool(finished.all())):

@@ -268,3 +268,55 @@ def test_half_precision_model_as_the_reference_script_runs_it(dev):
     eng.load_state([c[-1] for c in out.past_key_values])
     for t in range(1, 4):
         assert torch.equal(eng.step(toks[:, t - 1].to(dev)).cpu(), step_logits[t])
+
+
+def test_generation_mixin_steps_the_same_model(dev, tiny_bf16):
+    """transformers' GenerationMixin.generate driving this model (prepare_inputs_for_generation, RecurrentCache,
+    logits_to_keep) yields the oracle's greedy tokens, with and without a left-padding mask, and the call is what
+    generate() falls back to for keywords its own loop does not take."""
+    from transformers.generation import GenerationMixin
+    model = build(tiny_bf16, torch.bfloat16, dev)
+    torch.manual_seed(21)
+    ids = torch.randint(0, V, (3, 16))
+    ref_toks, _ = om.greedy(tiny_bf16, ids, L, 8, mode="spec")
+    hf = GenerationMixin.generate(model, ids.to(dev), attention_mask=torch.ones_like(ids).to(dev), max_new_tokens=8,
+                                  do_sample=False, pad_token_id=0)
+    assert hf.shape == (3, 24)
+    assert torch.equal(hf[:, 16:].cpu(), ref_toks)
+    # routed through generate(): a keyword of GenerationMixin (a no-op repetition penalty) selects transformers' loop
+    routed = model.generate(ids.to(dev), attention_mask=torch.ones_like(ids).to(dev), max_new_tokens=8,
+                            repetition_penalty=1.0, pad_token_id=0)
+    assert torch.equal(routed.cpu(), hf.cpu())
+    # left padding: the mask grows with the sequence inside transformers' loop, the model sees the new column only
+    mask = torch.ones(3, 16, dtype=torch.long)
+    mask[1, :6] = 0
+    own = model.generate(ids.to(dev), attention_mask=mask.to(dev), max_new_tokens=8)
+    hf_m = GenerationMixin.generate(model, ids.to(dev), attention_mask=mask.to(dev), max_new_tokens=8, do_sample=False,
+                                    pad_token_id=0)
+    assert torch.equal(own.cpu(), hf_m.cpu())
+
+
+def test_generation_mixin_beam_search_and_stopping(dev, tiny_bf16):
+    """Beam search reorders the recurrent state per beam (RecurrentCache.reorder_cache); the best beam's sequence
+    log-probability under the model is at least the greedy sequence's.  An eos token stops rows and pads them."""
+    model = build(tiny_bf16, torch.bfloat16, dev)
+    torch.manual_seed(22)
+    ids = torch.randint(0, V, (2, 12), device=dev)
+    n_new = 6
+    greedy = model.generate(ids, max_new_tokens=n_new)
+    beams = model.generate(ids, max_new_tokens=n_new, num_beams=3, pad_token_id=0, length_penalty=0.0)
+    assert beams.shape == greedy.shape and torch.equal(beams[:, :12], ids)
+
+    def seq_logprob(seq):
+        logits = model(input_ids=seq, use_cache=False).logits.float()
+        lp = torch.log_softmax(logits[:, 11:-1], dim=-1)
+        return lp.gather(-1, seq[:, 12:].unsqueeze(-1)).squeeze(-1).sum(-1)
+
+    assert bool((seq_logprob(beams) >= seq_logprob(greedy) - 1e-3).all())
+    # stopping: take the token greedy decoding emits third for row 0 as the eos token
+    eos = int(greedy[0, 14])
+    stopped = model.generate(ids, max_new_tokens=n_new, eos_token_id=eos, pad_token_id=0, repetition_penalty=1.0)
+    own = model.generate(ids, max_new_tokens=n_new, eos_token_id=eos, pad_token_id=0)
+    assert torch.equal(stopped[0, :15], greedy[0, :15])
+    assert bool((stopped[0, 15:] == 0).all())
+    assert torch.equal(own[:, :stopped.shape[1]], stopped)

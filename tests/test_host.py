@@ -189,3 +189,35 @@ def test_rejected_shapes_and_pointers_return_their_code_before_any_launch():
     assert lib.mmf_hgrn_recurrent(None, None, None, None, None, 0, 4, 64, 1, None) == 0
     # gate math: row stride shorter than the row
     assert lib.mmf_hgrn_gate(P, 32, P, 64, None, None, P, P, 2, 64, 1, None) == -1
+
+
+def test_generation_mixin_wiring():
+    """The causal LM is a transformers GenerationMixin model that brings its own cache: transformers must not
+    build a key/value cache for it, prepare_inputs_for_generation feeds only the new tokens once state exists,
+    and a call on CPU tensors reaches the HIP-only forward (there is no CPU path to fall back to)."""
+    import pytest
+    from transformers.generation import GenerationMixin
+    from matmulfreellm_amd.modeling_hgrn_bit import HGRNBitForCausalLM
+    from matmulfreellm_amd.configuration_hgrn_bit import HGRNBitConfig
+    from matmulfreellm_amd.cache import RecurrentCache
+    from matmulfreellm_amd._lib import MMFError
+    model = HGRNBitForCausalLM(HGRNBitConfig(vocab_size=64, hidden_size=64, num_hidden_layers=2, num_heads=1))
+    assert isinstance(model, GenerationMixin) and model.can_generate()
+    assert model._is_stateful and not model._supports_default_dynamic_cache()
+    ids = torch.arange(10).view(2, 5)
+    mask = torch.ones(2, 5, dtype=torch.long)
+    first = model.prepare_inputs_for_generation(ids, attention_mask=mask, use_cache=True, logits_to_keep=1,
+                                                is_first_iteration=True)
+    assert first["input_ids"].shape == (2, 5) and first["past_key_values"] is None and first["logits_to_keep"] == 1
+    cache = RecurrentCache()
+    for layer in range(2):
+        cache.update((torch.zeros(2, 64),), layer)
+    for kw in ({"next_sequence_length": 1}, {}, {"next_sequence_length": 2}):
+        step = model.prepare_inputs_for_generation(ids, past_key_values=cache, attention_mask=mask, use_cache=True, **kw)
+        n = kw.get("next_sequence_length", 1)
+        assert torch.equal(step["input_ids"], ids[:, -n:]) and step["attention_mask"].shape == (2, n)
+        assert step["past_key_values"] is cache
+    with pytest.raises(MMFError):
+        model.generate(ids, attention_mask=mask, max_new_tokens=2, num_beams=2, pad_token_id=0)
+    with pytest.raises(MMFError):
+        model.generate(ids, max_new_tokens=2)
