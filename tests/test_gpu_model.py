@@ -36,7 +36,7 @@ def tiny_bf16():
 
 
 def test_config1_logits_and_greedy_ids_fp32(dev, tiny_fp32):
-    """BASELINE config 1: tiny model, fp32, batch 1, seq 128: logits and greedy next-token ids."""
+    """The CPU-runnable benchmark configuration: tiny model, fp32, batch 1, seq 128: logits and greedy next-token ids."""
     torch.manual_seed(1)
     ids = torch.randint(0, V, (1, 128))
     ref, _ = om.forward(tiny_fp32, ids, L, mode="spec")

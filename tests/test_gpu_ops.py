@@ -2,7 +2,7 @@
 
 Integer codes must match bit for bit.  Float outputs of kernels that follow the spec
 arithmetic are compared for exact equality too (a mismatch count is reported), with the
-north-star tolerance (1e-2 relative in bf16, 1e-3 with fp32 tensors) as the hard bound.
+stated tolerance (1e-2 relative in bf16, 1e-3 with fp32 tensors) as the hard bound.
 """
 import numpy as np
 import pytest
@@ -230,7 +230,7 @@ def test_bitlinear_mfma_all_tile_configs(dev, config, m, k, n):
 
 
 def test_bitlinear_full_size_gate_proj(dev):
-    """BASELINE shape M=4096, K=2048, N=11264 against the exact integer accumulator on the device
+    """The 1.3B gate projection at prefill size, M=4096, K=2048, N=11264 against the exact integer accumulator on the device
     (int64 matmul of the oracle's codes is too slow on CPU at this size, so the check is
     torch's own integer matmul in fp64 on the GPU: exact for |acc| < 2**53)."""
     torch.manual_seed(9)
