@@ -17,14 +17,24 @@ __global__ __launch_bounds__(256) void embedding_kernel(const T* __restrict__ ta
     if (id < 0 || id >= vocab) id = 0;   // out-of-range ids read row 0 instead of faulting
     const T* src = table + id * H;
     T* dst = out + r * H;
-    for (int64_t c = threadIdx.x; c < H; c += 256) dst[c] = src[c];
+    constexpr int PER = 16 / (int)sizeof(T);
+    if (H % PER == 0 && ((reinterpret_cast<uintptr_t>(table) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0) {
+        // 16 bytes per thread: a 2048-wide 16-bit row is one load and one store per thread
+        const uint4* s4 = reinterpret_cast<const uint4*>(src);
+        uint4* d4 = reinterpret_cast<uint4*>(dst);
+        for (int64_t c = threadIdx.x; c < H / PER; c += 256) d4[c] = s4[c];
+    } else {
+        for (int64_t c = threadIdx.x; c < H; c += 256) dst[c] = src[c];
+    }
 }
 
-// One workgroup of 512 threads per row; 8 elements (16 B for 16-bit types) per thread per pass, so a
-// 32000-wide row is 8 passes of independent loads.  Lowest index wins ties; NaNs never win.
+// One workgroup of 512 threads per row; 8 elements (16 B for 16-bit types) per thread per pass.  The loads of 8 passes
+// (32768 elements, a whole 32000-wide row) are issued raw before the first compare, so the row costs one memory round
+// trip instead of one per pass.  Lowest index wins ties; NaNs never win.
 template <typename T>
 __global__ __launch_bounds__(512) void argmax_kernel(const T* __restrict__ logits, int64_t ld, int64_t V,
                                                      int64_t* __restrict__ out) {
+    constexpr int PASSES = 8;
     __shared__ float best_v[8];
     __shared__ int64_t best_i[8];
     const int64_t r = blockIdx.x;
@@ -32,13 +42,20 @@ __global__ __launch_bounds__(512) void argmax_kernel(const T* __restrict__ logit
     const bool vec_ok = (V % 8) == 0 && (ld % 8) == 0 && (reinterpret_cast<uintptr_t>(logits) & 15u) == 0;
     float bv = -INFINITY;
     int64_t bi = V;   // larger than any valid index: "nothing yet"
-    for (int64_t c0 = (int64_t)threadIdx.x * 8; c0 < V; c0 += 512 * 8) {
-        float v[8];
-        mmf_load8<T>(row, c0, V, vec_ok, v);
+    for (int64_t base = (int64_t)threadIdx.x * 8; base < V; base += (int64_t)PASSES * 512 * 8) {
+        Raw8<T> raw[PASSES];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int64_t c = c0 + i;
-            if (c < V && (v[i] > bv || (bi == V && v[i] == v[i]))) { bv = v[i]; bi = c; }   // ascending c: first max kept
+        for (int p = 0; p < PASSES; ++p) raw[p] = mmf_load8_raw<T>(row, base + (int64_t)p * 512 * 8, V, vec_ok);
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) {
+            const int64_t c0 = base + (int64_t)p * 512 * 8;
+            float v[8];
+            mmf_unpack8<T>(raw[p], v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int64_t c = c0 + i;
+                if (c < V && (v[i] > bv || (bi == V && v[i] == v[i]))) { bv = v[i]; bi = c; }   // ascending c: first max kept
+            }
         }
     }
     for (int o = 32; o > 0; o >>= 1) {

@@ -326,6 +326,18 @@ def test_embedding_and_argmax(dev):
     for r in range(2, 5):
         row = logits[r].float()
         assert am[r].item() == int((row == row.max()).nonzero()[0])
+    # ragged and wide rows (element path, more than one 32768-element sweep), fp32 / fp16 tables, NaNs never win
+    for dtype, v, h in ((torch.float32, 70001, 36), (torch.float16, 32768 + 8, 72), (torch.bfloat16, 301, 7)):
+        table = torch.randn(50, h).to(dtype)
+        ids = torch.randint(0, 50, (2, 3))
+        assert torch.equal(F().embedding(table.to(dev), ids.to(dev)).cpu(), table[ids])
+        logits = torch.randn(3, v).to(dtype)
+        logits[0, v - 1] = 60.0                     # the last element of the row wins
+        logits[1, 5] = float("nan")
+        logits[2, :] = float("nan")                 # nothing comparable: index 0
+        am = F().argmax(logits.to(dev)).cpu()
+        row1 = logits[1].float().nan_to_num(nan=-float("inf"))
+        assert am.tolist() == [v - 1, int(row1.argmax()), 0], (dtype, v, am.tolist())
 
 
 @pytest.mark.parametrize("m", [5, 300])
