@@ -316,12 +316,18 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
         last-position logits only and decode runs the captured whole-step HIP graph of DecodeEngine when
         use_graph is set (sampling draws from the graph's logits and feeds the drawn token back; the logits are
         bit-identical to the module path's, so a seeded generator gives the same tokens either way). Rows that
-        have produced eos_token_id are filled with pad_token_id (eos_token_id when not given).
+        have produced eos_token_id (default: the generation config's) are filled with pad_token_id (eos_token_id
+        when not given); generation ends early once every row has.
 
         Any further keyword (num_beams, repetition_penalty, logits_processor, stopping_criteria, streamer,
         generation_config, top_k, return_dict_in_generate, ...) sends the whole call to
         transformers' GenerationMixin.generate, which steps the module path through
         prepare_inputs_for_generation and the RecurrentCache."""
+        gen_cfg = getattr(self, "generation_config", None)
+        if eos_token_id is None and gen_cfg is not None:
+            eos_token_id = gen_cfg.eos_token_id          # as GenerationMixin does: the model's own end-of-sequence id
+            if pad_token_id is None:
+                pad_token_id = gen_cfg.pad_token_id
         if kwargs or input_ids is None or not isinstance(eos_token_id, (int, type(None))):
             hf = dict(kwargs)
             for name, value, default in (("attention_mask", attention_mask, None), ("max_new_tokens", max_new_tokens, None),
