@@ -185,6 +185,29 @@ int mmf_embedding(const void* table, const int64_t* ids, void* out, int64_t rows
                   int dtype, void* stream);
 int mmf_argmax(const void* logits, int64_t ld, int64_t rows, int64_t V, int64_t* out, int dtype, void* stream);
 
+/* ---- all layers of one batch-1 decode step in one persistent launch ---------------------------
+ * mmf_decode_layers replaces, for one token, the loop over HGRNBitBlock.forward in HGRNBitModel.forward
+ *   (mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py:236-262, the block at :97-109, the attention at
+ *   mmfreelm/layers/hgrn_bit.py:83-162): embedding row of *tok -> n_layers x [block norm, i/f/g BitLinear, gate math +
+ *   recurrence step, gated norm, o_proj BitLinear, residual + norm, gate_proj BitLinear, swiglu, down_proj BitLinear +
+ *   residual] -> h_out [H] (the input of the final norm + lm_head).  Same arithmetic, operation for operation, as the
+ *   chain of mmf_bitlinear_gemv_fused launches it stands for.
+ *   256 workgroups stay resident and hand activations to each other as 32-bit words (16-bit value | 16-bit tag of the
+ *   producing link), so the device must have at least 256 CUs free for the launch (fewer CUs: MMF_ERR_ARG).
+ *   phases: device array of 4 * n_layers records of mmf_decode_layers_phase_bytes() bytes each, in the order i/f/g, o,
+ *     gate, down: { const void* w1; const void* norm_w; const void* packed; const float* wdeq; const float* lower_bound;
+ *     float* state; double inv_K; float eps; float eps1; int K; int N; int seg_rows; int pad; } (w1: weight of the norm
+ *     in front of the BitLinear, null for down; norm weights in the activation dtype; inv_K = 1.0 / K).
+ *   h0, h1 [H], o, g [D], attn, res [H], z [I]: uint32 scratch words, zero-initialised once, owned by the caller and
+ *     reused by every call; epoch: one uint32, zero-initialised once, advanced by the kernel; err: one int, set to 1
+ *     if a wait ran out of its `spin` polling rounds (results are then invalid; the launch still terminates).
+ *   Requires D == H, H, I multiples of 128, H <= 2048, I <= 6144, 16-bit activations (dtype 1 or 2), batch 1.
+ *   Calls on one device must not overlap (they share the scratch words). */
+int mmf_decode_layers_phase_bytes(void);
+int mmf_decode_layers(const void* phases, int n_layers, const void* table, const int64_t* tok, int64_t vocab,
+                      uint32_t* h0, uint32_t* h1, uint32_t* o, uint32_t* g, uint32_t* attn, uint32_t* res, uint32_t* z,
+                      void* h_out, uint32_t* epoch, int* err, int H, int D, int I, int spin, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

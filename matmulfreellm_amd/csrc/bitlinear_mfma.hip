@@ -49,7 +49,7 @@ struct MfmaArgs {
 template <typename T>
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
     const T ta = mmf_from_float<T>(a), tb = mmf_from_float<T>(b);
-    return (uint32_t)(*reinterpret_cast<const uint16_t*>(&ta)) | ((uint32_t)(*reinterpret_cast<const uint16_t*>(&tb)) << 16);
+    return (uint32_t)mmf_bits16(ta) | ((uint32_t)mmf_bits16(tb) << 16);
 }
 
 // Epilogue of the tiled kernels.  The MFMAs are issued with the weights as the first operand,
@@ -140,13 +140,12 @@ __device__ __forceinline__ void mfma_epilogue(const MfmaArgs& p, v16i (&acc)[WM]
                     uint4 v = *reinterpret_cast<const uint4*>(stage + row * RS + cc * 16);
                     if (addend) {
                         const uint4 av = *reinterpret_cast<const uint4*>(addend + mr * p.ldo + n);
-                        const T* pe = reinterpret_cast<const T*>(&v);
-                        const T* ae = reinterpret_cast<const T*>(&av);
-                        uint4 ov;
-                        T* oe = reinterpret_cast<T*>(&ov);
+                        T pe[16 / E], ae[16 / E], oe[16 / E];
+                        __builtin_memcpy(pe, &v, 16);
+                        __builtin_memcpy(ae, &av, 16);
 #pragma unroll
                         for (int e = 0; e < 16 / E; ++e) oe[e] = mmf_from_float<T>(__fadd_rn(mmf_to_float(pe[e]), mmf_to_float(ae[e])));
-                        v = ov;
+                        __builtin_memcpy(&v, oe, 16);
                     }
                     *reinterpret_cast<uint4*>(out + mr * p.ldo + n) = v;
                 }
@@ -203,13 +202,12 @@ __device__ __forceinline__ void mfma_epilogue_fast(const MfmaArgs& p, v16i (&acc
                 uint4 v = *reinterpret_cast<const uint4*>(rd + r0 * RS);
                 if (addend) {
                     const uint4 av = *reinterpret_cast<const uint4*>(addend + off);
-                    const T* pe = reinterpret_cast<const T*>(&v);
-                    const T* ae = reinterpret_cast<const T*>(&av);
-                    uint4 ov;
-                    T* oe = reinterpret_cast<T*>(&ov);
+                    T pe[16 / E], ae[16 / E], oe[16 / E];
+                    __builtin_memcpy(pe, &v, 16);
+                    __builtin_memcpy(ae, &av, 16);
 #pragma unroll
                     for (int e = 0; e < 16 / E; ++e) oe[e] = mmf_from_float<T>(__fadd_rn(mmf_to_float(pe[e]), mmf_to_float(ae[e])));
-                    v = ov;
+                    __builtin_memcpy(&v, oe, 16);
                 }
                 *reinterpret_cast<uint4*>(out + off) = v;
             }

@@ -53,13 +53,13 @@ __device__ __forceinline__ void buf_store(float v, __amdgpu_buffer_rsrc_t r, uin
         __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, voff, soff, 0);
     } else {
         T t = mmf_from_float<T>(v);
-        __builtin_amdgcn_raw_buffer_store_b16(*reinterpret_cast<uint16_t*>(&t), r, voff, soff, 0);
+        __builtin_amdgcn_raw_buffer_store_b16(mmf_bits16(t), r, voff, soff, 0);
     }
 }
 template <typename T, typename R>
 __device__ __forceinline__ float raw_get(R v) {
     if constexpr (sizeof(T) == 4) return v;
-    else { T t; *reinterpret_cast<uint16_t*>(&t) = (uint16_t)v; return mmf_to_float(t); }
+    else return mmf_to_float(mmf_from_bits16<T>((uint16_t)v));
 }
 
 // Compile-time loop: the body sees its index as a constant from the front end on, so the

@@ -36,7 +36,17 @@ __device__ __forceinline__ float mmf_to_float(f16_t x) { return (float)x.v; }
 __device__ __forceinline__ uint16_t mmf_f32_to_bf16_bits(float f) {
     // round to nearest even; gfx950 has a hardware convert (v_cvt_pk_bf16_f32) the compiler selects
     const __bf16 b = (__bf16)f;
-    return *reinterpret_cast<const uint16_t*>(&b);
+    return __builtin_bit_cast(uint16_t, b);
+}
+
+// The 16 bits of a bf16_t / f16_t value and back (no pointer punning: _Float16 and uint16_t do not alias).
+template <typename T> __device__ __forceinline__ uint16_t mmf_bits16(T t) {
+    static_assert(sizeof(T) == 2, "16-bit types only");
+    return __builtin_bit_cast(uint16_t, t);
+}
+template <typename T> __device__ __forceinline__ T mmf_from_bits16(uint16_t b) {
+    static_assert(sizeof(T) == 2, "16-bit types only");
+    return __builtin_bit_cast(T, b);
 }
 
 template <typename T> __device__ __forceinline__ T mmf_from_float(float f);
@@ -63,8 +73,9 @@ __device__ __forceinline__ void mmf_load8(const T* __restrict__ p, int64_t k0, i
             out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
             out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
         } else {
-            uint4 a = *reinterpret_cast<const uint4*>(p + k0);
-            const T* e = reinterpret_cast<const T*>(&a);
+            const uint4 a = *reinterpret_cast<const uint4*>(p + k0);
+            T e[8];
+            __builtin_memcpy(e, &a, 16);
 #pragma unroll
             for (int i = 0; i < 8; ++i) out[i] = mmf_to_float(e[i]);
         }
@@ -161,9 +172,10 @@ __device__ __forceinline__ void mmf_store8(T* __restrict__ p, int64_t k0, int64_
             q[1] = make_float4(in[4], in[5], in[6], in[7]);
         } else {
             uint4 a;
-            T* e = reinterpret_cast<T*>(&a);
+            T e[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) e[i] = mmf_from_float<T>(in[i]);
+            __builtin_memcpy(&a, e, 16);
             *reinterpret_cast<uint4*>(p + k0) = a;
         }
     } else {

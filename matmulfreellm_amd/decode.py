@@ -1,5 +1,8 @@
 """Whole-model single-token decode step as one HIP graph.
 
+At batch 1 the 4L fused BitLinears of the layers run as ONE persistent launch (mmf_decode_layers: resident
+workgroups hand activations to each other as tagged words), followed by the lm_head launch and the argmax.
+
 The module path (HGRNBitForCausalLM.forward with T = 1) issues the same kernels through
 nn.Module calls and fresh output tensors; at batch 1 that host work dwarfs the ~40 us the
 weights take to stream.  DecodeEngine lays the step out once over static buffers, records it
@@ -12,6 +15,8 @@ embedding reads, so consecutive steps need no host round trip.
 Every launch is the same C-ABI call with the same arithmetic as the module path, so the two
 produce identical bits (tests/test_gpu_model.py checks that).
 """
+import ctypes
+import warnings
 from typing import List, Optional
 
 import torch
@@ -20,19 +25,28 @@ from . import _lib as L
 from . import functional as F_
 
 
+class _Phase(ctypes.Structure):
+    """One fused BitLinear of mmf_decode_layers' device table (include/mmf.h)."""
+    _fields_ = [("w1", ctypes.c_void_p), ("norm_w", ctypes.c_void_p), ("packed", ctypes.c_void_p), ("wdeq", ctypes.c_void_p),
+                ("lb", ctypes.c_void_p), ("state", ctypes.c_void_p), ("inv_K", ctypes.c_double), ("eps", ctypes.c_float),
+                ("eps1", ctypes.c_float), ("K", ctypes.c_int), ("N", ctypes.c_int), ("seg_rows", ctypes.c_int),
+                ("pad", ctypes.c_int)]
+
+
 class DecodeEngine:
+    SPIN = 1 << 15      # polling rounds a resident workgroup waits for its input before it gives up (mmf_decode_layers)
 
     @classmethod
-    def for_model(cls, model, batch_size: int, use_graph: bool = True, fuse: bool = True):
+    def for_model(cls, model, batch_size: int, use_graph: bool = True, fuse: bool = True, resident: Optional[bool] = None):
         engines = model.__dict__.setdefault("_decode_engines", {})
-        key = (batch_size, use_graph, fuse)
+        key = (batch_size, use_graph, fuse, resident)
         eng = engines.get(key)
         if eng is None or eng.stale():
-            eng = cls(model, batch_size, use_graph, fuse)
+            eng = cls(model, batch_size, use_graph, fuse, resident)
             engines[key] = eng
         return eng
 
-    def __init__(self, model, batch_size: int, use_graph: bool = True, fuse: bool = True):
+    def __init__(self, model, batch_size: int, use_graph: bool = True, fuse: bool = True, resident: Optional[bool] = None):
         cfg = model.config
         self.lib = L.load()
         self.model = model
@@ -98,6 +112,12 @@ class DecodeEngine:
         self.gemv = B <= F_.GEMV_MAX_M
         self.fused = fuse and self._can_fuse()
         self.fused_mfma = fuse and self._can_fuse_mfma()
+        # resident=None: the one-launch layer chain whenever the model fits it; True insists; False never
+        self.resident = self.fused and resident is not False and self._can_run_resident()
+        if resident and not self.resident:
+            raise L.MMFError("DecodeEngine: this model / batch / device does not fit the resident layer chain")
+        if self.resident:
+            self._build_resident()
         self.graph = None
 
     @staticmethod
@@ -139,6 +159,58 @@ class DecodeEngine:
             pro, epi, x.data_ptr(), ldx, L.ptr(aux), ldaux, L.ptr(res_out), L.ptr(w1), eps1, nw.data_ptr(), eps,
             pw.packed.data_ptr(), pw.wdeq.data_ptr(), pw.seg_rows, None, L.ptr(addend), out.data_ptr(), L.ptr(g_out),
             L.ptr(lb), L.ptr(state), self.B, k, n, self.dt_id, L.dtype_id(nw.dtype), L.stream()), "mmf_bitlinear_gemv_fused")
+
+    # ------------------------------------------------------------------ resident layer chain (batch 1)
+    def _can_run_resident(self):
+        props = torch.cuda.get_device_properties(self.dev)
+        return (self.B == 1 and self.dtype in (torch.bfloat16, torch.float16) and self.final_norm.dtype == self.dtype
+                and self.D == self.H and self.H % 128 == 0 and self.I % 128 == 0 and self.H <= 2048 and self.I <= 6144
+                and props.multi_processor_count >= 256)
+
+    def _build_resident(self):
+        H, D, I = self.H, self.D, self.I
+        assert self.lib.mmf_decode_layers_phase_bytes() == ctypes.sizeof(_Phase)
+        table = (_Phase * (4 * self.L))()
+
+        def fill(rec, w1, eps1, pw_nw_eps, k, n, lb=None, state=None):
+            pw, nw, eps = pw_nw_eps
+            rec.w1 = w1.data_ptr() if w1 is not None else None
+            rec.norm_w, rec.packed, rec.wdeq = nw.data_ptr(), pw.packed.data_ptr(), pw.wdeq.data_ptr()
+            rec.lb = lb.data_ptr() if lb is not None else None
+            rec.state = state.data_ptr() if state is not None else None
+            rec.inv_K, rec.eps, rec.eps1, rec.K, rec.N, rec.seg_rows = 1.0 / k, eps, eps1, k, n, pw.seg_rows
+
+        for li, ent in enumerate(self.layers):
+            fill(table[4 * li], ent["attn_norm"], self.eps, (ent["ifg"], ent["projs"][0][1], ent["projs"][0][2]), H, 3 * D,
+                 ent["lb"], ent["state"])
+            fill(table[4 * li + 1], ent["g_norm"], ent["g_eps"], ent["o"], D, H)
+            fill(table[4 * li + 2], ent["mlp_norm"], self.eps, ent["gate"], H, 2 * I)
+            fill(table[4 * li + 3], None, 0.0, ent["down"], I, H)
+        raw = torch.frombuffer(bytearray(bytes(table)), dtype=torch.uint8)
+        self.phases = raw.to(self.dev)
+        sizes = [H, H, D, D, H, H, I]                       # h0, h1, o, g, attn, res, z
+        words = torch.zeros(sum(sizes), dtype=torch.int32, device=self.dev)
+        self.words, off = [], 0
+        for n in sizes:
+            self.words.append(words[off:off + n])
+            off += n
+        self._words = words
+        self.epoch = torch.zeros(1, dtype=torch.int32, device=self.dev)
+        self.err = torch.zeros(1, dtype=torch.int32, device=self.dev)
+
+    def _launch_step_resident(self):
+        lib, s = self.lib, L.stream()
+        w = [t.data_ptr() for t in self.words]
+        L.check(lib.mmf_decode_layers(self.phases.data_ptr(), self.L, self.table.data_ptr(), self.tok.data_ptr(), self.V,
+                                      *w, self.h.data_ptr(), self.epoch.data_ptr(), self.err.data_ptr(), self.H, self.D,
+                                      self.I, self.SPIN, self.dt_id, s), "mmf_decode_layers")
+        self._fused(self.NORM, self.E_PLAIN, self.h, self.H, None, 0, None, self.final_norm, self.eps, self.head, self.logits,
+                    None, None, None, self.V, self.H)
+        L.check(lib.mmf_argmax(self.logits.data_ptr(), self.V, 1, self.V, self.tok.data_ptr(), self.dt_id, s), "mmf_argmax")
+
+    def resident_ok(self) -> bool:
+        """False once a wait inside the resident layer chain ran out of polling rounds (host synchronisation)."""
+        return not self.resident or int(self.err.item()) == 0
 
     def _launch_step_fused(self, ends=True):
         """Batch <= GEMV_MAX_M: four launches per layer, every elementwise op folded into a GEMV.
@@ -228,6 +300,8 @@ class DecodeEngine:
                 and max(self.H, self.D, self.I) <= kmax and self.D % 32 == 0 and self.I % 32 == 0)
 
     def _launch_step(self):
+        if self.resident:
+            return self._launch_step_resident()
         if self.fused:
             return self._launch_step_fused()
         if self.fused_mfma:
@@ -276,6 +350,19 @@ class DecodeEngine:
             self._launch_step()
         torch.cuda.current_stream(self.dev).wait_stream(side)
         torch.cuda.synchronize(self.dev)
+        if self.resident and not self.resident_ok():
+            # the workgroups were not all resident at once (another stream or process holds CUs): use the launch chain
+            warnings.warn("DecodeEngine: the resident layer chain timed out waiting for its workgroups; "
+                          "falling back to one launch per BitLinear")
+            self.resident = False
+            self.err.zero_()
+            for e, sv in zip(self.layers, saved):
+                e["state"].copy_(sv)
+            self.tok.copy_(tok)
+            with torch.cuda.stream(side):
+                self._launch_step()
+            torch.cuda.current_stream(self.dev).wait_stream(side)
+            torch.cuda.synchronize(self.dev)
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             self._launch_step()

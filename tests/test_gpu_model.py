@@ -320,3 +320,35 @@ def test_generation_mixin_beam_search_and_stopping(dev, tiny_bf16):
     assert torch.equal(stopped[0, :15], greedy[0, :15])
     assert bool((stopped[0, 15:] == 0).all())
     assert torch.equal(own[:, :stopped.shape[1]], stopped)
+
+
+@pytest.mark.parametrize("dtype_name", ["bf16", "fp16"])
+def test_resident_layer_chain_equals_the_launch_chain(dev, dtype_name):
+    """Batch 1: all layers in one persistent launch (mmf_decode_layers, activations handed over as tagged words)
+    against the chain of fused BitLinear launches: logits and recurrent states bit for bit on every step, eagerly
+    and graph-replayed, with an intermediate size that needs three passes over the down_proj row; no wait timed out."""
+    from matmulfreellm_amd.decode import DecodeEngine
+    dt = torch.bfloat16 if dtype_name == "bf16" else torch.float16
+    import matmulfreellm_amd as mm
+    torch.manual_seed(31)
+    cfg = mm.HGRNBitConfig(vocab_size=2048, hidden_size=512, num_hidden_layers=3, intermediate_size=4224)
+    model = mm.HGRNBitForCausalLM(cfg).to(device=dev, dtype=dt).eval()
+    ids = torch.randint(0, 2048, (1, 20), device=dev)
+    out = model(input_ids=ids, use_cache=True, logits_to_keep=1)
+    states = [c[-1] for c in out.past_key_values]
+    first = out.logits[:, -1].argmax(-1)
+    for use_graph in (False, True):
+        res = DecodeEngine.for_model(model, 1, use_graph=use_graph, resident=True)
+        ref = DecodeEngine.for_model(model, 1, use_graph=use_graph, resident=False)
+        assert res.resident and not ref.resident
+        res.load_state(states)
+        ref.load_state(states)
+        tok = first.clone()
+        for step in range(7):
+            lr = res.step(tok).clone()
+            lf = ref.step(tok).clone()
+            assert torch.equal(lr, lf), f"logits differ at step {step} (graph={use_graph})"
+            tok = lf.argmax(-1)
+        for a, b in zip(res.export_state(), ref.export_state()):
+            assert torch.equal(a, b)
+        assert res.resident_ok()

@@ -408,3 +408,20 @@ def test_bitlinear_prologue_equals_the_separate_ops(dev, m, k, kind):
             got, res_got = got
             assert torch.equal(res_got, res)
         assert torch.equal(got, want), f"{kind} M={m} K={k} addend={'yes' if add is not None else 'no'}"
+
+
+def test_fp16_outputs_are_rounded_fp32_results(dev):
+    """fp16 outputs at scale (2 M elements per op): every output is the fp32 result of the last operation rounded
+    once more to fp16, as the separately rounded operations of the reference give it -- not the exact product
+    rounded once (what a fused multiply-convert instruction returns; the two differ on about 1 output in 10^5,
+    exactly where the fp32 product lands on an fp16 tie)."""
+    torch.manual_seed(40)
+    x = torch.randn(1024, 2048).half()
+    o = (2 * torch.randn(1024, 2048)).half()
+    w = (1 + 0.1 * torch.randn(2048)).half()
+    y = F().rmsnorm_swishgate(x.to(dev), o.to(dev), w.to(dev), eps=1e-6).cpu()
+    assert torch.equal(y, on.rms_norm_swish_gate_spec(x, o, w, eps=1e-6))
+    y = F().rmsnorm(x.to(dev), w.to(dev), eps=1e-6).cpu()
+    assert torch.equal(y, on.rms_norm_spec(x, w, eps=1e-6))
+    z = F().swiglu(x.to(dev), o.to(dev)).cpu()
+    assert torch.equal(z, on.swiglu_spec(x, o))
