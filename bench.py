@@ -72,14 +72,14 @@ def timed(fn, iters, warmup=2):
     return s.elapsed_time(e) / iters
 
 
-def decode_bench(model, batch, steps, warmup, dev, prompt_len=128):
+def decode_bench(model, batch, steps, warmup, dev, prompt_len=128, resident=None):
     from matmulfreellm_amd.decode import DecodeEngine
     import matmulfreellm_amd.functional as F_
     g = torch.Generator(device=dev).manual_seed(1)
     ids = torch.randint(0, model.config.vocab_size, (batch, prompt_len), generator=g, device=dev)
     out = model(input_ids=ids, use_cache=True, logits_to_keep=1)
     first = F_.argmax(out.logits[:, -1])
-    eng = DecodeEngine.for_model(model, batch, use_graph=True)
+    eng = DecodeEngine.for_model(model, batch, use_graph=True, resident=resident)
     eng.load_state([c[-1] for c in out.past_key_values])
     eng.tok.copy_(first)
     for _ in range(max(warmup, 1)):
@@ -97,25 +97,48 @@ def decode_bench(model, batch, steps, warmup, dev, prompt_len=128):
     return ms, eng
 
 
-# HBM bytes per GEMV launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain copy of
-# known size); see profiles/bitlinear_gemv_decode_bs1_hbm_traffic.txt for the runs and the scale factors.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3629386
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain copy of known size);
+# see profiles/ for the runs and the scale factors.
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3629386          # one fused BitLinear GEMV launch of the launch chain
+LAYERS_TRAFFIC_BYTES_PER_LAUNCH = None           # the resident layer-chain launch
 
 
-def gemv_roofline(eng, iters=20):
-    """Replay a graph that holds exactly the fused BitLinear GEMV launches of one batch-1 decode step (the step
-    without its embedding gather and argmax): 4 per layer + lm_head, each with the model's own packed weights."""
-    assert eng.fused and eng.B == 1
+def _replay_time(launch, iters):
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
-        eng._launch_step_fused(ends=False)
+        launch()
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        eng._launch_step_fused(ends=False)
-    ms = timed(graph.replay, iters)
+        launch()
+    return timed(graph.replay, iters)
+
+
+def gemv_roofline(eng, iters=20):
+    """The dominant kernel of a batch-1 decode step, timed on its own inside a graph.
+
+    Resident engine: the one persistent launch that runs the 4L fused BitLinears of the layers (algorithmic bytes: the
+    layers' packed weights once, plus each link's activations, norm weights and state).  Otherwise: a graph that holds
+    exactly the fused BitLinear GEMV launches of one step (4 per layer + lm_head), averaged per launch."""
+    assert eng.fused and eng.B == 1
+    if eng.resident:
+        def launch():
+            w = [t.data_ptr() for t in eng.words]
+            L_ = __import__("matmulfreellm_amd._lib", fromlist=["x"])
+            L_.check(eng.lib.mmf_decode_layers(eng.phases.data_ptr(), eng.L, eng.table.data_ptr(), eng.tok.data_ptr(), eng.V,
+                                               *w, eng.h.data_ptr(), eng.epoch.data_ptr(), eng.err.data_ptr(), eng.H, eng.D,
+                                               eng.I, eng.SPIN, eng.dt_id, L_.stream()), "mmf_decode_layers")
+        ms = _replay_time(launch, iters)
+        assert eng.resident_ok(), "a wait inside the resident layer chain timed out"
+        total_bytes = eng.fused_step_bytes(head=False)
+        achieved = total_bytes / (ms * 1e-3) / 1e9
+        return {"bound": "hbm", "kernel": "decode_layers_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": LAYERS_TRAFFIC_BYTES_PER_LAUNCH,
+                "launches_per_step": 1, "links_per_launch": 4 * eng.L, "algorithmic_bytes_per_launch": total_bytes,
+                "avg_launch_us": round(ms * 1e3, 3), "us_per_link": round(ms * 1e3 / (4 * eng.L), 3)}
+    ms = _replay_time(lambda: eng._launch_step_fused(ends=False), iters)
     n = 4 * eng.L + 1
     total_bytes = eng.fused_step_bytes()
     us_per_launch = ms * 1e3 / n
@@ -226,6 +249,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--shape", default="1.3B", choices=list(SHAPES))
+    ap.add_argument("--launch-chain", action="store_true",
+                    help="batch 1: one launch per fused BitLinear instead of the resident layer chain")
     ap.add_argument("--no-extra", action="store_true", help="skip the batch-64 / matrix-core / scan / norm / CPU legs")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by)")
@@ -248,7 +273,7 @@ def main():
         dst.copy_(src)          # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
-    ms, eng = decode_bench(model, args.batch, args.steps, args.warmup, dev)
+    ms, eng = decode_bench(model, args.batch, args.steps, args.warmup, dev, resident=False if args.launch_chain else None)
     tok_s = args.batch * 1e3 / ms
     result = {
         "metric": "decode tok/s 1.3B-shape bs=1/64; BitLinear HBM GB/s & int8 MFMA util",
@@ -257,7 +282,9 @@ def main():
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": f"{args.shape}-shape HGRNBit greedy decode, batch {args.batch}, 128-token prompt, "
                                f"{args.steps} timed steps, whole step = one HIP graph",
-                   "batch": args.batch, "ternary_weights": n_tern, "packed_weight_bytes": n_tern // 4},
+                   "batch": args.batch, "ternary_weights": n_tern, "packed_weight_bytes": n_tern // 4,
+                   "decode_path": "resident layer chain + lm_head + argmax (3 launches)" if getattr(eng, "resident", False)
+                   else "one launch per fused BitLinear"},
     }
     hbm_step_us = (n_tern / 4) / (HBM_PEAK_GBS * 1e3)
     result["decode_frac_of_weight_stream_bound"] = round(hbm_step_us / (ms * 1e3), 4)
@@ -265,7 +292,7 @@ def main():
     eng1 = eng
     if args.batch != 1:
         from matmulfreellm_amd.decode import DecodeEngine
-        eng1 = DecodeEngine.for_model(model, 1, use_graph=True)
+        eng1 = DecodeEngine.for_model(model, 1, use_graph=True, resident=False if args.launch_chain else None)
     result["roofline"] = gemv_roofline(eng1)
 
     if not args.no_extra:

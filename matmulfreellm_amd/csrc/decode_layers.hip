@@ -90,30 +90,31 @@ __device__ __forceinline__ void row_load4(const RowSrc& s, int k0, int spin, int
     }
     const uint64_t* p = reinterpret_cast<const uint64_t*>(s.words + k0);
     const uint64_t want = ((uint64_t)s.tag << 32) | s.tag, mask = 0x0000ffff0000ffffull;
-    uint64_t a, b;
+    // two polls in flight: the next pair of loads is issued before the current pair is examined, which halves the
+    // time between a word's arrival and its detection
+    uint64_t a = ll_ld8(p), b = ll_ld8(p + 1);
     int n = 0;
-    bool ok;
-    do {
-        a = ll_ld8(p);
-        b = ll_ld8(p + 1);
-        ok = ((a & mask) == want) && ((b & mask) == want);
-    } while (!ok && ++n < spin);
-    if (!ok) *err = 1;
+    for (;;) {
+        const uint64_t a2 = ll_ld8(p), b2 = ll_ld8(p + 1);
+        if (((a & mask) == want) && ((b & mask) == want)) break;
+        a = a2;
+        b = b2;
+        if (++n >= spin) {
+            if (!(((a & mask) == want) && ((b & mask) == want))) *err = 1;
+            break;
+        }
+    }
     out[0] = word_value<T>((uint32_t)a);
     out[1] = word_value<T>((uint32_t)(a >> 32));
     out[2] = word_value<T>((uint32_t)b);
     out[3] = word_value<T>((uint32_t)(b >> 32));
 }
+// One word whose first read `w` was issued long before (at the start of the phase): usually it already carries the tag.
 template <typename T>
-__device__ __forceinline__ float word_load1(const uint32_t* p, uint32_t tag, int spin, int* err) {
-    uint32_t w;
+__device__ __forceinline__ float word_finish1(uint32_t w, const uint32_t* p, uint32_t tag, int spin, int* err) {
     int n = 0;
-    bool ok;
-    do {
-        w = ll_ld4(p);
-        ok = (w & 0xffffu) == tag;
-    } while (!ok && ++n < spin);
-    if (!ok) *err = 1;
+    while ((w & 0xffffu) != tag && n++ < spin) w = ll_ld4(p);
+    if ((w & 0xffffu) != tag) *err = 1;
     return word_value<T>(w);
 }
 
@@ -179,6 +180,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
     }
     uint4 wreg[NWREG];
     float ep_wdeq[R], ep_lb = 0.0f, ep_state = 0.0f;
+    uint32_t ep_add = 0u;
     auto load_block = [&](int vb) {
         const int nb = vb / S, sub = vb % S;
         if constexpr (S == 1) {
@@ -210,6 +212,9 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
                     if (ph.lb) ep_lb = ph.lb[ch];
                     ep_state = ph.state[ch];
                 }
+            }
+            if constexpr (EPI == EPI_PLAIN) {
+                if (add_words && lane < CHN && ch < Nseg) ep_add = ll_ld4(add_words + ch);   // checked (and re-read if early) in the epilogue
             }
         }
     };
@@ -381,7 +386,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
             }
             if constexpr (EPI == EPI_PLAIN) {
                 float o = res[0];
-                if (add_words) o = __fadd_rn(mmf_round_to<T>(o), word_load1<T>(add_words + ch, add_tag, a.spin, a.err));
+                if (add_words) o = __fadd_rn(mmf_round_to<T>(o), word_finish1<T>(ep_add, add_words + ch, add_tag, a.spin, a.err));
                 ll_st4(out_words + ch, make_word<T>(o, tag_out));
                 if (plain_out) plain_out[ch] = mmf_from_float<T>(o);
             } else if constexpr (EPI == EPI_STEP) {
