@@ -260,6 +260,7 @@ __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
     }
     amax = block_max_once<kGemvWaves>(amax, red_f);
     const float scale = __fdiv_rn(127.0f, fmaxf(amax, 1e-5f));
+    const float deq = __fdiv_rn(1.0f, scale);                 // needed by the epilogue only: computed here, in the shadow of the barriers
     int qs = 0;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
@@ -326,7 +327,6 @@ __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
         int qtot = 0;
 #pragma unroll
         for (int w = 0; w < kGemvWaves; ++w) qtot += red_q[w];
-        const float deq = __fdiv_rn(1.0f, scale);
         float res[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {

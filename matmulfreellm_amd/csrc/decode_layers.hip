@@ -297,6 +297,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
     }
     amax = block_max_once(amax, sm.red_f);
     const float scale = __fdiv_rn(127.0f, fmaxf(amax, 1e-5f));
+    const float deq = __fdiv_rn(1.0f, scale);                 // needed by the epilogue only: computed here, in the shadow of the barriers
     int qs = 0;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
@@ -365,7 +366,6 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
             int qtot = 0;
 #pragma unroll
             for (int w = 0; w < kNW; ++w) qtot += sm.red_q[w];
-            const float deq = __fdiv_rn(1.0f, scale);
             float res[R];
 #pragma unroll
             for (int r = 0; r < R; ++r) {
