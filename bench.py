@@ -99,8 +99,8 @@ def decode_bench(model, batch, steps, warmup, dev, prompt_len=128, resident=None
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain copy of known size);
 # see profiles/ for the runs and the scale factors.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3629386          # one fused BitLinear GEMV launch of the launch chain
-LAYERS_TRAFFIC_BYTES_PER_LAUNCH = None           # the resident layer-chain launch
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3623910          # one fused BitLinear GEMV launch of the launch chain
+LAYERS_TRAFFIC_BYTES_PER_LAUNCH = 330841649         # the resident layer-chain launch
 
 
 def _replay_time(launch, iters):
@@ -132,7 +132,7 @@ def gemv_roofline(eng, iters=20):
                                                eng.I, eng.SPIN, eng.dt_id, L_.stream()), "mmf_decode_layers")
         ms = _replay_time(launch, iters)
         assert eng.resident_ok(), "a wait inside the resident layer chain timed out"
-        total_bytes = eng.fused_step_bytes(head=False)
+        total_bytes = eng.fused_step_bytes(with_head=False)
         achieved = total_bytes / (ms * 1e-3) / 1e9
         return {"bound": "hbm", "kernel": "decode_layers_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": LAYERS_TRAFFIC_BYTES_PER_LAUNCH,

@@ -236,7 +236,7 @@ class DecodeEngine:
             L.check(lib.mmf_argmax(self.logits.data_ptr(), self.V, B, self.V, self.tok.data_ptr(), self.dt_id, s),
                     "mmf_argmax")
 
-    def fused_step_bytes(self, head: bool = True):
+    def fused_step_bytes(self, with_head: bool = True):
         """Algorithmic bytes of the 4L (+1 with head) fused BitLinears of one batch-B step: 2-bit weights once, plus
         each link's activation / norm-weight / state reads and its outputs."""
         B, H, D, I, V, e = self.B, self.H, self.D, self.I, self.V, self.h.element_size()
@@ -246,7 +246,7 @@ class DecodeEngine:
                      + B * (2 * H * e + H * e + I * e) + 2 * H * e          # C: a, h in; res, z out; two norm weights
                      + B * (I * e + 2 * H * e) + I * e)                     # D: z, res in; h out; norm weight
         head = V * H // 4 + B * (H * e + V * e) + 2 * H * e
-        return self.L * per_layer + (head if head else 0)
+        return self.L * per_layer + (head if with_head else 0)
 
     def _qfused(self, pro, x, ldx, aux, ldaux, aux2, ldaux2, res_out, w1, eps1, nw, eps, lb, state, k):
         L.check(self.lib.mmf_rmsnorm_quant_fused(
