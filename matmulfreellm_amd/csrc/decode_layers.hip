@@ -488,6 +488,8 @@ int mmf_decode_layers(const void* phases, int n_layers, const void* table, const
         !epoch || !err || H <= 0 || D <= 0 || I <= 0 || spin <= 0)
         return MMF_ERR_ARG;
     if (H % 128 != 0 || D != H || I % 128 != 0) return MMF_ERR_ARG;      // rows are whole k-blocks: no ragged tail in a phase
+    if (dtype != MMF_BF16 && dtype != MMF_F16) return MMF_ERR_ARG;        // a tagged word carries a 16-bit value
+    if (H > 2048 || I > 6144) return MMF_ERR_WIDE;                        // one pass over an H-wide row, three over an I-wide one
     for (const void* p : {(const void*)h0, (const void*)h1, (const void*)o, (const void*)g, (const void*)attn, (const void*)res,
                           (const void*)z, (const void*)table, (const void*)h_out})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return MMF_ERR_ALIGN;
