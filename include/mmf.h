@@ -201,7 +201,7 @@ int mmf_argmax(const void* logits, int64_t ld, int64_t rows, int64_t V, int64_t*
  *   h0, h1 [H], o, g [D], attn, res [H], z [I]: uint32 scratch words, zero-initialised once, owned by the caller and
  *     reused by every call; epoch: one uint32, zero-initialised once, advanced by the kernel; err: one int, set to 1
  *     if a wait ran out of its `spin` polling rounds (results are then invalid; the launch still terminates).
- *   Requires D == H, H, I multiples of 128, H <= 2048, I <= 6144, 16-bit activations (dtype 1 or 2), batch 1.
+ *   Requires D == H, H, I multiples of 128, H <= 4096, I <= 8192 (else MMF_ERR_WIDE), 16-bit activations (dtype 1 or 2), batch 1.
  *   Calls on one device must not overlap (they share the scratch words). */
 int mmf_decode_layers_phase_bytes(void);
 int mmf_decode_layers(const void* phases, int n_layers, const void* table, const int64_t* tok, int64_t vocab,

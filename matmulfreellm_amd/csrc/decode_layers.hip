@@ -469,6 +469,7 @@ template <typename T>
 int launch_layers(const LayersArgs& a, hipStream_t s) {
     const int nvh = (int)mmf_ceil_div(a.H > a.D ? a.H : a.D, 2048), nvi = (int)mmf_ceil_div(a.I, 2048);
     if (nvh == 1 && nvi <= 3) decode_layers_kernel<T, 1, 3><<<kWGs, kNT, 0, s>>>(a);
+    else if (nvh <= 2 && nvi <= 4) decode_layers_kernel<T, 2, 4><<<kWGs, kNT, 0, s>>>(a);
     else return MMF_ERR_WIDE;
     MMF_CHECK_LAUNCH();
     return 0;
@@ -489,7 +490,7 @@ int mmf_decode_layers(const void* phases, int n_layers, const void* table, const
         return MMF_ERR_ARG;
     if (H % 128 != 0 || D != H || I % 128 != 0) return MMF_ERR_ARG;      // rows are whole k-blocks: no ragged tail in a phase
     if (dtype != MMF_BF16 && dtype != MMF_F16) return MMF_ERR_ARG;        // a tagged word carries a 16-bit value
-    if (H > 2048 || I > 6144) return MMF_ERR_WIDE;                        // one pass over an H-wide row, three over an I-wide one
+    if (H > 4096 || I > 8192) return MMF_ERR_WIDE;                        // at most two passes over an H-wide row, four over an I-wide one
     for (const void* p : {(const void*)h0, (const void*)h1, (const void*)o, (const void*)g, (const void*)attn, (const void*)res,
                           (const void*)z, (const void*)table, (const void*)h_out})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return MMF_ERR_ALIGN;

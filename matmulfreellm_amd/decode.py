@@ -164,7 +164,7 @@ class DecodeEngine:
     def _can_run_resident(self):
         props = torch.cuda.get_device_properties(self.dev)
         return (self.B == 1 and self.dtype in (torch.bfloat16, torch.float16) and self.final_norm.dtype == self.dtype
-                and self.D == self.H and self.H % 128 == 0 and self.I % 128 == 0 and self.H <= 2048 and self.I <= 6144
+                and self.D == self.H and self.H % 128 == 0 and self.I % 128 == 0 and self.H <= 4096 and self.I <= 8192
                 and props.multi_processor_count >= 256)
 
     def _build_resident(self):

@@ -322,16 +322,17 @@ def test_generation_mixin_beam_search_and_stopping(dev, tiny_bf16):
     assert torch.equal(own[:, :stopped.shape[1]], stopped)
 
 
-@pytest.mark.parametrize("dtype_name", ["bf16", "fp16"])
-def test_resident_layer_chain_equals_the_launch_chain(dev, dtype_name):
+@pytest.mark.parametrize("dtype_name,hidden,inter", [("bf16", 512, 4224), ("fp16", 512, 4224), ("bf16", 2304, 6400), ("fp16", 1024, 2816)])
+def test_resident_layer_chain_equals_the_launch_chain(dev, dtype_name, hidden, inter):
     """Batch 1: all layers in one persistent launch (mmf_decode_layers, activations handed over as tagged words)
     against the chain of fused BitLinear launches: logits and recurrent states bit for bit on every step, eagerly
-    and graph-replayed, with an intermediate size that needs three passes over the down_proj row; no wait timed out."""
+    and graph-replayed; widths that need one and two passes over a hidden row, two to four over the down_proj row,
+    8-row and 32-row virtual blocks, more virtual blocks than workgroups; no wait timed out."""
     from matmulfreellm_amd.decode import DecodeEngine
     dt = torch.bfloat16 if dtype_name == "bf16" else torch.float16
     import matmulfreellm_amd as mm
     torch.manual_seed(31)
-    cfg = mm.HGRNBitConfig(vocab_size=2048, hidden_size=512, num_hidden_layers=3, intermediate_size=4224)
+    cfg = mm.HGRNBitConfig(vocab_size=2048, hidden_size=hidden, num_hidden_layers=3, intermediate_size=inter)
     model = mm.HGRNBitForCausalLM(cfg).to(device=dev, dtype=dt).eval()
     ids = torch.randint(0, 2048, (1, 20), device=dev)
     out = model(input_ids=ids, use_cache=True, logits_to_keep=1)

@@ -194,7 +194,7 @@ def test_rejected_shapes_and_pointers_return_their_code_before_any_launch():
                                                                           spin, dtype, None)
     assert layers(512, 256, 1536) == -1 and layers(500, 500, 1536) == -1 and layers(512, 512, 1500) == -1
     assert layers(512, 512, 1536, dtype=0) == -1 and layers(512, 512, 1536, spin=0) == -1
-    assert layers(4096, 4096, 4096) == -2 and layers(2048, 2048, 8192) == -2
+    assert layers(4224, 4224, 4096) == -2 and layers(2048, 2048, 8320) == -2
     assert layers(512, 512, 1536, h0=P + 4) == -3
     assert lib.mmf_decode_layers(None, 2, P, P, 1000, P, P, P, P, P, P, P, P, P, P, 512, 512, 1536, 100, 1, None) == -1
     assert lib.mmf_decode_layers_phase_bytes() == 80
