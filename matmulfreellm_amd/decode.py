@@ -212,6 +212,16 @@ class DecodeEngine:
         """False once a wait inside the resident layer chain ran out of polling rounds (host synchronisation)."""
         return not self.resident or int(self.err.item()) == 0
 
+    def check(self):
+        """Raise if a wait inside the resident layer chain timed out since the engine was built: its workgroups were
+        not all resident at once (other work held CUs), so the steps since then are invalid.  One host synchronisation;
+        callers run it once per generation, not per step."""
+        if not self.resident_ok():
+            self.err.zero_()
+            raise L.MMFError("DecodeEngine: a wait inside the resident layer chain timed out (were other kernels running "
+                             "on this device?); the tokens of this generation are invalid. Build the engine with "
+                             "resident=False to decode with one launch per BitLinear.")
+
     def _launch_step_fused(self, ends=True):
         """Batch <= GEMV_MAX_M: four launches per layer, every elementwise op folded into a GEMV.
         ends=False leaves out the embedding gather and the argmax (the 4L+1 GEMV launches only)."""
@@ -409,4 +419,5 @@ class DecodeEngine:
         for t in range(n_steps):
             self.advance()
             out[t].copy_(self.tok)
+        self.check()
         return out.t().contiguous()

@@ -367,6 +367,8 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
                 out = self(input_ids=nxt.view(B, 1), past_key_values=cache, use_cache=True)
                 cache = out.past_key_values
                 logits = out.logits[:, -1, :]
+        if engine is not None:
+            engine.check()
         return torch.cat(tokens, dim=1)
 
 

@@ -353,3 +353,37 @@ def test_resident_layer_chain_equals_the_launch_chain(dev, dtype_name, hidden, i
         for a, b in zip(res.export_state(), ref.export_state()):
             assert torch.equal(a, b)
         assert res.resident_ok()
+
+
+def test_resident_layer_chain_timeout_is_reported_and_recoverable(dev, tiny_bf16):
+    """A wait that runs out of polling rounds (forced from the host with a one-round limit) must not hang: the launch
+    drains, the error word is raised, DecodeEngine.check() reports it, and with the normal limit the same engine
+    reproduces the launch chain again."""
+    import matmulfreellm_amd._lib as L_
+    from matmulfreellm_amd.decode import DecodeEngine
+    model = build(tiny_bf16, torch.bfloat16, dev)
+    torch.manual_seed(33)
+    ids = torch.randint(0, V, (1, 12), device=dev)
+    out = model(input_ids=ids, use_cache=True, logits_to_keep=1)
+    states = [c[-1] for c in out.past_key_values]
+    tok = out.logits[:, -1].argmax(-1)
+    eng = DecodeEngine(model, 1, use_graph=False, resident=True)
+    ref = DecodeEngine(model, 1, use_graph=False, resident=False)
+    eng.SPIN = 1
+    eng.load_state(states)
+    for _ in range(3):
+        eng.step(tok)
+    torch.cuda.synchronize()
+    assert not eng.resident_ok()
+    with pytest.raises(L_.MMFError):
+        eng.check()
+    eng.SPIN = DecodeEngine.SPIN
+    assert eng.resident_ok()                      # check() cleared the error word
+    eng.load_state(states)
+    ref.load_state(states)
+    for _ in range(3):
+        a = eng.step(tok).clone()
+        b = ref.step(tok).clone()
+        assert torch.equal(a, b)
+        tok = b.argmax(-1)
+    eng.check()
