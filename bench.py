@@ -124,12 +124,7 @@ def gemv_roofline(eng, iters=20):
     exactly the fused BitLinear GEMV launches of one step (4 per layer + lm_head), averaged per launch."""
     assert eng.fused and eng.B == 1
     if eng.resident:
-        def launch():
-            w = [t.data_ptr() for t in eng.words]
-            L_ = __import__("matmulfreellm_amd._lib", fromlist=["x"])
-            L_.check(eng.lib.mmf_decode_layers(eng.phases.data_ptr(), eng.L, eng.table.data_ptr(), eng.tok.data_ptr(), eng.V,
-                                               *w, eng.h.data_ptr(), eng.epoch.data_ptr(), eng.err.data_ptr(), eng.H, eng.D,
-                                               eng.I, eng.SPIN, eng.dt_id, L_.stream()), "mmf_decode_layers")
+        launch = lambda: eng._launch_layers(False)
         ms = _replay_time(launch, iters)
         assert eng.resident_ok(), "a wait inside the resident layer chain timed out"
         total_bytes = eng.fused_step_bytes(with_head=False)
@@ -283,7 +278,8 @@ def main():
         "config": {"workload": f"{args.shape}-shape HGRNBit greedy decode, batch {args.batch}, 128-token prompt, "
                                f"{args.steps} timed steps, whole step = one HIP graph",
                    "batch": args.batch, "ternary_weights": n_tern, "packed_weight_bytes": n_tern // 4,
-                   "decode_path": "resident layer chain + lm_head + argmax (3 launches)" if getattr(eng, "resident", False)
+                   "decode_path": ("one resident launch (embedding row, layers, lm_head, argmax)" if eng.head_inside
+                                   else "resident layer chain + lm_head + argmax (3 launches)") if getattr(eng, "resident", False)
                    else "one launch per fused BitLinear"},
     }
     hbm_step_us = (n_tern / 4) / (HBM_PEAK_GBS * 1e3)

@@ -201,12 +201,17 @@ int mmf_argmax(const void* logits, int64_t ld, int64_t rows, int64_t V, int64_t*
  *   h0, h1 [H], o, g [D], attn, res [H], z [I]: uint32 scratch words, zero-initialised once, owned by the caller and
  *     reused by every call; epoch: one uint32, zero-initialised once, advanced by the kernel; err: one int, set to 1
  *     if a wait ran out of its `spin` polling rounds (results are then invalid; the launch still terminates).
+ *   head: null, or a device record like the ones of `phases` for the final norm + lm_head (w1 = final norm weight,
+ *     K = H, N = vocabulary size); the launch then also writes the logits [N] (activation dtype), and the greedy token
+ *     (lowest index of the largest logit; NaNs never win) to *tok_out, which may be the buffer `tok` points to.
+ *     am_words: 256 uint64 scratch words, zero-initialised once.  With head == null the three pointers are ignored.
  *   Requires D == H, H, I multiples of 128, H <= 4096, I <= 8192 (else MMF_ERR_WIDE), 16-bit activations (dtype 1 or 2), batch 1.
  *   Calls on one device must not overlap (they share the scratch words). */
 int mmf_decode_layers_phase_bytes(void);
 int mmf_decode_layers(const void* phases, int n_layers, const void* table, const int64_t* tok, int64_t vocab,
                       uint32_t* h0, uint32_t* h1, uint32_t* o, uint32_t* g, uint32_t* attn, uint32_t* res, uint32_t* z,
-                      void* h_out, uint32_t* epoch, int* err, int H, int D, int I, int spin, int dtype, void* stream);
+                      void* h_out, const void* head, void* logits, uint64_t* am_words, int64_t* tok_out, uint32_t* epoch, int* err,
+                      int H, int D, int I, int spin, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

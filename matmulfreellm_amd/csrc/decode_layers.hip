@@ -48,6 +48,10 @@ struct LayersArgs {
     uint32_t* rb;             //   summed residual [H]
     uint32_t* zb;             //   swiglu output [I]
     void* h_out;              // plain copy of the final residual stream [H]
+    const Phase* head;        // final norm + lm_head (device record) or null: stop after the layers
+    void* logits;             // head: plain logits [V]
+    uint64_t* am_words;       // head: one (index | value | tag) record per workgroup
+    int64_t* tok_out;         // head: the greedy token
     uint32_t* epoch;          // tag base; advanced by 4 * n_layers at the end of the launch
     int* err;                 // set to 1 when a poll ran out of rounds
     int n_layers, H, D, I, spin;
@@ -59,6 +63,16 @@ struct RowSrc {
     const uint32_t* words;
     uint32_t tag;
 };
+
+// Running greedy choice of one epilogue lane: lowest index of the largest value seen; NaNs never win.
+struct Best {
+    float v;
+    uint32_t i;               // 0xffffffff: nothing yet
+};
+constexpr uint32_t kNone = 0xffffffffu;
+__device__ __forceinline__ void best_take(Best& b, float v, uint32_t i) {
+    if (i != kNone && (b.i == kNone || v > b.v || (v == b.v && i < b.i))) { b.v = v; b.i = i; }
+}
 
 struct Smem {
     int8_t q[4 * kNT * kEl];                  // int8 codes of the row (K <= 8192)
@@ -145,10 +159,12 @@ __device__ __forceinline__ float block_max_once(float v, float* slot) {
 // One phase.  NV passes over the row (K <= NV * 2048); S = 4: a virtual block owns 8 of an n-block's 32 rows.
 // Virtual block vb -> (n-block vb / S, row group vb % S); a workgroup takes vb = blockIdx.x, + gridDim.x, ...
 // The prologue (the row's int8 codes) is computed once per workgroup, whatever the number of virtual blocks.
-template <typename T, int NV, int PRO, int EPI, int S>
+// PF: the workgroup walks several virtual blocks (the lm_head link): request the next block's weights as soon as the
+// dot of the current one has consumed its registers, so they travel under the epilogue.
+template <typename T, int NV, int PRO, int EPI, int S, bool PF = false>
 __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, Smem& sm, const RowSrc& xs, const RowSrc& auxs,
                                           const uint32_t* add_words, uint32_t add_tag, uint32_t* res_words,
-                                          uint32_t* out_words, uint32_t* g_words, T* plain_out, uint32_t tag_out) {
+                                          uint32_t* out_words, uint32_t* g_words, T* plain_out, uint32_t tag_out, Best* am = nullptr) {
     constexpr int R = EPI == EPI_STEP ? 3 : EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int BPW = 2 * NV;
     constexpr int GMAX = NV * kNW / 2;
@@ -178,10 +194,9 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
         if constexpr (HAS_W1) w1raw[v] = raw4_load<T, true>(w1, k0, K);
         nwraw[v] = raw4_load<T, true>(nw, k0, K);
     }
-    uint4 wreg[NWREG];
     float ep_wdeq[R], ep_lb = 0.0f, ep_state = 0.0f;
     uint32_t ep_add = 0u;
-    auto load_block = [&](int vb) {
+    auto load_weights = [&](int vb, uint4 (&wreg)[NWREG]) {
         const int nb = vb / S, sub = vb % S;
         if constexpr (S == 1) {
 #pragma unroll
@@ -203,6 +218,9 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
                 }
             }
         }
+    };
+    auto load_ep = [&](int vb) {
+        const int nb = vb / S, sub = vb % S;
         if (wave == 0) {
 #pragma unroll
             for (int r = 0; r < R; ++r) ep_wdeq[r] = ph.wdeq[(uint32_t)((nb + r * NBseg) * 32) / (uint32_t)ph.seg_rows];
@@ -218,7 +236,14 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
             }
         }
     };
-    load_block((int)blockIdx.x);
+    // PF: the weights of this workgroup's first four virtual blocks are requested now, together (one block in
+    // flight at a time would stream them at a fraction of the CU's share of the bandwidth)
+    constexpr int NPF = PF ? 4 : 1;
+    uint4 wpf[NPF][NWREG];
+#pragma unroll
+    for (int j = 0; j < NPF; ++j)
+        if ((int)blockIdx.x + j * (int)gridDim.x < nvb) load_weights((int)blockIdx.x + j * (int)gridDim.x, wpf[j]);
+    load_ep((int)blockIdx.x);
 
     // ---- the row (and the prologue's second operand): poll until every word carries the producer's tag
     float xv[NV][4], av[HAS_AUX ? NV : 1][4];
@@ -330,8 +355,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
         return acc;
     };
 
-    for (int vb = (int)blockIdx.x; vb < nvb; vb += (int)gridDim.x) {
-        if (vb != (int)blockIdx.x) load_block(vb);
+    auto process = [&](int vb, const uint4 (&wreg)[NWREG]) {
         const int nb = vb / S, sub = vb % S;
         if constexpr (S == 1) {
             int acc[R];
@@ -387,8 +411,12 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
             if constexpr (EPI == EPI_PLAIN) {
                 float o = res[0];
                 if (add_words) o = __fadd_rn(mmf_round_to<T>(o), word_finish1<T>(ep_add, add_words + ch, add_tag, a.spin, a.err));
-                ll_st4(out_words + ch, make_word<T>(o, tag_out));
+                if (out_words) ll_st4(out_words + ch, make_word<T>(o, tag_out));
                 if (plain_out) plain_out[ch] = mmf_from_float<T>(o);
+                if (am) {
+                    const float ov = mmf_round_to<T>(o);
+                    if (ov == ov) best_take(*am, ov, (uint32_t)ch);
+                }
             } else if constexpr (EPI == EPI_STEP) {
                 const float iv = mmf_round_to<T>(res[0]), fv = mmf_round_to<T>(res[1]);
                 float s = mmf_sigmoid(fv);
@@ -405,6 +433,19 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
             }
         }
         __syncthreads();                                        // part[] and the wave-0 registers are reused by the next block
+    };
+#pragma unroll
+    for (int j = 0; j < NPF; ++j) {
+        const int vb = (int)blockIdx.x + j * (int)gridDim.x;
+        if (vb < nvb) {
+            if (j > 0) load_ep(vb);
+            process(vb, wpf[j]);
+        }
+    }
+    for (int vb = (int)blockIdx.x + NPF * (int)gridDim.x; vb < nvb; vb += (int)gridDim.x) {
+        load_weights(vb, wpf[0]);
+        load_ep(vb);
+        process(vb, wpf[0]);
     }
 }
 
@@ -460,9 +501,56 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
                 run_phase<T, NVI, PRO_PLAIN, EPI_PLAIN, 1>(p, a, sm, z_in, none, a.rb, tag_of(4 * l + 2), nullptr, a.hb[l & 1], nullptr, plain, tag_of(4 * l + 3));
         }
     }
-    // Every workgroup read the tag base before any workgroup could get here (the last phase's inputs depend,
-    // through the chain, on an output of every workgroup), so the next launch's base can be published now.
-    if (blockIdx.x == 0 && threadIdx.x == 0) *a.epoch = e + 4u * (uint32_t)a.n_layers;
+    if (a.head) {
+        // final norm -> lm_head: plain logits, and this workgroup's candidate for the greedy token
+        const int L = a.n_layers;
+        const Phase p = *a.head;
+        const RowSrc h_last{nullptr, a.hb[(L - 1) & 1], tag_of(4 * (L - 1) + 3)}, none{nullptr, nullptr, 0u};
+        const uint32_t tag_h = tag_of(4 * L);
+        Best best{0.0f, kNone};
+        run_phase<T, NVH, PRO_NORM, EPI_PLAIN, 1, true>(p, a, sm, h_last, none, nullptr, 0u, nullptr, nullptr, nullptr,
+                                                  static_cast<T*>(a.logits), tag_h, &best);
+        const int lane = threadIdx.x & 63;
+        if (threadIdx.x < 64) {                                  // wave 0 holds the candidates of its 32 epilogue lanes
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float ov = __shfl_xor(best.v, o, 64);
+                const uint32_t oi = (uint32_t)__shfl_xor((int)best.i, o, 64);
+                best_take(best, ov, oi);
+            }
+            if (lane == 0)
+                ll_st8(a.am_words + blockIdx.x, ((uint64_t)best.i << 32) | (uint64_t)make_word<T>(best.i == kNone ? 0.0f : best.v, tag_h));
+        }
+        if (blockIdx.x == 0) {
+            // the greedy token: lowest index of the largest logit over the workgroups' candidates
+            __syncthreads();                                    // run_phase is done with the shared arrays
+            Best b{0.0f, kNone};
+            if (threadIdx.x < gridDim.x) {
+                uint64_t w;
+                int n = 0;
+                do { w = ll_ld8(a.am_words + threadIdx.x); } while (((uint32_t)w & 0xffffu) != tag_h && ++n < a.spin);
+                if (((uint32_t)w & 0xffffu) != tag_h) *a.err = 1;
+                b.i = (uint32_t)(w >> 32);
+                b.v = word_value<T>((uint32_t)w);
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float ov = __shfl_xor(b.v, o, 64);
+                const uint32_t oi = (uint32_t)__shfl_xor((int)b.i, o, 64);
+                best_take(b, ov, oi);
+            }
+            if (lane == 0) { sm.red_f[threadIdx.x >> 6] = b.v; sm.red_q[threadIdx.x >> 6] = (int)b.i; }
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                for (int w = 1; w < kNW; ++w) best_take(b, sm.red_f[w], (uint32_t)sm.red_q[w]);
+                *a.tok_out = b.i == kNone ? 0 : (int64_t)b.i;
+            }
+        }
+    }
+    // Every workgroup read the tag base (and the token) before any workgroup could get here (the last link's inputs
+    // depend, through the chain, on an output of every workgroup that takes part), so the next launch's base can be
+    // published now.
+    if (blockIdx.x == 0 && threadIdx.x == 0) *a.epoch = e + 4u * (uint32_t)a.n_layers + 2u;
 }
 
 template <typename T>
@@ -483,11 +571,13 @@ int mmf_decode_layers_phase_bytes(void) { return (int)sizeof(Phase); }
 
 int mmf_decode_layers(const void* phases, int n_layers, const void* table, const int64_t* tok, int64_t vocab,
                       uint32_t* h0, uint32_t* h1, uint32_t* o, uint32_t* g, uint32_t* attn, uint32_t* res, uint32_t* z,
-                      void* h_out, uint32_t* epoch, int* err, int H, int D, int I, int spin, int dtype, void* stream_) {
+                      void* h_out, const void* head, void* logits, uint64_t* am_words, int64_t* tok_out, uint32_t* epoch, int* err,
+                      int H, int D, int I, int spin, int dtype, void* stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (!phases || n_layers <= 0 || !table || !tok || vocab <= 0 || !h0 || !h1 || !o || !g || !attn || !res || !z || !h_out ||
         !epoch || !err || H <= 0 || D <= 0 || I <= 0 || spin <= 0)
         return MMF_ERR_ARG;
+    if (head && (!logits || !am_words || !tok_out)) return MMF_ERR_ARG;
     if (H % 128 != 0 || D != H || I % 128 != 0) return MMF_ERR_ARG;      // rows are whole k-blocks: no ragged tail in a phase
     if (dtype != MMF_BF16 && dtype != MMF_F16) return MMF_ERR_ARG;        // a tagged word carries a 16-bit value
     if (H > 4096 || I > 8192) return MMF_ERR_WIDE;                        // at most two passes over an H-wide row, four over an I-wide one
@@ -500,7 +590,8 @@ int mmf_decode_layers(const void* phases, int n_layers, const void* table, const
     if (cus < kWGs) return MMF_ERR_ARG;                                       // the resident grid needs one CU per workgroup
     LayersArgs a{};
     a.phases = static_cast<const Phase*>(phases); a.n_layers = n_layers; a.table = table; a.tok = tok; a.vocab = vocab;
-    a.hb[0] = h0; a.hb[1] = h1; a.ob = o; a.gb = g; a.ab = attn; a.rb = res; a.zb = z; a.h_out = h_out; a.epoch = epoch;
+    a.hb[0] = h0; a.hb[1] = h1; a.ob = o; a.gb = g; a.ab = attn; a.rb = res; a.zb = z; a.h_out = h_out; a.head = static_cast<const Phase*>(head); a.logits = logits; a.am_words = am_words; a.tok_out = tok_out;
+    a.epoch = epoch;
     a.err = err; a.H = H; a.D = D; a.I = I; a.spin = spin;
     switch (dtype) {
         case MMF_BF16: return launch_layers<bf16_t>(a, stream);

@@ -170,7 +170,7 @@ class DecodeEngine:
     def _build_resident(self):
         H, D, I = self.H, self.D, self.I
         assert self.lib.mmf_decode_layers_phase_bytes() == ctypes.sizeof(_Phase)
-        table = (_Phase * (4 * self.L))()
+        table = (_Phase * (4 * self.L + 1))()            # the last record is the final norm + lm_head
 
         def fill(rec, w1, eps1, pw_nw_eps, k, n, lb=None, state=None):
             pw, nw, eps = pw_nw_eps
@@ -186,6 +186,7 @@ class DecodeEngine:
             fill(table[4 * li + 1], ent["g_norm"], ent["g_eps"], ent["o"], D, H)
             fill(table[4 * li + 2], ent["mlp_norm"], self.eps, ent["gate"], H, 2 * I)
             fill(table[4 * li + 3], None, 0.0, ent["down"], I, H)
+        fill(table[4 * self.L], self.final_norm, self.eps, self.head, H, self.V)
         raw = torch.frombuffer(bytearray(bytes(table)), dtype=torch.uint8)
         self.phases = raw.to(self.dev)
         sizes = [H, H, D, D, H, H, I]                       # h0, h1, o, g, attn, res, z
@@ -195,18 +196,27 @@ class DecodeEngine:
             self.words.append(words[off:off + n])
             off += n
         self._words = words
+        self.am_words = torch.zeros(256, dtype=torch.int64, device=self.dev)
+        self.head_inside = True     # final norm, lm_head and argmax as the last two links of the same launch
         self.epoch = torch.zeros(1, dtype=torch.int32, device=self.dev)
         self.err = torch.zeros(1, dtype=torch.int32, device=self.dev)
 
-    def _launch_step_resident(self):
-        lib, s = self.lib, L.stream()
+    def _launch_layers(self, with_head: bool):
         w = [t.data_ptr() for t in self.words]
-        L.check(lib.mmf_decode_layers(self.phases.data_ptr(), self.L, self.table.data_ptr(), self.tok.data_ptr(), self.V,
-                                      *w, self.h.data_ptr(), self.epoch.data_ptr(), self.err.data_ptr(), self.H, self.D,
-                                      self.I, self.SPIN, self.dt_id, s), "mmf_decode_layers")
+        head = self.phases.data_ptr() + 4 * self.L * ctypes.sizeof(_Phase) if with_head else None
+        L.check(self.lib.mmf_decode_layers(self.phases.data_ptr(), self.L, self.table.data_ptr(), self.tok.data_ptr(), self.V,
+                                           *w, self.h.data_ptr(), head, self.logits.data_ptr(), self.am_words.data_ptr(),
+                                           self.tok.data_ptr(), self.epoch.data_ptr(), self.err.data_ptr(), self.H, self.D,
+                                           self.I, self.SPIN, self.dt_id, L.stream()), "mmf_decode_layers")
+
+    def _launch_step_resident(self):
+        if self.head_inside:
+            return self._launch_layers(True)                    # the whole step is this one launch
+        self._launch_layers(False)
         self._fused(self.NORM, self.E_PLAIN, self.h, self.H, None, 0, None, self.final_norm, self.eps, self.head, self.logits,
                     None, None, None, self.V, self.H)
-        L.check(lib.mmf_argmax(self.logits.data_ptr(), self.V, 1, self.V, self.tok.data_ptr(), self.dt_id, s), "mmf_argmax")
+        L.check(self.lib.mmf_argmax(self.logits.data_ptr(), self.V, 1, self.V, self.tok.data_ptr(), self.dt_id, L.stream()),
+                "mmf_argmax")
 
     def resident_ok(self) -> bool:
         """False once a wait inside the resident layer chain ran out of polling rounds (host synchronisation)."""

@@ -349,6 +349,7 @@ def test_resident_layer_chain_equals_the_launch_chain(dev, dtype_name, hidden, i
             lr = res.step(tok).clone()
             lf = ref.step(tok).clone()
             assert torch.equal(lr, lf), f"logits differ at step {step} (graph={use_graph})"
+            assert torch.equal(res.tok, ref.tok), f"greedy token differs at step {step} (graph={use_graph})"
             tok = lf.argmax(-1)
         for a, b in zip(res.export_state(), ref.export_state()):
             assert torch.equal(a, b)
