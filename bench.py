@@ -100,7 +100,7 @@ def decode_bench(model, batch, steps, warmup, dev, prompt_len=128, resident=None
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain copy of known size);
 # see profiles/ for the runs and the scale factors.
 GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3623910          # one fused BitLinear GEMV launch of the launch chain
-LAYERS_TRAFFIC_BYTES_PER_LAUNCH = 330841649         # the resident layer-chain launch
+LAYERS_TRAFFIC_BYTES_PER_LAUNCH = 347655641         # the resident layer-chain launch
 
 
 def _replay_time(launch, iters):
@@ -119,20 +119,21 @@ def _replay_time(launch, iters):
 def gemv_roofline(eng, iters=20):
     """The dominant kernel of a batch-1 decode step, timed on its own inside a graph.
 
-    Resident engine: the one persistent launch that runs the 4L fused BitLinears of the layers (algorithmic bytes: the
-    layers' packed weights once, plus each link's activations, norm weights and state).  Otherwise: a graph that holds
+    Resident engine: the one persistent launch that is the whole step -- the 4L fused BitLinears of the layers, the
+    lm_head and the argmax (algorithmic bytes: every packed weight once, plus each link's activations, norm weights
+    and state).  Otherwise: a graph that holds
     exactly the fused BitLinear GEMV launches of one step (4 per layer + lm_head), averaged per launch."""
     assert eng.fused and eng.B == 1
     if eng.resident:
-        launch = lambda: eng._launch_layers(False)
+        launch = lambda: eng._launch_layers(eng.head_inside)
         ms = _replay_time(launch, iters)
         assert eng.resident_ok(), "a wait inside the resident layer chain timed out"
-        total_bytes = eng.fused_step_bytes(with_head=False)
+        total_bytes = eng.fused_step_bytes(with_head=eng.head_inside)
         achieved = total_bytes / (ms * 1e-3) / 1e9
         return {"bound": "hbm", "kernel": "decode_layers_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": LAYERS_TRAFFIC_BYTES_PER_LAUNCH,
-                "launches_per_step": 1, "links_per_launch": 4 * eng.L, "algorithmic_bytes_per_launch": total_bytes,
-                "avg_launch_us": round(ms * 1e3, 3), "us_per_link": round(ms * 1e3 / (4 * eng.L), 3)}
+                "launches_per_step": 1, "links_per_launch": 4 * eng.L + (2 if eng.head_inside else 0),
+                "algorithmic_bytes_per_launch": total_bytes, "avg_launch_us": round(ms * 1e3, 3)}
     ms = _replay_time(lambda: eng._launch_step_fused(ends=False), iters)
     n = 4 * eng.L + 1
     total_bytes = eng.fused_step_bytes()
