@@ -226,7 +226,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
             for (int r = 0; r < R; ++r) ep_wdeq[r] = ph.wdeq[(uint32_t)((nb + r * NBseg) * 32) / (uint32_t)ph.seg_rows];
             const int ch = nb * 32 + sub * CHN + (lane & (CHN - 1));
             if constexpr (EPI == EPI_STEP) {
-                if (lane < CHN && ch < Nseg) {
+                if (lane < (S == 4 ? 2 * CHN : CHN) && ch < Nseg) {   // S = 4: lanes 8..15 run the f rows of the same channels
                     if (ph.lb) ep_lb = ph.lb[ch];
                     ep_state = ph.state[ch];
                 }
@@ -386,7 +386,40 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
         }
         __syncthreads();
         const int ch = nb * 32 + sub * CHN + (lane & (CHN - 1));
-        if (wave == 0 && lane < CHN && ch < Nseg) {
+        if constexpr (EPI == EPI_STEP && S == 4) {
+            // Lanes 0-7 take the i rows, 8-15 the f rows, 16-23 the g rows of the same 8 channels, so the two exp /
+            // divide chains of the gate math run side by side instead of one after the other.  Every lane executes
+            // the same instructions (1 + exp(-v), then its reciprocal); the f lanes' gate reaches the i lanes by a
+            // rotate within the 16-lane row.  Operation for operation the arithmetic of the single-lane form.
+            if (wave == 0 && lane < 24) {
+                const int r3 = lane >> 3;
+                int qtot = 0;
+#pragma unroll
+                for (int w = 0; w < kNW; ++w) qtot += sm.red_q[w];
+                int tot = 0;
+                for (int gi = 0; gi < G; ++gi) {
+                    const int2 pr = sm.part[(r3 * G + gi) * 8 + (lane & 7)];
+                    tot += pr.x + pr.y;
+                }
+                const float wd = r3 == 0 ? ep_wdeq[0] : r3 == 1 ? ep_wdeq[1] : ep_wdeq[2];
+                const float res = __fmul_rn(__fmul_rn((float)(tot - qtot), deq), wd);
+                const float v16 = mmf_round_to<T>(res);                       // iv on the i lanes, fv on the f lanes
+                const float ex = __fadd_rn(1.0f, mmf_exp(-v16));
+                float sg = __fdiv_rn(1.0f, ex);                               // sigmoid(fv) on the f lanes
+                if (ph.lb) sg = __fadd_rn(ep_lb, __fmul_rn(__fsub_rn(1.0f, ep_lb), sg));
+                const float go = mmf_dpp<0x128>(mmf_round_to<T>(sg));         // lanes 0-7 read lanes 8-15
+                const float xo = mmf_round_to<T>(__fdiv_rn(__fmul_rn(v16, __fsub_rn(1.0f, go)), ex));
+                const float h = __fadd_rn(__fmul_rn(go, ep_state), xo);
+                if (ch < Nseg) {
+                    if (r3 == 0) {
+                        ph.state[ch] = h;
+                        ll_st4(out_words + ch, make_word<T>(h, tag_out));
+                    } else if (r3 == 2) {
+                        ll_st4(g_words + ch, make_word<T>(res, tag_out));
+                    }
+                }
+            }
+        } else if (wave == 0 && lane < CHN && ch < Nseg) {
             int qtot = 0;
 #pragma unroll
             for (int w = 0; w < kNW; ++w) qtot += sm.red_q[w];
