@@ -338,9 +338,10 @@ __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
                     tot += pr.x + pr.y;
                 }
             } else {
-                for (int gi = 0; gi < G; ++gi) {
-                    const int2 pr = part[(r * G + gi) * 8 + lane];
-                    tot += pr.x + pr.y;
+#pragma unroll
+                for (int gi = 0; gi < GMAX; ++gi) {                 // compile-time bound: the reads are issued together
+                    const int2 pr = part[(r * G + (gi < G ? gi : 0)) * 8 + lane];
+                    tot += gi < G ? pr.x + pr.y : 0;
                 }
             }
             res[r] = __fmul_rn(__fmul_rn((float)(tot - qtot), deq), ep_wdeq[r]);

@@ -397,9 +397,10 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
 #pragma unroll
                 for (int w = 0; w < kNW; ++w) qtot += sm.red_q[w];
                 int tot = 0;
-                for (int gi = 0; gi < G; ++gi) {
-                    const int2 pr = sm.part[(r3 * G + gi) * 8 + (lane & 7)];
-                    tot += pr.x + pr.y;
+#pragma unroll
+                for (int gi = 0; gi < GMAX; ++gi) {                 // compile-time bound: the reads are issued together
+                    const int2 pr = sm.part[(r3 * G + (gi < G ? gi : 0)) * 8 + (lane & 7)];
+                    tot += gi < G ? pr.x + pr.y : 0;
                 }
                 const float wd = r3 == 0 ? ep_wdeq[0] : r3 == 1 ? ep_wdeq[1] : ep_wdeq[2];
                 const float res = __fmul_rn(__fmul_rn((float)(tot - qtot), deq), wd);
@@ -434,9 +435,10 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
                         tot += pr.x + pr.y;
                     }
                 } else {
-                    for (int gi = 0; gi < G; ++gi) {
-                        const int2 pr = sm.part[(r * G + gi) * 8 + lane];
-                        tot += pr.x + pr.y;
+#pragma unroll
+                    for (int gi = 0; gi < GMAX; ++gi) {             // compile-time bound: the reads are issued together
+                        const int2 pr = sm.part[(r * G + (gi < G ? gi : 0)) * 8 + lane];
+                        tot += gi < G ? pr.x + pr.y : 0;
                     }
                 }
                 res[r] = __fmul_rn(__fmul_rn((float)(tot - qtot), deq), ep_wdeq[r]);
