@@ -245,20 +245,70 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
         if ((int)blockIdx.x + j * (int)gridDim.x < nvb) load_weights((int)blockIdx.x + j * (int)gridDim.x, wpf[j]);
     load_ep((int)blockIdx.x);
 
-    // ---- the row (and the prologue's second operand): poll until every word carries the producer's tag
+    // ---- the row (and the prologue's second operand): poll until every word carries the producer's tag.  The first
+    // read of every piece of both rows is issued before anything is examined, so an operand that was produced links
+    // ago (the residual stream) costs no round trip of its own, and the passes over a wide row do not queue up.
     float xv[NV][4], av[HAS_AUX ? NV : 1][4];
+    {
+        uint64_t xw[NV][2], aw[HAS_AUX ? NV : 1][2];
+        const bool x_tagged = xs.plain == nullptr, a_tagged = HAS_AUX && auxs.plain == nullptr;
+        auto issue = [&](const RowSrc& src, int k0, uint64_t (&w)[2]) {
+            const uint64_t* p = reinterpret_cast<const uint64_t*>(src.words + k0);
+            w[0] = ll_ld8(p);
+            w[1] = ll_ld8(p + 1);
+        };
+        auto valid = [&](const RowSrc& src, const uint64_t (&w)[2]) {
+            const uint64_t want = ((uint64_t)src.tag << 32) | src.tag, mask = 0x0000ffff0000ffffull;
+            return ((w[0] & mask) == want) && ((w[1] & mask) == want);
+        };
+        auto unpack = [&](const uint64_t (&w)[2], float (&out)[4]) {
+            out[0] = word_value<T>((uint32_t)w[0]);
+            out[1] = word_value<T>((uint32_t)(w[0] >> 32));
+            out[2] = word_value<T>((uint32_t)w[1]);
+            out[3] = word_value<T>((uint32_t)(w[1] >> 32));
+        };
 #pragma unroll
-    for (int v = 0; v < NV; ++v) {
-        const int k0 = (v * kNT + (int)threadIdx.x) * kEl;
+        for (int v = 0; v < NV; ++v) {
+            const int k0 = (v * kNT + (int)threadIdx.x) * kEl;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) xv[v][i] = 0.0f;
-        if constexpr (HAS_AUX) {
+            for (int i = 0; i < 4; ++i) xv[v][i] = 0.0f;
+            if constexpr (HAS_AUX) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) av[v][i] = 0.0f;
+                for (int i = 0; i < 4; ++i) av[v][i] = 0.0f;
+            }
+            if (k0 < K) {
+                if (x_tagged) issue(xs, k0, xw[v]);
+                else row_load4<T>(xs, k0, a.spin, a.err, xv[v]);
+                if constexpr (HAS_AUX) {
+                    if (a_tagged) issue(auxs, k0, aw[v]);
+                    else row_load4<T>(auxs, k0, a.spin, a.err, av[v]);
+                }
+            }
         }
-        if (k0 < K) {
-            row_load4<T>(xs, k0, a.spin, a.err, xv[v]);
-            if constexpr (HAS_AUX) row_load4<T>(auxs, k0, a.spin, a.err, av[v]);
+        for (int n = 0;; ++n) {
+            bool all = true;
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                const int k0 = (v * kNT + (int)threadIdx.x) * kEl;
+                if (k0 < K) {
+                    if (x_tagged && !valid(xs, xw[v])) { all = false; issue(xs, k0, xw[v]); }
+                    if constexpr (HAS_AUX) {
+                        if (a_tagged && !valid(auxs, aw[v])) { all = false; issue(auxs, k0, aw[v]); }
+                    }
+                }
+            }
+            if (all) break;
+            if (n >= a.spin) { *a.err = 1; break; }
+        }
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int k0 = (v * kNT + (int)threadIdx.x) * kEl;
+            if (k0 < K) {
+                if (x_tagged) unpack(xw[v], xv[v]);
+                if constexpr (HAS_AUX) {
+                    if (a_tagged) unpack(aw[v], av[v]);
+                }
+            }
         }
     }
 
