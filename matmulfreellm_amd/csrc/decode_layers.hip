@@ -1,4 +1,4 @@
-// All layers of one batch-1 decode step in ONE persistent launch.
+// One batch-1 decode step -- embedding row, all layers, final norm + lm_head, greedy argmax -- in ONE persistent launch.
 //
 // A decode step is a chain of 4 dependent fused BitLinears per layer (mmfreelm/models/hgrn_bit/
 // modeling_hgrn_bit.py:97-109 around mmfreelm/layers/hgrn_bit.py:83-162): block norm -> i/f/g -> gate math +
@@ -10,6 +10,15 @@
 // polled with relaxed device-scope accesses, so a consumer's poll is both the synchronisation and the
 // data transfer and no fence or grid barrier is needed.  The arithmetic of every phase is
 // that of bitlinear_gemv_kernel with the same prologue / epilogue, operation for operation.
+// With a head record the launch goes on with final norm -> lm_head (each workgroup walks several 32-row blocks behind
+// one prologue, writes plain logits and keeps its best candidate) and the greedy argmax (workgroup 0 combines the
+// workgroups' candidates and writes the token the next launch embeds; mmfreelm/models/hgrn_bit/
+// modeling_hgrn_bit.py:386 followed by the argmax of greedy decoding).
+//
+// Why a buffer is never rewritten under a reader: a workgroup stores a link's outputs only after it has polled that
+// link's whole input, i.e. after every producer of the previous link has finished that link -- and a producer reads
+// its inputs before it stores.  Every buffer is rewritten at the earliest two links after it was read (the residual
+// stream alternates between two buffers), and the chain of polls between those links passes through every reader.
 //
 // Every wait is bounded: a poll gives up after `spin` rounds, raises the error word and carries on
 // with whatever it read, so the grid always drains.  The host must make sure all 256 workgroups can
@@ -94,35 +103,13 @@ template <typename T> __device__ __forceinline__ uint32_t make_word(float v, uin
     return ((uint32_t)mmf_bits16(mmf_from_float<T>(v)) << 16) | tag;
 }
 
-// Four consecutive elements k0..k0+3 of a row (k0 a multiple of 4, k0 < K).
+// Four consecutive plain elements k0..k0+3 of a row (k0 a multiple of 4, k0 < K).
 template <typename T>
-__device__ __forceinline__ void row_load4(const RowSrc& s, int k0, int spin, int* err, float (&out)[4]) {
-    if (s.plain) {
-        Raw4<T> r = raw4_load<T, true>(static_cast<const T*>(s.plain), k0, k0 + 4);
-        raw4_unpack<T>(r, out);
-        return;
-    }
-    const uint64_t* p = reinterpret_cast<const uint64_t*>(s.words + k0);
-    const uint64_t want = ((uint64_t)s.tag << 32) | s.tag, mask = 0x0000ffff0000ffffull;
-    // two polls in flight: the next pair of loads is issued before the current pair is examined, which halves the
-    // time between a word's arrival and its detection
-    uint64_t a = ll_ld8(p), b = ll_ld8(p + 1);
-    int n = 0;
-    for (;;) {
-        const uint64_t a2 = ll_ld8(p), b2 = ll_ld8(p + 1);
-        if (((a & mask) == want) && ((b & mask) == want)) break;
-        a = a2;
-        b = b2;
-        if (++n >= spin) {
-            if (!(((a & mask) == want) && ((b & mask) == want))) *err = 1;
-            break;
-        }
-    }
-    out[0] = word_value<T>((uint32_t)a);
-    out[1] = word_value<T>((uint32_t)(a >> 32));
-    out[2] = word_value<T>((uint32_t)b);
-    out[3] = word_value<T>((uint32_t)(b >> 32));
+__device__ __forceinline__ void plain_load4(const RowSrc& s, int k0, float (&out)[4]) {
+    Raw4<T> r = raw4_load<T, true>(static_cast<const T*>(s.plain), k0, k0 + 4);
+    raw4_unpack<T>(r, out);
 }
+
 // One word whose first read `w` was issued long before (at the start of the phase): usually it already carries the tag.
 template <typename T>
 __device__ __forceinline__ float word_finish1(uint32_t w, const uint32_t* p, uint32_t tag, int spin, int* err) {
@@ -278,10 +265,10 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
             }
             if (k0 < K) {
                 if (x_tagged) issue(xs, k0, xw[v]);
-                else row_load4<T>(xs, k0, a.spin, a.err, xv[v]);
+                else plain_load4<T>(xs, k0, xv[v]);
                 if constexpr (HAS_AUX) {
                     if (a_tagged) issue(auxs, k0, aw[v]);
-                    else row_load4<T>(auxs, k0, a.spin, a.err, av[v]);
+                    else plain_load4<T>(auxs, k0, av[v]);
                 }
             }
         }
