@@ -94,6 +94,7 @@ def decode_bench(model, batch, steps, warmup, dev, prompt_len=128, resident=None
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms = max(s.elapsed_time(e), wall * 1e3) / steps      # never report less than the wall clock
+    eng.check()                                          # a timed-out wait inside the resident launch voids the figure
     return ms, eng
 
 
