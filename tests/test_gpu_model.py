@@ -388,3 +388,33 @@ def test_resident_layer_chain_timeout_is_reported_and_recoverable(dev, tiny_bf16
         assert torch.equal(a, b)
         tok = b.argmax(-1)
     eng.check()
+
+
+def test_resident_launch_at_the_full_1p3b_shape(dev):
+    """The benchmarked configuration itself (hidden 2048, 24 layers, vocabulary 32000, random weights on the device):
+    16 self-feeding greedy steps through the one-launch decode step and through the launch chain give the same
+    logits, tokens and recurrent states bit for bit (two independent schedules of the same arithmetic: every
+    workgroup of the resident launch takes part in every link at this size)."""
+    import bench
+    from matmulfreellm_amd.decode import DecodeEngine
+    model = bench.build_model("1.3B", torch.bfloat16, dev, seed=3)
+    g = torch.Generator(device=dev).manual_seed(5)
+    ids = torch.randint(0, 32000, (1, 64), generator=g, device=dev)
+    out = model(input_ids=ids, use_cache=True, logits_to_keep=1)
+    states = [c[-1] for c in out.past_key_values]
+    first = out.logits[:, -1].argmax(-1)
+    res = DecodeEngine(model, 1, use_graph=True, resident=True)
+    ref = DecodeEngine(model, 1, use_graph=True, resident=False)
+    for eng in (res, ref):
+        eng.load_state(states)
+        eng.tok.copy_(first)
+    for step in range(16):
+        res.advance()
+        ref.advance()
+        assert torch.equal(res.logits, ref.logits), f"logits differ at step {step}"
+        assert torch.equal(res.tok, ref.tok), f"token differs at step {step}"
+    for a, b in zip(res.export_state(), ref.export_state()):
+        assert torch.equal(a, b)
+    res.check()
+    del model, res, ref
+    torch.cuda.empty_cache()
