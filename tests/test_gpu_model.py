@@ -418,3 +418,23 @@ def test_resident_launch_at_the_full_1p3b_shape(dev):
     res.check()
     del model, res, ref
     torch.cuda.empty_cache()
+
+
+def test_resident_launch_across_the_tag_wrap(dev, tiny_bf16):
+    """The 16-bit tags of the resident launch wrap every 65536 links (3640 steps of this 4-layer model): 4000
+    self-feeding greedy steps give the launch chain's tokens, and no wait times out."""
+    from matmulfreellm_amd.decode import DecodeEngine
+    model = build(tiny_bf16, torch.bfloat16, dev)
+    torch.manual_seed(34)
+    ids = torch.randint(0, V, (1, 8), device=dev)
+    out = model(input_ids=ids, use_cache=True, logits_to_keep=1)
+    states = [c[-1] for c in out.past_key_values]
+    first = out.logits[:, -1].argmax(-1)
+    toks = []
+    for resident in (True, False):
+        eng = DecodeEngine(model, 1, use_graph=True, resident=resident)
+        eng.load_state(states)
+        toks.append(eng.greedy(first, 4000))
+        if resident:
+            assert int(eng.epoch.item()) >= 65536                  # the tag base went past the 16-bit range
+    assert torch.equal(toks[0], toks[1])
