@@ -126,14 +126,14 @@ def gemv_roofline(eng, iters=20):
     exactly the fused BitLinear GEMV launches of one step (4 per layer + lm_head), averaged per launch."""
     assert eng.fused and eng.B == 1
     if eng.resident:
-        launch = lambda: eng._launch_layers(eng.head_inside)
+        launch = lambda: eng._launch_layers(True)
         ms = _replay_time(launch, iters)
         assert eng.resident_ok(), "a wait inside the resident layer chain timed out"
-        total_bytes = eng.fused_step_bytes(with_head=eng.head_inside)
+        total_bytes = eng.fused_step_bytes()
         achieved = total_bytes / (ms * 1e-3) / 1e9
         return {"bound": "hbm", "kernel": "decode_layers_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": LAYERS_TRAFFIC_BYTES_PER_LAUNCH,
-                "launches_per_step": 1, "links_per_launch": 4 * eng.L + (2 if eng.head_inside else 0),
+                "launches_per_step": 1, "links_per_launch": 4 * eng.L + 2,
                 "algorithmic_bytes_per_launch": total_bytes, "avg_launch_us": round(ms * 1e3, 3)}
     ms = _replay_time(lambda: eng._launch_step_fused(ends=False), iters)
     n = 4 * eng.L + 1
@@ -280,9 +280,10 @@ def main():
         "config": {"workload": f"{args.shape}-shape HGRNBit greedy decode, batch {args.batch}, 128-token prompt, "
                                f"{args.steps} timed steps, whole step = one HIP graph",
                    "batch": args.batch, "ternary_weights": n_tern, "packed_weight_bytes": n_tern // 4,
-                   "decode_path": ("one resident launch (embedding row, layers, lm_head, argmax)" if eng.head_inside
-                                   else "resident layer chain + lm_head + argmax (3 launches)") if getattr(eng, "resident", False)
-                   else "one launch per fused BitLinear"},
+                   "decode_path": ("one resident launch (embedding row, layers, lm_head, argmax)" if eng.resident
+                                   else "one launch per fused BitLinear (4 per layer)" if eng.fused
+                                   else "fused quantiser + matrix-core contraction per BitLinear (8 launches per layer)"
+                                   if eng.fused_mfma else "one launch per reference op")},
     }
     hbm_step_us = (n_tern / 4) / (HBM_PEAK_GBS * 1e3)
     result["decode_frac_of_weight_stream_bound"] = round(hbm_step_us / (ms * 1e3), 4)

@@ -197,7 +197,6 @@ class DecodeEngine:
             off += n
         self._words = words
         self.am_words = torch.zeros(256, dtype=torch.int64, device=self.dev)
-        self.head_inside = True     # final norm, lm_head and argmax as the last two links of the same launch
         self.epoch = torch.zeros(1, dtype=torch.int32, device=self.dev)
         self.err = torch.zeros(1, dtype=torch.int32, device=self.dev)
 
@@ -210,13 +209,7 @@ class DecodeEngine:
                                            self.I, self.SPIN, self.dt_id, L.stream()), "mmf_decode_layers")
 
     def _launch_step_resident(self):
-        if self.head_inside:
-            return self._launch_layers(True)                    # the whole step is this one launch
-        self._launch_layers(False)
-        self._fused(self.NORM, self.E_PLAIN, self.h, self.H, None, 0, None, self.final_norm, self.eps, self.head, self.logits,
-                    None, None, None, self.V, self.H)
-        L.check(self.lib.mmf_argmax(self.logits.data_ptr(), self.V, 1, self.V, self.tok.data_ptr(), self.dt_id, L.stream()),
-                "mmf_argmax")
+        self._launch_layers(True)       # the whole step: final norm, lm_head and argmax are the launch's last two links
 
     def resident_ok(self) -> bool:
         """False once a wait inside the resident layer chain ran out of polling rounds (host synchronisation)."""
