@@ -350,6 +350,10 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
             from .decode import DecodeEngine
             engine = DecodeEngine.for_model(self, B)
             engine.load_state([c[-1] for c in cache])
+        if engine is not None and not do_sample:
+            new = _greedy_self_feeding(engine, F_.argmax(logits), max_new_tokens, eos_token_id, pad_token_id)
+            engine.check()
+            return torch.cat([input_ids, new], dim=1)
         for step in range(max_new_tokens):
             if do_sample:
                 nxt = _sample_top_p(logits.float(), top_p, temperature, generator)
@@ -370,6 +374,36 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
         if engine is not None:
             engine.check()
         return torch.cat(tokens, dim=1)
+
+
+def _greedy_self_feeding(engine, first, max_new_tokens, eos_token_id, pad_token_id, chunk=32):
+    """Greedy decoding without a host round trip per token: every replay of the engine's graph leaves its argmax in
+    the token buffer the next replay embeds.  The end-of-sequence test looks at a whole chunk of steps at a time; the
+    steps decoded past the point where every row had finished are cut off, and a finished row's later tokens are
+    replaced by the padding id, so the result is the one of the token-by-token loop."""
+    B = first.shape[0]
+    buf = torch.empty(max_new_tokens, B, dtype=torch.int64, device=first.device)
+    buf[0].copy_(first)
+    engine.tok.copy_(first.reshape(B))
+    produced = 1
+    while produced < max_new_tokens:
+        n = min(chunk, max_new_tokens - produced)
+        for _ in range(n):
+            engine.advance()
+            buf[produced].copy_(engine.tok)
+            produced += 1
+        if eos_token_id is not None and bool((buf[:produced] == eos_token_id).any(0).all()):
+            break
+    seq = buf[:produced].t()                                                    # [B, produced]
+    if eos_token_id is None:
+        return seq.contiguous()
+    is_eos = seq == eos_token_id
+    after = (is_eos.cumsum(1) - is_eos.long()) > 0                              # strictly after a row's first eos
+    seq = torch.where(after, torch.full_like(seq, eos_token_id if pad_token_id is None else pad_token_id), seq)
+    if bool(is_eos.any(1).all()):                                               # every row finished: stop where the last one did
+        last = int(is_eos.long().argmax(1).max()) + 1
+        seq = seq[:, :last]
+    return seq.contiguous()
 
 
 def _sample_top_p(logits, top_p, temperature, generator):
