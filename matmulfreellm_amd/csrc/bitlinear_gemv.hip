@@ -65,34 +65,6 @@ struct GemvArgs {
     double inv_K;         // RN(1 / K)
 };
 
-// Pairwise combination of the NW per-wave slots: log2(NW) dependent additions instead of NW - 1
-// (the kernel's time is its longest dependent chain).  Every thread adds in the same order.
-template <int N>
-__device__ __forceinline__ double tree_sum(const double* v) {
-    if constexpr (N == 1) return v[0];
-    else return tree_sum<N / 2>(v) + tree_sum<N - N / 2>(v + N / 2);
-}
-template <int NW>
-__device__ __forceinline__ double block_sum_once(double v, double* slot) {
-    v = mmf_wave_sum(v);
-    if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = v;
-    __syncthreads();
-    double t[NW];
-#pragma unroll
-    for (int i = 0; i < NW; ++i) t[i] = slot[i];
-    return tree_sum<NW>(t);
-}
-template <int NW>
-__device__ __forceinline__ float block_max_once(float v, float* slot) {
-    v = mmf_wave_max(v);
-    if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float s = slot[0];
-#pragma unroll
-    for (int i = 1; i < NW; ++i) s = fmaxf(s, slot[i]);
-    return s;
-}
-
 // NW waves per workgroup, NV passes over the row (Kp <= NV * NW * 256); a wave then owns at most
 // 2 * NV of the row's 1 KiB weight blocks per n-block.  The launcher takes the fewest passes, then
 // the fewest waves, that cover K: a thread's instruction stream, not bandwidth, sets the time.  VEC: K, the row strides and every pointer allow 4-element accesses.
@@ -209,7 +181,7 @@ __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
         for (int v = 0; v < NV; ++v)
 #pragma unroll
             for (int i = 0; i < 4; ++i) s1 += (double)xv[v][i] * (double)xv[v][i];
-        s1 = block_sum_once<kGemvWaves>(s1, red_a);
+        s1 = mmf_block_sum_once<kGemvWaves>(s1, red_a);
         const float rstd1 = mmf_rstd(s1, K, a.inv_K, a.eps1);
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
@@ -243,7 +215,7 @@ __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
     for (int v = 0; v < NV; ++v)
 #pragma unroll
         for (int i = 0; i < 4; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
-    ss = block_sum_once<kGemvWaves>(ss, red_b);
+    ss = mmf_block_sum_once<kGemvWaves>(ss, red_b);
     const float rstd = mmf_rstd(ss, K, a.inv_K, a.eps);
     float amax = 0.0f;
 #pragma unroll
@@ -258,7 +230,7 @@ __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
             amax = fmaxf(amax, fabsf(y));
         }
     }
-    amax = block_max_once<kGemvWaves>(amax, red_f);
+    amax = mmf_block_max_once<kGemvWaves>(amax, red_f);
     const float scale = __fdiv_rn(127.0f, fmaxf(amax, 1e-5f));
     const float deq = __fdiv_rn(1.0f, scale);                 // needed by the epilogue only: computed here, in the shadow of the barriers
     int qs = 0;
@@ -283,18 +255,7 @@ __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
     if (lane == 0) red_q[wave] = qs;
 
     // ---- main: sum_k q[k] * (t[n,k] + 1) over this wave's blocks
-    auto dot_block = [&](const uint4& wq, int kb, int acc) {
-#pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4) {
-            const int4 qv = *reinterpret_cast<const int4*>(q_lds + kb * 128 + s4 * 32 + half * 16);
-            const uint32_t w = s4 == 0 ? wq.x : s4 == 1 ? wq.y : s4 == 2 ? wq.z : wq.w;
-            acc = __builtin_amdgcn_sdot4((int)(w & 0x03030303u), qv.x, acc, false);
-            acc = __builtin_amdgcn_sdot4((int)((w >> 2) & 0x03030303u), qv.y, acc, false);
-            acc = __builtin_amdgcn_sdot4((int)((w >> 4) & 0x03030303u), qv.z, acc, false);
-            acc = __builtin_amdgcn_sdot4((int)((w >> 6) & 0x03030303u), qv.w, acc, false);
-        }
-        return acc;
-    };
+    auto dot_block = [&](const uint4& wq, int kb, int acc) { return mmf_dot_block(q_lds, wq, kb, half, acc); };
     if constexpr (S == 1) {
         int acc[R];
 #pragma unroll

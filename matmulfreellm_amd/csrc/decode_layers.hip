@@ -119,30 +119,6 @@ __device__ __forceinline__ float word_finish1(uint32_t w, const uint32_t* p, uin
     return word_value<T>(w);
 }
 
-template <int N>
-__device__ __forceinline__ double tree_sum(const double* v) {
-    if constexpr (N == 1) return v[0];
-    else return tree_sum<N / 2>(v) + tree_sum<N - N / 2>(v + N / 2);
-}
-__device__ __forceinline__ double block_sum_once(double v, double* slot) {
-    v = mmf_wave_sum(v);
-    if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = v;
-    __syncthreads();
-    double t[kNW];
-#pragma unroll
-    for (int i = 0; i < kNW; ++i) t[i] = slot[i];
-    return tree_sum<kNW>(t);
-}
-__device__ __forceinline__ float block_max_once(float v, float* slot) {
-    v = mmf_wave_max(v);
-    if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float s = slot[0];
-#pragma unroll
-    for (int i = 1; i < kNW; ++i) s = fmaxf(s, slot[i]);
-    return s;
-}
-
 // One phase.  NV passes over the row (K <= NV * 2048); S = 4: a virtual block owns 8 of an n-block's 32 rows.
 // Virtual block vb -> (n-block vb / S, row group vb % S); a workgroup takes vb = blockIdx.x, + gridDim.x, ...
 // The prologue (the row's int8 codes) is computed once per workgroup, whatever the number of virtual blocks.
@@ -321,7 +297,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
         for (int v = 0; v < NV; ++v)
 #pragma unroll
             for (int i = 0; i < 4; ++i) s1 += (double)xv[v][i] * (double)xv[v][i];
-        s1 = block_sum_once(s1, sm.red_a);
+        s1 = mmf_block_sum_once<kNW>(s1, sm.red_a);
         const float rstd1 = mmf_rstd(s1, K, ph.inv_K, ph.eps1);
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
@@ -343,7 +319,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
     for (int v = 0; v < NV; ++v)
 #pragma unroll
         for (int i = 0; i < 4; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
-    ss = block_sum_once(ss, sm.red_b);
+    ss = mmf_block_sum_once<kNW>(ss, sm.red_b);
     const float rstd = mmf_rstd(ss, K, ph.inv_K, ph.eps);
     float amax = 0.0f;
 #pragma unroll
@@ -357,7 +333,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
             amax = fmaxf(amax, fabsf(y));
         }
     }
-    amax = block_max_once(amax, sm.red_f);
+    amax = mmf_block_max_once<kNW>(amax, sm.red_f);
     const float scale = __fdiv_rn(127.0f, fmaxf(amax, 1e-5f));
     const float deq = __fdiv_rn(1.0f, scale);                 // needed by the epilogue only: computed here, in the shadow of the barriers
     int qs = 0;
@@ -379,18 +355,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
     qs = mmf_wave_sum(qs);
     if (lane == 0) sm.red_q[wave] = qs;
 
-    auto dot_block = [&](const uint4& wq, int kb, int acc) {
-#pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4) {
-            const int4 qv = *reinterpret_cast<const int4*>(sm.q + kb * 128 + s4 * 32 + half * 16);
-            const uint32_t w = s4 == 0 ? wq.x : s4 == 1 ? wq.y : s4 == 2 ? wq.z : wq.w;
-            acc = __builtin_amdgcn_sdot4((int)(w & 0x03030303u), qv.x, acc, false);
-            acc = __builtin_amdgcn_sdot4((int)((w >> 2) & 0x03030303u), qv.y, acc, false);
-            acc = __builtin_amdgcn_sdot4((int)((w >> 4) & 0x03030303u), qv.z, acc, false);
-            acc = __builtin_amdgcn_sdot4((int)((w >> 6) & 0x03030303u), qv.w, acc, false);
-        }
-        return acc;
-    };
+    auto dot_block = [&](const uint4& wq, int kb, int acc) { return mmf_dot_block(sm.q, wq, kb, half, acc); };
 
     auto process = [&](int vb, const uint4 (&wreg)[NWREG]) {
         const int nb = vb / S, sub = vb % S;

@@ -302,6 +302,51 @@ __device__ __forceinline__ int mmf_block_sum(int v, int* red) {
     return s;
 }
 
+// One 1 KiB packed weight block (a lane holds 64 weights of one output row: 4 dwords = 4 k-steps of 16) against the
+// int8 codes of k-block kb in LDS: each dword expands to four byte-wide code dwords (shift + mask), v_dot4_i32_i8
+// accumulates.  `half` selects the lane's 16 of each k-step's 32 inputs.
+__device__ __forceinline__ int mmf_dot_block(const int8_t* q_lds, const uint4& wq, int kb, int half, int acc) {
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) {
+        const int4 qv = *reinterpret_cast<const int4*>(q_lds + kb * 128 + s4 * 32 + half * 16);
+        const uint32_t w = s4 == 0 ? wq.x : s4 == 1 ? wq.y : s4 == 2 ? wq.z : wq.w;
+        acc = __builtin_amdgcn_sdot4((int)(w & 0x03030303u), qv.x, acc, false);
+        acc = __builtin_amdgcn_sdot4((int)((w >> 2) & 0x03030303u), qv.y, acc, false);
+        acc = __builtin_amdgcn_sdot4((int)((w >> 4) & 0x03030303u), qv.z, acc, false);
+        acc = __builtin_amdgcn_sdot4((int)((w >> 6) & 0x03030303u), qv.w, acc, false);
+    }
+    return acc;
+}
+
+// One-barrier block reductions of the decode kernels: the NW per-wave results meet in `slot` (LDS, NW entries,
+// one array per reduction so that no second barrier is needed before its reuse) and every thread combines them
+// pairwise in the same order: log2(NW) dependent additions instead of NW - 1.
+template <int N>
+__device__ __forceinline__ double mmf_tree_sum(const double* v) {
+    if constexpr (N == 1) return v[0];
+    else return mmf_tree_sum<N / 2>(v) + mmf_tree_sum<N - N / 2>(v + N / 2);
+}
+template <int NW>
+__device__ __forceinline__ double mmf_block_sum_once(double v, double* slot) {
+    v = mmf_wave_sum(v);
+    if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = v;
+    __syncthreads();
+    double t[NW];
+#pragma unroll
+    for (int i = 0; i < NW; ++i) t[i] = slot[i];
+    return mmf_tree_sum<NW>(t);
+}
+template <int NW>
+__device__ __forceinline__ float mmf_block_max_once(float v, float* slot) {
+    v = mmf_wave_max(v);
+    if ((threadIdx.x & 63) == 0) slot[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float s = slot[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) s = fmaxf(s, slot[i]);
+    return s;
+}
+
 // rstd = 1 / sqrt( fp32(sumsq / K) + eps ).
 // sumsq / K is the correctly rounded fp64 quotient without the division sequence: with
 // inv_K = RN(1 / K) from the host, q0 = sumsq * inv_K is within two ulps, one residual step
