@@ -100,8 +100,8 @@ def decode_bench(model, batch, steps, warmup, dev, prompt_len=128, resident=None
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain copy of known size);
 # see profiles/ for the runs and the scale factors.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3623910          # one fused BitLinear GEMV launch of the launch chain
-LAYERS_TRAFFIC_BYTES_PER_LAUNCH = 347655641         # the resident layer-chain launch
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3625495          # one fused BitLinear GEMV launch of the launch chain
+LAYERS_TRAFFIC_BYTES_PER_LAUNCH = 348021769         # the resident layer-chain launch
 
 
 def _replay_time(launch, iters):
