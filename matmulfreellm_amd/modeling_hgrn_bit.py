@@ -308,7 +308,7 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
     def generate(self, input_ids: Optional[torch.LongTensor] = None, attention_mask: Optional[torch.Tensor] = None,
                  max_new_tokens: Optional[int] = None, max_length: Optional[int] = None, do_sample: bool = False,
                  top_p: float = 1.0, temperature: float = 1.0, eos_token_id: Optional[int] = None,
-                 pad_token_id: Optional[int] = None, use_graph: bool = True,
+                 pad_token_id: Optional[int] = None, use_graph: bool = True, resident: Optional[bool] = None,
                  generator: Optional[torch.Generator] = None, **kwargs) -> torch.LongTensor:
         """Greedy (default) or top-p sampling; returns [B, T + new] token ids like HF's generate.
 
@@ -317,7 +317,8 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
         use_graph is set (sampling draws from the graph's logits and feeds the drawn token back; the logits are
         bit-identical to the module path's, so a seeded generator gives the same tokens either way). Rows that
         have produced eos_token_id (default: the generation config's) are filled with pad_token_id (eos_token_id
-        when not given); generation ends early once every row has.
+        when not given); generation ends early once every row has.  At batch 1 the whole decode step is one resident
+        launch when the model fits it; resident=False keeps one launch per fused BitLinear.
 
         Any further keyword (num_beams, repetition_penalty, logits_processor, stopping_criteria, streamer,
         generation_config, top_k, return_dict_in_generate, ...) sends the whole call to
@@ -348,7 +349,7 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
         engine = None
         if use_graph and max_new_tokens > 1:
             from .decode import DecodeEngine
-            engine = DecodeEngine.for_model(self, B)
+            engine = DecodeEngine.for_model(self, B, resident=resident)
             engine.load_state([c[-1] for c in cache])
         if engine is not None and not do_sample:
             new = _greedy_self_feeding(engine, F_.argmax(logits), max_new_tokens, eos_token_id, pad_token_id)

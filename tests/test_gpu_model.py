@@ -438,3 +438,13 @@ def test_resident_launch_across_the_tag_wrap(dev, tiny_bf16):
         if resident:
             assert int(eng.epoch.item()) >= 65536                  # the tag base went past the 16-bit range
     assert torch.equal(toks[0], toks[1])
+
+
+def test_generate_is_the_same_with_and_without_the_resident_launch(dev, tiny_bf16):
+    model = build(tiny_bf16, torch.bfloat16, dev)
+    torch.manual_seed(35)
+    ids = torch.randint(0, V, (1, 9), device=dev)
+    a = model.generate(ids, max_new_tokens=40)
+    b = model.generate(ids, max_new_tokens=40, resident=False)
+    c = model.generate(ids, max_new_tokens=40, use_graph=False)
+    assert a.shape == (1, 49) and torch.equal(a, b) and torch.equal(a, c)
