@@ -448,3 +448,43 @@ def test_generate_is_the_same_with_and_without_the_resident_launch(dev, tiny_bf1
     b = model.generate(ids, max_new_tokens=40, resident=False)
     c = model.generate(ids, max_new_tokens=40, use_graph=False)
     assert a.shape == (1, 49) and torch.equal(a, b) and torch.equal(a, c)
+
+
+def test_batch_128_decode_at_the_2p7b_shape_equals_batch_1_rows(dev):
+    """The large-batch configuration (hidden 2560, 32 layers, intermediate 6912, vocabulary 32000; prompts of 512
+    tokens at batch 128): prefill and 8 greedy steps run on the matrix-core path at M = 65536 and M = 128; rows
+    0, 77 and 127 of that batch must carry, bit for bit, the logits, tokens and recurrent states that the batch-1
+    paths (the wave-reduction launch chain and the resident launch) produce from the same prompt alone."""
+    import bench
+    from matmulfreellm_amd.decode import DecodeEngine
+    model = bench.build_model("2.7B", torch.bfloat16, dev, seed=4)
+    g = torch.Generator(device=dev).manual_seed(6)
+    ids = torch.randint(0, 32000, (128, 512), generator=g, device=dev)
+    out = model(input_ids=ids, use_cache=True, logits_to_keep=1)
+    states = [c[-1] for c in out.past_key_values]
+    first = out.logits[:, -1].argmax(-1)
+    big = DecodeEngine(model, 128, use_graph=True)
+    big.load_state(states)
+    big.tok.copy_(first)
+    rows = (0, 77, 127)
+    small = []
+    for i, r in enumerate(rows):
+        o1 = model(input_ids=ids[r:r + 1], use_cache=True, logits_to_keep=1)
+        assert torch.equal(o1.logits[0, -1], out.logits[r, -1]), f"prefill logits of row {r} depend on the batch"
+        eng = DecodeEngine(model, 1, use_graph=True, resident=(i != 1))
+        eng.load_state([c[-1] for c in o1.past_key_values])
+        eng.tok.copy_(first[r:r + 1])
+        small.append(eng)
+    for step in range(8):
+        big.advance()
+        for r, eng in zip(rows, small):
+            eng.advance()
+            assert torch.equal(eng.logits[0], big.logits[r]), f"row {r}: logits differ at step {step}"
+            assert torch.equal(eng.tok[0], big.tok[r]), f"row {r}: token differs at step {step}"
+    final = big.export_state()
+    for r, eng in zip(rows, small):
+        for a, b in zip(eng.export_state(), final):
+            assert torch.equal(a[0], b[r])
+        eng.check()
+    del model, big, small
+    torch.cuda.empty_cache()
