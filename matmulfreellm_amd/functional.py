@@ -449,3 +449,29 @@ def argmax(logits):
         L.check(lib.mmf_argmax(l2.data_ptr(), v, l2.shape[0], v, out.data_ptr(), L.dtype_id(l2.dtype), L.stream()),
                 "mmf_argmax")
     return out.reshape(logits.shape[:-1])
+
+
+def sample_top_p(logits, top_p, temperature, u, out=None):
+    """One top-p (nucleus) draw per row; logits [..., V], u fp32 [...] uniform in [0, 1) -> int64 [...].
+
+    What transformers' sampling path does per token for the reference's generate.py:11 (temperature, softmax,
+    sort, cumulative sum, nucleus mask, multinomial), as one launch: integer probability masses decide the nucleus
+    and the draw is the inverse CDF of u over the kept tokens in index order (include/mmf.h gives the arithmetic).
+    The caller owns the random stream: u = torch.rand(..., generator=g)."""
+    lib = L.load()
+    dev = L.require_gpu(logits)
+    v = logits.shape[-1]
+    l2 = _as_2d(logits)
+    rows = l2.shape[0]
+    if not (isinstance(u, torch.Tensor) and u.dtype == torch.float32 and u.device == dev and u.numel() == rows):
+        raise L.MMFError("sample_top_p: u must be an fp32 tensor on the logits' device with one number per row")
+    if not u.is_contiguous():
+        u = u.contiguous()
+    if out is None:
+        out = torch.empty(rows, dtype=torch.int64, device=dev)
+    elif not (out.dtype == torch.int64 and out.device == dev and out.numel() == rows and out.is_contiguous()):
+        raise L.MMFError("sample_top_p: out must be a contiguous int64 tensor with one element per row")
+    with torch.cuda.device(dev):
+        L.check(lib.mmf_sample_top_p(l2.data_ptr(), l2.stride(0), rows, v, float(temperature), float(top_p), u.data_ptr(),
+                                     out.data_ptr(), L.dtype_id(l2.dtype), L.stream()), "mmf_sample_top_p")
+    return out.reshape(logits.shape[:-1])

@@ -1,0 +1,100 @@
+"""GPU parity of the top-p sampler: the drawn token must be the integer restatement's, exactly, on the same logits
+and the same uniform numbers (the arithmetic is integer, so there is no tolerance)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import sampling as S
+
+pytestmark = pytest.mark.gpu
+
+
+def F():
+    import matmulfreellm_amd.functional as F_
+    return F_
+
+
+def _check_rows(dev, logits, temperature, top_p, u, what):
+    got = F().sample_top_p(logits.to(dev), top_p, temperature, u.to(dev)).cpu()
+    want = [S.sample_top_p_spec(logits[r].float().numpy(), temperature, top_p, float(u[r]))[0] for r in range(logits.shape[0])]
+    bad = [(r, int(got[r]), want[r]) for r in range(len(want)) if int(got[r]) != want[r]]
+    print(f"{what}: {len(want)} rows, {len(bad)} differ", flush=True)
+    assert not bad, (what, bad[:5])
+    return got
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_tokens_equal_the_integer_restatement_at_vocabulary_32000(dev, dtype):
+    g = torch.Generator().manual_seed(21)
+    rows = 48
+    sharp = torch.tensor([0.3, 1.0, 2.5, 6.0]).repeat(rows // 4)[:, None]
+    logits = (torch.randn(rows, 32000, generator=g) * sharp).to(dtype)
+    u = torch.rand(rows, generator=g)
+    for temperature, top_p in ((0.6, 0.4), (1.0, 0.9), (0.25, 0.05), (1.3, 1.0)):
+        _check_rows(dev, logits, temperature, top_p, u, f"{dtype} T={temperature} top_p={top_p}")
+
+
+def test_ragged_vocabularies_strided_rows_and_two_passes_per_thread(dev):
+    g = torch.Generator().manual_seed(22)
+    for v in (1, 7, 33, 1000, 4097, 32768, 50257, 65536):
+        rows = 6
+        wide = torch.randn(rows, v + 5, generator=g) * 2.0
+        logits = wide[:, :v]                                    # row stride v + 5: the unaligned path
+        u = torch.rand(rows, generator=g)
+        got = F().sample_top_p(logits.to(dev), 0.8, 0.7, u.to(dev)).cpu()
+        want = [S.sample_top_p_spec(logits[r].numpy(), 0.7, 0.8, float(u[r]))[0] for r in range(rows)]
+        assert got.tolist() == want, (v, got.tolist(), want)
+        lb = logits.contiguous().bfloat16()
+        _check_rows(dev, lb, 0.7, 0.8, u, f"V={v} bf16")
+
+
+def test_edge_values_of_top_p_u_and_the_logits(dev):
+    g = torch.Generator().manual_seed(23)
+    logits = (torch.randn(8, 2048, generator=g) * 3).bfloat16()
+    logits[1, 5] = float("nan")
+    logits[2, 9] = float("inf")
+    logits[3] = float("-inf")
+    logits[3, 100] = 0.0
+    logits[4] = 1.5                                             # every token ties: all are kept whatever top_p says
+    logits[5, :] = float("nan")                                 # nothing to prefer: uniform over the row
+    u = torch.tensor([0.0, 0.5, 0.99, 0.3, 0.7, 0.25, 0.99999994, 0.5])
+    for top_p in (0.0, 1e-9, 0.4, 1.0, 3.0, -1.0):
+        got = _check_rows(dev, logits, 0.6, top_p, u, f"edges top_p={top_p}")
+        assert int(got[2]) == 9 and int(got[3]) == 100
+        if top_p <= 1e-9:                                       # only the most probable tokens stay
+            assert got[0] == logits[0].float().argmax()
+    assert int(got[4]) == int(0.7 * 2048) and int(got[5]) == 512
+    # out-of-range uniform numbers are clamped, never read past the row
+    bad_u = torch.tensor([1.0, 7.0, -3.0, float("nan"), 0.5, 0.5, 0.5, 0.5])
+    _check_rows(dev, logits, 0.6, 0.9, bad_u, "clamped u")
+
+
+def test_draws_follow_the_renormalised_nucleus(dev):
+    """20000 draws from one row (stratified uniforms): only kept tokens appear, with the kept masses' frequencies."""
+    g = torch.Generator().manual_seed(24)
+    row = (torch.randn(512, generator=g) * 2).bfloat16()
+    n = 20000
+    u = ((torch.arange(n, dtype=torch.float64) + 0.5) / n).float()
+    got = F().sample_top_p(row[None].expand(n, -1).contiguous().to(dev), 0.9, 0.8, u.to(dev)).cpu().numpy()
+    _, keep, m = S.sample_top_p_spec(row.float().numpy(), 0.8, 0.9, 0.0)
+    want = np.where(keep, m.astype(np.float64), 0.0)
+    want /= want.sum()
+    freq = np.bincount(got, minlength=512) / n
+    assert (freq[~keep] == 0).all() and np.abs(freq - want).max() < 2e-4
+
+
+def test_rejected_arguments(dev):
+    from matmulfreellm_amd._lib import MMFError
+    logits = torch.zeros(2, 64, device=dev)
+    u = torch.rand(2, device=dev)
+    for bad_t in (0.0, -1.0, float("nan")):
+        with pytest.raises(MMFError):
+            F().sample_top_p(logits, 0.5, bad_t, u)
+    with pytest.raises(MMFError):
+        F().sample_top_p(logits, float("nan"), 1.0, u)
+    with pytest.raises(MMFError):
+        F().sample_top_p(torch.zeros(1, 70000, device=dev), 0.5, 1.0, u[:1])      # wider than the kernel's registers hold
+    with pytest.raises(MMFError):
+        F().sample_top_p(logits, 0.5, 1.0, u.double())
+    with pytest.raises(MMFError):
+        F().sample_top_p(logits.cpu(), 0.5, 1.0, u)
