@@ -475,3 +475,8 @@ def sample_top_p(logits, top_p, temperature, u, out=None):
         L.check(lib.mmf_sample_top_p(l2.data_ptr(), l2.stride(0), rows, v, float(temperature), float(top_p), u.data_ptr(),
                                      out.data_ptr(), L.dtype_id(l2.dtype), L.stream()), "mmf_sample_top_p")
     return out.reshape(logits.shape[:-1])
+
+
+def sample_top_p_max_vocab():
+    """Widest row sample_top_p accepts."""
+    return int(L.load().mmf_sample_top_p_max_vocab())

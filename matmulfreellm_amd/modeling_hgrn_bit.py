@@ -314,8 +314,11 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
 
         With the arguments above (what the reference's generate.py passes), prefill runs the module path with
         last-position logits only and decode runs the captured whole-step HIP graph of DecodeEngine when
-        use_graph is set (sampling draws from the graph's logits and feeds the drawn token back; the logits are
-        bit-identical to the module path's, so a seeded generator gives the same tokens either way). Rows that
+        use_graph is set.  Sampling draws every token with one launch of the top-p kernel (functional.sample_top_p)
+        on the step's logits and feeds it back without a host round trip; the uniform numbers of the whole run are
+        drawn up front from `generator` (torch.rand), and the logits are bit-identical to the module path's, so a
+        seeded generator gives the same tokens either way (not the tokens torch.multinomial would draw from the
+        same seed).  Rows that
         have produced eos_token_id (default: the generation config's) are filled with pad_token_id (eos_token_id
         when not given); generation ends early once every row has.  At batch 1 the whole decode step is one resident
         launch when the model fits it; resident=False keeps one launch per fused BitLinear.
@@ -340,6 +343,8 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
             return GenerationMixin.generate(self, input_ids, do_sample=do_sample, **hf)
         if max_new_tokens is None:
             max_new_tokens = (max_length - input_ids.shape[1]) if max_length is not None else 20
+        if max_new_tokens <= 0:
+            return input_ids
         B = input_ids.shape[0]
         out = self(input_ids=input_ids, attention_mask=attention_mask, use_cache=True, logits_to_keep=1)
         cache = out.past_key_values
@@ -351,37 +356,44 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
             from .decode import DecodeEngine
             engine = DecodeEngine.for_model(self, B, resident=resident)
             engine.load_state([c[-1] for c in cache])
-        if engine is not None and not do_sample:
-            new = _greedy_self_feeding(engine, F_.argmax(logits), max_new_tokens, eos_token_id, pad_token_id)
+        choose = None
+        if do_sample:
+            temperature = max(float(temperature), 1e-6)
+            if logits.shape[-1] <= F_.sample_top_p_max_vocab():
+                # every uniform number of the run is drawn here, so the random stream does not depend on the path taken
+                g_dev = generator.device if generator is not None else input_ids.device
+                uniforms = torch.rand(max_new_tokens, B, generator=generator, device=g_dev).to(input_ids.device)
+                choose = lambda lg, step, out=None: F_.sample_top_p(lg, top_p, temperature, uniforms[step], out=out)
+            else:
+                choose = lambda lg, step, out=None: _sample_top_p(lg.float(), top_p, temperature, generator, out)
+        first = choose(logits, 0) if do_sample else F_.argmax(logits)
+        if engine is not None:
+            pick = (lambda step: choose(engine.logits, step, engine.tok)) if do_sample else None
+            new = _self_feeding(engine, first, max_new_tokens, eos_token_id, pad_token_id, pick=pick)
             engine.check()
             return torch.cat([input_ids, new], dim=1)
+        nxt = first
         for step in range(max_new_tokens):
-            if do_sample:
-                nxt = _sample_top_p(logits.float(), top_p, temperature, generator)
-            else:
-                nxt = F_.argmax(logits)
+            if step > 0:
+                out = self(input_ids=nxt.view(B, 1), past_key_values=cache, use_cache=True)
+                cache = out.past_key_values
+                logits = out.logits[:, -1, :]
+                nxt = choose(logits, step) if do_sample else F_.argmax(logits)
             if eos_token_id is not None:
                 nxt = torch.where(finished, torch.full_like(nxt, eos_token_id if pad_token_id is None else pad_token_id), nxt)
                 finished |= nxt == eos_token_id
             tokens.append(nxt.view(B, 1))
-            if step == max_new_tokens - 1 or (eos_token_id is not None and bool(finished.all())):
+            if eos_token_id is not None and bool(finished.all()):
                 break
-            if engine is not None:
-                logits = engine.step(nxt)
-            else:
-                out = self(input_ids=nxt.view(B, 1), past_key_values=cache, use_cache=True)
-                cache = out.past_key_values
-                logits = out.logits[:, -1, :]
-        if engine is not None:
-            engine.check()
         return torch.cat(tokens, dim=1)
 
 
-def _greedy_self_feeding(engine, first, max_new_tokens, eos_token_id, pad_token_id, chunk=32):
-    """Greedy decoding without a host round trip per token: every replay of the engine's graph leaves its argmax in
-    the token buffer the next replay embeds.  The end-of-sequence test looks at a whole chunk of steps at a time; the
-    steps decoded past the point where every row had finished are cut off, and a finished row's later tokens are
-    replaced by the padding id, so the result is the one of the token-by-token loop."""
+def _self_feeding(engine, first, max_new_tokens, eos_token_id, pad_token_id, chunk=32, pick=None):
+    """Decoding without a host round trip per token: every replay of the engine's graph leaves its argmax in the
+    token buffer the next replay embeds; pick(step), when given, replaces that token by one drawn from the step's
+    logits (sampling) before it is recorded.  The end-of-sequence test looks at a whole chunk of steps at a time;
+    the steps decoded past the point where every row had finished are cut off, and a finished row's later tokens
+    are replaced by the padding id, so the result is the one of the token-by-token loop."""
     B = first.shape[0]
     buf = torch.empty(max_new_tokens, B, dtype=torch.int64, device=first.device)
     buf[0].copy_(first)
@@ -391,6 +403,8 @@ def _greedy_self_feeding(engine, first, max_new_tokens, eos_token_id, pad_token_
         n = min(chunk, max_new_tokens - produced)
         for _ in range(n):
             engine.advance()
+            if pick is not None:
+                pick(produced)
             buf[produced].copy_(engine.tok)
             produced += 1
         if eos_token_id is not None and bool((buf[:produced] == eos_token_id).any(0).all()):
@@ -407,11 +421,16 @@ def _greedy_self_feeding(engine, first, max_new_tokens, eos_token_id, pad_token_
     return seq.contiguous()
 
 
-def _sample_top_p(logits, top_p, temperature, generator):
+def _sample_top_p(logits, top_p, temperature, generator, out=None):
+    """Vocabularies wider than the sampling kernel holds: the same nucleus with library calls."""
     probs = torch.softmax(logits / max(temperature, 1e-6), dim=-1)
     sp, si = torch.sort(probs, dim=-1, descending=True)
     keep = (sp.cumsum(-1) - sp) < top_p
     sp = sp * keep
     sp = sp / sp.sum(-1, keepdim=True)
     choice = torch.multinomial(sp, 1, generator=generator)
-    return si.gather(-1, choice).squeeze(-1)
+    tok = si.gather(-1, choice).squeeze(-1)
+    if out is not None:
+        out.copy_(tok)
+        return out
+    return tok

@@ -250,6 +250,34 @@ def test_top_p_sampling_is_the_same_through_the_decode_graph(dev, tiny_bf16):
     assert torch.equal(outs[0], outs[1])
 
 
+def test_sampled_tokens_equal_the_oracle_driven_by_the_same_uniform_numbers(dev, tiny_bf16):
+    """generate(do_sample=True) end to end against the CPU oracle: the oracle's forward gives each step's logits, its
+    integer top-p restatement draws with the uniform numbers generate() takes from the seeded generator
+    (torch.rand(max_new_tokens, B)), and the tokens must be identical on the graph path (batch 1: the resident
+    launch; batch 3: the launch chain) and on the module path."""
+    from oracle import sampling as osamp
+    model = build(tiny_bf16, torch.bfloat16, dev)
+    n_new, top_p, temperature = 6, 0.4, 0.6
+    for batch in (1, 3):
+        torch.manual_seed(40 + batch)
+        ids = torch.randint(0, V, (batch, 12))
+        u = torch.rand(n_new, batch, generator=torch.Generator(device=dev).manual_seed(77), device=dev).cpu()
+        ops = om._Ops("spec", 1e-8)
+        logits, states = om.forward(tiny_bf16, ids, L, mode="spec", last_only=True, ops=ops)
+        want = []
+        for step in range(n_new):
+            lg = logits[:, -1, :].float().numpy()
+            nxt = torch.tensor([osamp.sample_top_p_spec(lg[b], temperature, top_p, float(u[step, b]))[0] for b in range(batch)])
+            want.append(nxt)
+            logits, states = om.forward(tiny_bf16, nxt.reshape(-1, 1), L, states=states, mode="spec", ops=ops)
+        want = torch.stack(want, dim=1)
+        for use_graph in (True, False):
+            g = torch.Generator(device=dev).manual_seed(77)
+            got = model.generate(ids.to(dev), max_new_tokens=n_new, do_sample=True, top_p=top_p, temperature=temperature,
+                                 use_graph=use_graph, generator=g).cpu()
+            assert torch.equal(got[:, 12:], want), (batch, use_graph, got[:, 12:].tolist(), want.tolist())
+
+
 def test_half_precision_model_as_the_reference_script_runs_it(dev):
     """mmfreelm's generate.py runs the model with .cuda().half(): fp16 parameters and activations end to end.
     Prefill logits, greedy tokens and graph-replayed decode logits against the oracle's spec arithmetic in fp16."""
