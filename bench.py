@@ -198,6 +198,27 @@ def norm_bench(dev, m=16384, k=2048, iters=20):
             "rmsnorm_swishgate_GBs": round(3 * m * k * 2 / ms_g / 1e6, 1)}
 
 
+def sampler_bench(model, dev, n_new=256):
+    """Top-p sampling as the reference's generate.py asks for it (top_p 0.4, temperature 0.6): the sampling kernel
+    alone on one 32000-wide row, and generate() end to end (128-token prompt, prefill included) against greedy."""
+    import matmulfreellm_amd.functional as F_
+    g = torch.Generator(device=dev).manual_seed(5)
+    lg = (torch.randn(1, 32000, generator=g, device=dev) * 3).bfloat16()
+    u = torch.rand(1, generator=g, device=dev)
+    out = torch.empty(1, dtype=torch.int64, device=dev)
+    us = timed(lambda: F_.sample_top_p(lg, 0.4, 0.6, u, out=out), 50) * 1e3
+    ids = torch.randint(0, model.config.vocab_size, (1, 128), generator=g, device=dev)
+    res = {"sample_top_p_us_per_row_of_32000": round(us, 2)}
+    for name, kw in (("greedy", {}), ("top_p", dict(do_sample=True, top_p=0.4, temperature=0.6, generator=g))):
+        model.generate(ids, max_new_tokens=8, eos_token_id=None, **kw)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        model.generate(ids, max_new_tokens=n_new, eos_token_id=None, **kw)
+        torch.cuda.synchronize()
+        res[f"generate_{name}_tok_s"] = round(n_new / (time.perf_counter() - t0), 1)
+    return res
+
+
 def cpu_baseline(shape="1.3B", budget_s=25.0):
     """Reference PyTorch formulation (oracle literal mode) on the host cores: batch-1 decode of a
     1.3B-shape model, timed on 2 of its 24 layers plus the head and scaled to 24 layers."""
@@ -306,6 +327,7 @@ def main():
         extra["bitlinear_mfma_down_proj"] = mfma_bench(dev, 4096, 5632, 2048)
         extra["hgrn_scan"] = scan_bench(dev)
         extra["norms"] = norm_bench(dev)
+        extra["sampling"] = sampler_bench(model, dev)
         result["extra"] = extra
         del model, eng, eng1
         torch.cuda.empty_cache()
