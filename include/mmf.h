@@ -147,6 +147,16 @@ int mmf_bitlinear_mfma(const int8_t* codes_tiled, const float* deq, const int* q
                        const float* wdeq, int64_t seg_rows, const void* bias, const void* addend, void* out,
                        int64_t ldo, int64_t M, int64_t K, int64_t N, int out_dtype, int config, void* stream);
 
+/* mmf_bitlinear_mfma_swiglu: the tiled matrix-core contraction on the STACKED [gate; up] weight of the MLP
+ *   (N = 2 * I rows, I a multiple of 32: rows [0, I) = gate, [I, 2I) = up, as gate_proj stores them) with the activation
+ *   of mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py:55-59 (swiglu, mmfreelm/modules/activations.py:143) in its epilogue:
+ *     out[m, c] = T((g * u) / (1 + exp(-g))),  g = T(gate projection [m, c]),  u = T(up projection [m, c]),
+ *   i.e. exactly what mmf_bitlinear_mfma followed by mmf_swiglu on the two halves gives, without the [M, 2I] round trip.
+ *   out: [M, I] with leading dimension ldo (16-byte aligned rows: else MMF_ERR_ALIGN).  Other arguments as above. */
+int mmf_bitlinear_mfma_swiglu(const int8_t* codes_tiled, const float* deq, const int* qsum, const void* packed,
+                              const float* wdeq, int64_t seg_rows, void* out, int64_t ldo, int64_t M, int64_t K, int64_t N,
+                              int out_dtype, void* stream);
+
 /* ---- HGRN recurrence ------------------------------------------------------------------
  * x, g, o: [BH, T, D] contiguous (BH = batch * heads); h0 / ht: [BH, D] fp32 or NULL.
  * mmf_hgrn_recurrent replaces fused_recurrent_hgrn, mmfreelm/ops/hgrn/recurrent_fuse.py:

@@ -40,6 +40,7 @@ SIGNATURES = {
     "mmf_bitlinear_gemv_fused": (_i32, [_i32, _i32, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _f32, _ptr, _f32, _ptr, _ptr, _i64, _ptr,
                                         _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i32, _i32, _ptr]),
     "mmf_bitlinear_mfma": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _i32, _i32, _ptr]),
+    "mmf_bitlinear_mfma_swiglu": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _i64, _i64, _i64, _i32, _ptr]),
     "mmf_hgrn_recurrent": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i32, _ptr]),
     "mmf_hgrn_chunk": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i32, _i32, _ptr]),
     "mmf_hgrn_gate": (_i32, [_ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _ptr]),

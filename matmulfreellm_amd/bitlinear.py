@@ -78,11 +78,11 @@ class BitLinear(nn.Linear):
         fe = getattr(self, "fused_eps", None)
         return self.norm.eps if fe is None else fe
 
-    def forward_fused(self, x, prologue, addend=None):
+    def forward_fused(self, x, prologue, addend=None, epilogue=None):
         """forward() with the elementwise op that produces x folded into the same launch(es);
-        ``prologue`` as functional.bitlinear takes it."""
+        ``prologue`` / ``epilogue`` as functional.bitlinear takes them."""
         return F_.bitlinear(x, self.norm.weight, self.packed_weight(), bias=self.bias, eps=self.run_eps(), addend=addend,
-                            prologue=prologue)
+                            prologue=prologue, epilogue=epilogue)
 
     def forward(self, x):
         return layer_norm_linear_quant_fn(x, self.norm.weight, self.norm.bias, self.weight, self.bias,

@@ -218,6 +218,59 @@ __device__ __forceinline__ void mfma_epilogue_fast(const MfmaArgs& p, v16i (&acc
     }
 }
 
+// Epilogue of the gate/up contraction with the MLP activation folded in (mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py:55-59):
+// the wave's two n-blocks are the gate and the up projection of the same 32 channels, so a lane holds both operands of
+// out = T((g * u) / (1 + exp(-g))), g = T(gate), u = T(up), and the wave writes 32 columns of the [M, N/2] result.
+// Same conditions as the lean epilogue (accumulators started at -qsum, 16-byte stores).
+template <typename T, int WM>
+__device__ __forceinline__ void mfma_epilogue_swiglu(const MfmaArgs& p, v16i (&acc)[WM][2], const EpiScales<WM, 2>& sc,
+                                                     unsigned char* smem, int lane, int wave, int wm, int64_t mb0, int64_t nbg) {
+    T* out = static_cast<T*>(p.out);
+    constexpr int E = sizeof(T);
+    constexpr int RS = 32 * E + 16;               // LDS row stride of a wave's 32 x 32 staging tile
+    constexpr int CPR = 32 * E / 16;              // 16-byte chunks per row
+    constexpr int RPI = 64 / CPR;                 // rows covered by one 64-lane store
+    unsigned char* stage = smem + wave * (32 * RS);
+    const int half = lane >> 5, mloc = lane & 31;
+    const int cc = lane % CPR, rsub = lane / CPR;
+    const int64_t nseg = p.N >> 1;
+    const int64_t m_first = (mb0 + wm * WM) * 32, n_first = nbg * 32;
+    const bool interior = m_first + WM * 32 <= p.M && n_first + 32 <= nseg;
+    const int64_t n = n_first + cc * (16 / E);
+    const int64_t lane_off = (m_first + rsub) * p.ldo + n;
+    unsigned char* wr = stage + mloc * RS + 4 * half * E;
+    const unsigned char* rd = stage + rsub * RS + cc * 16;
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+        const float dq = sc.dq[i];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float o[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const float gv = mmf_round_to<T>(__fmul_rn(__fmul_rn((float)acc[i][0][4 * g + t], dq), sc.wdq[0]));
+                const float uv = mmf_round_to<T>(__fmul_rn(__fmul_rn((float)acc[i][1][4 * g + t], dq), sc.wdq[1]));
+                o[t] = __fdiv_rn(__fmul_rn(gv, uv), __fadd_rn(1.0f, mmf_exp(-gv)));
+            }
+            unsigned char* w = wr + (8 * g) * E;
+            if constexpr (E == 2) *reinterpret_cast<uint2*>(w) = make_uint2(pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]));
+            else *reinterpret_cast<float4*>(w) = make_float4(o[0], o[1], o[2], o[3]);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int r0 = 0; r0 < 32; r0 += RPI) {
+            const int64_t off = lane_off + (int64_t)(i * 32 + r0) * p.ldo;
+            if (interior || (m_first + i * 32 + r0 + rsub < p.M && n < nseg))
+                *reinterpret_cast<uint4*>(out + off) = *reinterpret_cast<const uint4*>(rd + r0 * RS);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
 template <typename T, int WGM, int WGN, int WM, int WN, int KSL>
 __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs p) {
     constexpr int NT = 64 * WGM * WGN;
@@ -350,7 +403,9 @@ typedef __attribute__((address_space(1))) const void* mmf_glb_ptr;
 // boundaries therefore carry no synchronisation: the A fragments of the next k-block's first
 // step are read while the current one's last MFMAs run, and the matrix pipe never drains.
 // FAST (chosen by the launcher): 16-byte stores possible and no bias -> lean epilogue, accumulators start at -qsum.
-template <typename T, int WGM, int WGN, int WM, int WN, bool FAST>
+// SWI: the weight is the stacked [gate; up] projection (N = 2 * I): a wave's two n-blocks are the gate and the up rows
+// of the same 32 channels, a workgroup tile covers WGN such channel blocks, and the epilogue writes swiglu(gate, up).
+template <typename T, int WGM, int WGN, int WM, int WN, bool FAST, bool SWI = false>
 __global__ __launch_bounds__(64 * WGM * WGN, (WM * WN <= 4 ? 4 : 1))   // small wave tiles: 4 waves per SIMD = two workgroups per CU
 void bitlinear_mfma_dma3_kernel(MfmaArgs p) {
     constexpr int NW = WGM * WGN;
@@ -384,9 +439,20 @@ void bitlinear_mfma_dma3_kernel(MfmaArgs p) {
     const int64_t MB = (p.M + 31) >> 5, NB = (p.N + 31) >> 5;
     const int KB = (int)(p.Kp >> 7);
     const int64_t KG = p.Kp >> 4;
-    const int64_t mb0 = tile_m * BMB, nb0 = tile_n * BNB + wn * WN;
+    static_assert(!SWI || (WN == 2 && FAST), "the swiglu epilogue pairs a gate and an up n-block per wave");
+    const int64_t NBs = NB >> 1;                                  // SWI: n-blocks per stacked segment
+    const int64_t mb0 = tile_m * BMB, nb0 = SWI ? tile_n * WGN + wn : tile_n * BNB + wn * WN;
+    // the n-block behind accumulator column j (columns past the end re-read a valid block and are never stored)
+    auto nblock = [&](int j) -> int64_t {
+        if constexpr (SWI) return (nb0 < NBs ? nb0 : NBs - 1) + j * NBs;
+        else return nb0 + j < NB ? nb0 + j : NB - 1;
+    };
     EpiScales<WM, WN> sc;
     mfma_prefetch_scales<WM, WN>(p, sc, lane, wm, mb0, nb0);
+    if constexpr (SWI) {
+#pragma unroll
+        for (int j = 0; j < WN; ++j) sc.wdq[j] = p.wdeq[(uint32_t)(nblock(j) * 32) / (uint32_t)p.seg_rows];
+    }
 
     auto dma_block = [&](int kb, int boff) {                      // k-block kb -> buffer at byte offset boff
 #pragma unroll
@@ -403,7 +469,7 @@ void bitlinear_mfma_dma3_kernel(MfmaArgs p) {
     auto load_b = [&](int kb, uint4 (&dst)[WN]) {                 // unconditional: the barrier's vmcnt counts on WN loads
 #pragma unroll
         for (int j = 0; j < WN; ++j) {
-            const int64_t nb = nb0 + j < NB ? nb0 + j : NB - 1;   // columns past N are never stored
+            const int64_t nb = nblock(j);
             const int kbc = kb < KB ? kb : KB - 1;                // past the end: never consumed
             dst[j] = p.b[(nb * KB + kbc) * 64 + lane];
         }
@@ -475,8 +541,30 @@ void bitlinear_mfma_dma3_kernel(MfmaArgs p) {
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);            // the trailing DMA must not land in the epilogue's staging area
     __syncthreads();
-    if constexpr (FAST) mfma_epilogue_fast<T, WM, WN>(p, acc, sc, smem, lane, wave, wm, mb0, nb0);
+    if constexpr (SWI) mfma_epilogue_swiglu<T, WM>(p, acc, sc, smem, lane, wave, wm, mb0, nb0);
+    else if constexpr (FAST) mfma_epilogue_fast<T, WM, WN>(p, acc, sc, smem, lane, wave, wm, mb0, nb0);
     else mfma_epilogue<T, WM, WN>(p, acc, sc, smem, lane, wave, wm, mb0, nb0);
+}
+
+// The 64 x 512 tile on the stacked [gate; up] weight with the swiglu epilogue: a tile is 64 rows x 256 channels.
+template <typename T>
+int launch_mfma_dma3_swiglu(MfmaArgs a, hipStream_t s) {
+    constexpr int WGM = 1, WGN = 8, WM = 2, WN = 2;
+    a.tiles_m = (int)mmf_ceil_div(a.M, WGM * WM * 32);
+    a.tiles_n = (int)mmf_ceil_div(a.N / 2, WGN * 32);
+    size_t lds = 3u * (WGM * WM) * 4096u;
+    const size_t lds_epi = (size_t)(WGM * WGN) * 32u * (32u * sizeof(T) + 16u);
+    if (lds_epi > lds) lds = lds_epi;
+    a.vec_store = 1;
+    auto kern = bitlinear_mfma_dma3_kernel<T, WGM, WGN, WM, WN, true, true>;
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)lds);
+        if (e != hipSuccess) return (int)e;
+    }
+    kern<<<dim3((unsigned)((int64_t)a.tiles_m * a.tiles_n)), dim3(64 * WGM * WGN), lds, s>>>(a);
+    MMF_CHECK_LAUNCH();
+    return 0;
 }
 
 template <typename T, int WGM, int WGN, int WM, int WN>
@@ -688,6 +776,29 @@ int mmf_bitlinear_mfma(const int8_t* codes_tiled, const float* deq, const int* q
         case MMF_F32: return dispatch_mfma<float>(a, config, stream);
         case MMF_BF16: return dispatch_mfma<bf16_t>(a, config, stream);
         case MMF_F16: return dispatch_mfma<f16_t>(a, config, stream);
+    }
+    return MMF_ERR_ARG;
+}
+
+int mmf_bitlinear_mfma_swiglu(const int8_t* codes_tiled, const float* deq, const int* qsum, const void* packed,
+                              const float* wdeq, int64_t seg_rows, void* out, int64_t ldo, int64_t M, int64_t K, int64_t N,
+                              int out_dtype, void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (M < 0 || K <= 0 || N <= 0 || N % 64 != 0 || seg_rows <= 0 || seg_rows % 32 != 0 || ldo < N / 2 || N > 0x7fffffff)
+        return MMF_ERR_ARG;
+    if (M == 0) return 0;
+    if (!codes_tiled || !deq || !qsum || !packed || !wdeq || !out) return MMF_ERR_ARG;
+    const int64_t per_vec = out_dtype == MMF_F32 ? 4 : 8;
+    if ((reinterpret_cast<uintptr_t>(codes_tiled) & 15u) || (reinterpret_cast<uintptr_t>(packed) & 15u) ||
+        (reinterpret_cast<uintptr_t>(out) & 15u) || ldo % per_vec != 0)
+        return MMF_ERR_ALIGN;
+    MfmaArgs a{};
+    a.a = codes_tiled; a.b = static_cast<const uint4*>(packed); a.deq = deq; a.qsum = qsum; a.wdeq = wdeq;
+    a.out = out; a.M = M; a.N = N; a.Kp = mmf_round_up(K, 128); a.seg_rows = seg_rows; a.ldo = ldo;
+    switch (out_dtype) {
+        case MMF_F32: return launch_mfma_dma3_swiglu<float>(a, stream);
+        case MMF_BF16: return launch_mfma_dma3_swiglu<bf16_t>(a, stream);
+        case MMF_F16: return launch_mfma_dma3_swiglu<f16_t>(a, stream);
     }
     return MMF_ERR_ARG;
 }

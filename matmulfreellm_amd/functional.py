@@ -3,6 +3,7 @@ import torch
 
 from . import _lib as L
 
+SWIGLU_EPILOGUE_MIN_M = 512      # rows from which the gate/up contraction runs tiled and can carry the swiglu in its epilogue
 GEMV_MAX_M = 8      # rows handled by the fused norm+quant+GEMV launch (every workgroup redoes the row's prologue,
                     # which stops paying off around 8 rows); above: quantise once per row, then the matrix cores
 
@@ -210,6 +211,26 @@ def bitlinear_mfma(q_tiled, deq, qsum, pw, m, out_dtype, bias=None, config=-1, o
     return out
 
 
+def bitlinear_mfma_swiglu(q_tiled, deq, qsum, pw, m, out_dtype):
+    """The tiled matrix-core contraction on the stacked [gate; up] weight with swiglu in its epilogue -> [m, N/2]."""
+    lib = L.load()
+    dev = L.require_gpu(q_tiled, deq, qsum, pw.packed)
+    inter = pw.n // 2
+    out = torch.empty(m, inter, dtype=out_dtype, device=dev)
+    with torch.cuda.device(dev):
+        L.check(lib.mmf_bitlinear_mfma_swiglu(q_tiled.data_ptr(), deq.data_ptr(), qsum.data_ptr(), pw.packed.data_ptr(),
+                                              pw.wdeq.data_ptr(), pw.seg_rows, out.data_ptr(), inter, m, pw.k, pw.n,
+                                              L.dtype_id(out_dtype), L.stream()), "mmf_bitlinear_mfma_swiglu")
+    return out
+
+
+def swiglu_epilogue_fits(m, pw, dtype):
+    """Whether bitlinear_mfma_swiglu serves this problem: enough rows for the tiled kernel, whole 32-channel blocks,
+    16-byte rows of the result."""
+    inter = pw.n // 2
+    return m >= SWIGLU_EPILOGUE_MIN_M and pw.n % 64 == 0 and inter % (4 if dtype == torch.float32 else 8) == 0
+
+
 def bitlinear_gemv(x2, norm_weight, pw, eps, bias=None, addend=None):
     lib = L.load()
     dev = L.require_gpu(x2, norm_weight, pw.packed, bias)
@@ -233,7 +254,7 @@ def bitlinear_gemv(x2, norm_weight, pw, eps, bias=None, addend=None):
 _PROLOGUES = {"norm": (1, 1), "resnorm": (2, 2), "gatednorm": (3, 5), "swiglu": (4, 4)}
 
 
-def _bitlinear_prologue(x, norm_weight, pw, bias, eps, addend, prologue):
+def _bitlinear_prologue(x, norm_weight, pw, bias, eps, addend, prologue, epilogue=None):
     """BitLinear with the op in front of it folded into the same launch (M <= GEMV_MAX_M) or into the quantiser
     (larger M).  prologue: ("norm", w1, eps1) | ("resnorm", residual, w1, eps1) | ("gatednorm", gate, w1, eps1)
     | ("swiglu", up).  x and the second operand may be column slices of a wider tensor.
@@ -265,7 +286,9 @@ def _bitlinear_prologue(x, norm_weight, pw, bias, eps, addend, prologue):
     if w1c is not None and nw is not None and w1c.dtype != nw.dtype:
         raise ValueError("the two norm weights must share a dtype")
     res_out = torch.empty(m, k, dtype=x2.dtype, device=dev) if kind == "resnorm" else None
-    out = torch.empty(m, pw.n, dtype=x2.dtype, device=dev)
+    if epilogue is not None:
+        _check_swiglu_epilogue(epilogue, m, pw, x2.dtype, bias, addend)
+    out = torch.empty(m, pw.n, dtype=x2.dtype, device=dev) if epilogue is None else None
     if bias is not None:
         bias = bias.detach().to(x2.dtype).contiguous()
     if addend is not None:
@@ -287,22 +310,34 @@ def _bitlinear_prologue(x, norm_weight, pw, bias, eps, addend, prologue):
             L.check(lib.mmf_rmsnorm_quant_fused(qid, x2.data_ptr(), ldx, L.ptr(a2), lda, None, 0, L.ptr(res_out), L.ptr(w1c), eps1,
                                                 L.ptr(nw), eps, None, None, q.data_ptr(), deq.data_ptr(), qsum.data_ptr(), m, k,
                                                 L.dtype_id(x2.dtype), L.dtype_id(wdt), L.stream()), "mmf_rmsnorm_quant_fused")
-            bitlinear_mfma(q, deq, qsum, pw, m, x2.dtype, bias, out=out, addend=addend)
-    out = out.reshape(*shp[:-1], pw.n)
+            if epilogue is None:
+                bitlinear_mfma(q, deq, qsum, pw, m, x2.dtype, bias, out=out, addend=addend)
+            else:
+                out = bitlinear_mfma_swiglu(q, deq, qsum, pw, m, x2.dtype)
+    out = out.reshape(*shp[:-1], out.shape[-1])
     return (out, res_out.reshape(shp)) if kind == "resnorm" else out
 
 
+def _check_swiglu_epilogue(epilogue, m, pw, dtype, bias, addend):
+    if epilogue != "swiglu":
+        raise ValueError("epilogue must be None or 'swiglu'")
+    if bias is not None or addend is not None or not swiglu_epilogue_fits(m, pw, dtype):
+        raise ValueError("the swiglu epilogue takes no bias or addend and needs swiglu_epilogue_fits(m, weight, dtype)")
+
+
 def bitlinear(x, norm_weight, pw, bias=None, eps=1e-8, residual=None, prenorm=False, residual_in_fp32=False,
-              path=None, addend=None, prologue=None):
+              path=None, addend=None, prologue=None, epilogue=None):
     """Fused BitLinear forward on x [..., K] -> [..., N] (x.dtype).
 
     path: None (by M), "gemv" or "mfma".  With a residual (or prenorm) the two-launch path is used.
     prologue: see _bitlinear_prologue (the elementwise op that produces this BitLinear's input, fused).
+    epilogue: "swiglu" on a stacked [gate; up] weight returns swiglu(gate, up) [..., N/2] from the contraction's own
+    epilogue (large M only: swiglu_epilogue_fits).
     """
     if prologue is not None:
         if residual is not None or prenorm or path is not None:
             raise ValueError("prologue= excludes residual=, prenorm= and path=")
-        return _bitlinear_prologue(x, norm_weight, pw, bias, eps, addend, prologue)
+        return _bitlinear_prologue(x, norm_weight, pw, bias, eps, addend, prologue, epilogue)
     lib = L.load()
     L.require_gpu(x)
     shp = x.shape
@@ -322,7 +357,11 @@ def bitlinear(x, norm_weight, pw, bias=None, eps=1e-8, residual=None, prenorm=Fa
     res = rmsnorm_quant(x, norm_weight, residual=residual, eps=eps, tiled=True, prenorm=prenorm,
                         residual_in_fp32=residual_in_fp32)
     q, deq, qsum = res[:3]
-    out = bitlinear_mfma(q, deq, qsum, pw, m, x.dtype, bias, addend=addend).reshape(*shp[:-1], pw.n)
+    if epilogue is not None:
+        _check_swiglu_epilogue(epilogue, m, pw, x.dtype, bias, addend)
+        out = bitlinear_mfma_swiglu(q, deq, qsum, pw, m, x.dtype).reshape(*shp[:-1], pw.n // 2)
+    else:
+        out = bitlinear_mfma(q, deq, qsum, pw, m, x.dtype, bias, addend=addend).reshape(*shp[:-1], pw.n)
     return (out, res[3]) if prenorm else out
 
 

@@ -69,11 +69,20 @@ class HGRNBitMLP(nn.Module):
         fused into down_proj's epilogue; with ``pre_norm`` (the block's mlp_norm) x is the attention
         output and the residual add + RMSNorm in front of gate_proj (:107) is folded into gate_proj."""
         inter = self.intermediate_size
+        rows = x.numel() // x.shape[-1]
+        # long prompts: the tiled gate/up contraction applies the swiglu itself and down_proj quantises its result
+        in_epilogue = (self.gate_proj.bias is None and x.is_cuda
+                       and F_.swiglu_epilogue_fits(rows, self.gate_proj.packed_weight(), x.dtype))
+        epilogue = "swiglu" if in_epilogue else None
         if pre_norm is not None:
-            y, residual = self.gate_proj.forward_fused(x, ("resnorm", residual, pre_norm.weight, pre_norm.eps))
+            y, residual = self.gate_proj.forward_fused(x, ("resnorm", residual, pre_norm.weight, pre_norm.eps), epilogue=epilogue)
+        elif in_epilogue:
+            y = self.gate_proj.forward_fused(x, None, epilogue=epilogue)
         else:
             y = self.gate_proj(x)
         addend = residual.contiguous() if residual is not None else None
+        if in_epilogue:
+            return self.down_proj.forward_fused(y, None, addend=addend)
         return self.down_proj.forward_fused(y[..., :inter], ("swiglu", y[..., inter:]), addend=addend)
 
 

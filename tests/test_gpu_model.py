@@ -516,3 +516,21 @@ def test_batch_128_decode_at_the_2p7b_shape_equals_batch_1_rows(dev):
         eng.check()
     del model, big, small
     torch.cuda.empty_cache()
+
+
+def test_long_prompt_with_the_swiglu_in_the_contraction_epilogue(dev, tiny_bf16, monkeypatch):
+    """640 prompt rows: gate_proj runs the tiled kernel with the swiglu in its epilogue.  Last-position logits and
+    recurrent states equal the oracle's, and the path that keeps the swiglu in down_proj's quantiser."""
+    import matmulfreellm_amd.functional as F_
+    torch.manual_seed(60)
+    ids = torch.randint(0, V, (5, 128))
+    ref, ref_states = om.forward(tiny_bf16, ids, L, mode="spec", last_only=True)
+    model = build(tiny_bf16, torch.bfloat16, dev)
+    assert F_.swiglu_epilogue_fits(640, model.model.layers[0].mlp.gate_proj.packed_weight(), torch.bfloat16)
+    out = model(input_ids=ids.to(dev), use_cache=True, logits_to_keep=1)
+    assert torch.equal(out.logits[:, -1].cpu(), ref[:, -1])
+    for c, r in zip(out.past_key_values, ref_states):
+        assert torch.equal(c[-1].reshape(5, -1).cpu(), r.reshape(5, -1).float())
+    monkeypatch.setattr(F_, "SWIGLU_EPILOGUE_MIN_M", 1 << 30)
+    out2 = model(input_ids=ids.to(dev), use_cache=True, logits_to_keep=1)
+    assert torch.equal(out2.logits, out.logits)

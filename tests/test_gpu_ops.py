@@ -425,3 +425,33 @@ def test_fp16_outputs_are_rounded_fp32_results(dev):
     assert torch.equal(y, on.rms_norm_spec(x, w, eps=1e-6))
     z = F().swiglu(x.to(dev), o.to(dev)).cpu()
     assert torch.equal(z, on.swiglu_spec(x, o))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,k,i", [(4096, 2048, 5632), (513, 512, 96), (70, 640, 32), (1000, 2560, 6912), (64, 128, 8000)])
+def test_mfma_swiglu_epilogue_equals_contraction_then_swiglu(dev, dtype, m, k, i):
+    """mmf_bitlinear_mfma_swiglu against the two ops it folds together (each checked against the oracle above): the
+    contraction on the stacked [gate; up] weight, then swiglu on the two halves."""
+    g = torch.Generator(device=dev).manual_seed(63)
+    x = torch.randn(m, k, generator=g, device=dev).to(dtype)
+    nw = (1 + 0.1 * torch.randn(k, generator=g, device=dev)).to(dtype)
+    pw = F().ternarize_pack((torch.randn(2 * i, k, generator=g, device=dev) * 0.02).to(dtype))
+    q, deq, qsum = F().rmsnorm_quant(x, nw, eps=1e-8, tiled=True)[:3]
+    full = F().bitlinear_mfma(q, deq, qsum, pw, m, dtype)
+    want = F().swiglu(full[:, :i], full[:, i:])
+    got = F().bitlinear_mfma_swiglu(q, deq, qsum, pw, m, dtype)
+    assert got.shape == (m, i) and torch.equal(got, want)
+
+
+def test_mfma_swiglu_rejects_what_it_cannot_run(dev):
+    from matmulfreellm_amd._lib import load
+    lib = load()
+    z = torch.zeros(1 << 16, device=dev)
+    p = z.data_ptr()
+    call = lambda n, ldo, out=p, seg=32: lib.mmf_bitlinear_mfma_swiglu(p, p, p, p, p, seg, out, ldo, 8, 128, n, 1, None)
+    assert call(96, 48) == -1           # the two halves are not whole 32-row blocks
+    assert call(128, 32) == -1          # rows of the result overlap
+    assert call(128, 68) == -3          # rows of the result are not 16-byte aligned
+    assert call(128, 64, out=p + 2) == -3
+    assert call(128, 64, seg=48) == -1
+    assert call(128, 64, out=None) == -1
