@@ -92,3 +92,29 @@ def test_sample_top_p_random_shapes(dev, case):
     got = F().sample_top_p(logits.to(dev), top_p, temperature, u.to(dev)).cpu().tolist()
     want = [osamp.sample_top_p_spec(logits[r].float().numpy(), temperature, top_p, float(u[r]))[0] for r in range(rows)]
     assert got == want
+
+
+MODELS = _cases(105, 24, lambda r: (r.choice([torch.bfloat16, torch.float32, torch.float16]), r.choice([128, 256, 384, 640]), r.randint(1, 3),
+                                    r.choice([517, 1000, 4099, 32]), r.choice([1, 1, 2, 5, 9, 20]), r.randint(1, 40)))
+
+
+@pytest.mark.parametrize("case", MODELS, ids=lambda c: f"{str(c[0]).split('.')[-1]}-H{c[1]}-L{c[2]}-V{c[3]}-B{c[4]}-T{c[5]}")
+def test_model_greedy_random_configurations(dev, case):
+    """Small random model configurations (ragged vocabularies, 1-3 layers, batches on every decode path): prefill +
+    greedy tokens equal the oracle's on the module path and through the decode engine's graph."""
+    import matmulfreellm_amd as mm
+    from oracle import model as om
+    dtype, hidden, layers, vocab, batch, t = case
+    params = om.init_params(vocab, hidden, layers, seed=7, dtype=dtype)
+    cfg = mm.HGRNBitConfig(vocab_size=vocab, hidden_size=hidden, num_hidden_layers=layers)
+    model = mm.HGRNBitForCausalLM(cfg)
+    model.load_state_dict(params, strict=True)
+    model = model.to(device=dev, dtype=dtype).eval()
+    model.generation_config.eos_token_id = None                # tiny vocabularies hit the default end-of-sequence id (2)
+    torch.manual_seed(6000 + hidden + t)
+    ids = torch.randint(0, vocab, (batch, t))
+    n_new = 5
+    ref_toks, _ = om.greedy(params, ids, layers, n_new, mode="spec")
+    for use_graph in (False, True):
+        got = model.generate(ids.to(dev), max_new_tokens=n_new, use_graph=use_graph).cpu()
+        assert torch.equal(got[:, t:], ref_toks), (use_graph, got[:, t:].tolist(), ref_toks.tolist())
