@@ -195,6 +195,15 @@ int mmf_embedding(const void* table, const int64_t* ids, void* out, int64_t rows
                   int dtype, void* stream);
 int mmf_argmax(const void* logits, int64_t ld, int64_t rows, int64_t V, int64_t* out, int dtype, void* stream);
 
+/* ---- next-token loss (forward only) -----------------------------------------------------------
+ * mmf_cross_entropy_fwd replaces the loss that HGRNBitForCausalLM.forward computes from labels
+ *   (mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py:388-397: FusedCrossEntropyLoss / nn.CrossEntropyLoss on
+ *   logits.view(-1, V); forward of mmfreelm/modules/fused_cross_entropy.py with its default zero smoothing and z-loss):
+ *   loss[r] = logsumexp(logits[r, :]) - logits[r, labels[r]] in fp32, 0 where labels[r] == ignore_index (or lies
+ *   outside [0, V)).  The caller shifts the labels and takes the mean over the rows that count.  No backward. */
+int mmf_cross_entropy_fwd(const void* logits, int64_t ld, const int64_t* labels, int64_t ignore_index, float* loss,
+                          int64_t rows, int64_t V, int dtype, void* stream);
+
 /* ---- top-p (nucleus) sampling of the next token -----------------------------------------------
  * mmf_sample_top_p replaces, per decoded token of the loop that mmfreelm's generate.py:11 runs
  *   (model.generate(do_sample=True, top_p=0.4, temperature=0.6)), what transformers' sampling path does with the

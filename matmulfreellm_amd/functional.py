@@ -519,3 +519,22 @@ def sample_top_p(logits, top_p, temperature, u, out=None):
 def sample_top_p_max_vocab():
     """Widest row sample_top_p accepts."""
     return int(L.load().mmf_sample_top_p_max_vocab())
+
+
+def cross_entropy(logits, labels, ignore_index=-100):
+    """Mean next-token cross entropy as nn.CrossEntropyLoss()(logits.view(-1, V), labels.view(-1)) gives it, computed
+    in fp32 from logits of any supported dtype (forward only); labels int64, already shifted by the caller.
+    Returns a 0-dim fp32 tensor (NaN when every label is ignored, as torch returns)."""
+    lib = L.load()
+    dev = L.require_gpu(logits, labels)
+    v = logits.shape[-1]
+    l2 = _as_2d(logits)
+    lab = labels.reshape(-1).to(torch.int64).contiguous()
+    if lab.numel() != l2.shape[0]:
+        raise ValueError("one label per row of logits")
+    rows = torch.empty(l2.shape[0], dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        L.check(lib.mmf_cross_entropy_fwd(l2.data_ptr(), l2.stride(0), lab.data_ptr(), int(ignore_index), rows.data_ptr(),
+                                          l2.shape[0], v, L.dtype_id(l2.dtype), L.stream()), "mmf_cross_entropy_fwd")
+    counted = ((lab != ignore_index) & (lab >= 0) & (lab < v)).sum()
+    return rows.sum() / counted

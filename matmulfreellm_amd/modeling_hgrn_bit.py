@@ -11,7 +11,7 @@ Differences, all on the host side:
     PreTrainedModel a generate());
   * ``logits_to_keep`` lets a caller ask for the last positions' logits only (the
     reference projects all T positions through the 32000-wide head);
-  * the loss head is not part of the inference path: passing ``labels`` raises.
+  * ``labels`` gives the evaluation loss (forward only, fp32): there is no backward.
 """
 from __future__ import annotations
 
@@ -296,8 +296,7 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
                 output_attentions: Optional[bool] = None, output_hidden_states: Optional[bool] = None,
                 return_dict: Optional[bool] = None, logits_to_keep: int = 0) -> Union[Tuple, CausalLMOutputWithPast]:
         if labels is not None:
-            raise NotImplementedError("the loss head (fused cross entropy) is a training component; "
-                                      "this package implements the inference forward only")
+            logits_to_keep = 0                           # the loss scores every position
         return_dict = return_dict if return_dict is not None else bool(getattr(self.config, "return_dict", True))
         outputs = self.model(input_ids=input_ids, attention_mask=attention_mask, inputs_embeds=inputs_embeds,
                              past_key_values=past_key_values, use_cache=use_cache,
@@ -307,9 +306,15 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
         if logits_to_keep:
             hidden_states = hidden_states[:, -logits_to_keep:, :]
         logits = self.lm_head(hidden_states)
+        loss = None
+        if labels is not None:
+            # as mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py:388-397: position t is scored against token t + 1
+            labels = labels.to(logits.device)
+            targets = torch.cat((labels[..., 1:], torch.full_like(labels[:, :1], -100)), 1)
+            loss = F_.cross_entropy(logits, targets, ignore_index=-100)
         if not return_dict:
-            return tuple(x for x in (logits, outputs.past_key_values, outputs.hidden_states) if x is not None)
-        return CausalLMOutputWithPast(loss=None, logits=logits, past_key_values=outputs.past_key_values,
+            return tuple(x for x in (loss, logits, outputs.past_key_values, outputs.hidden_states) if x is not None)
+        return CausalLMOutputWithPast(loss=loss, logits=logits, past_key_values=outputs.past_key_values,
                                       hidden_states=outputs.hidden_states, attentions=None)
 
     # ------------------------------------------------------------------ generation
