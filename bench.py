@@ -198,6 +198,18 @@ def norm_bench(dev, m=16384, k=2048, iters=20):
             "rmsnorm_swishgate_GBs": round(3 * m * k * 2 / ms_g / 1e6, 1)}
 
 
+def loss_bench(dev, m=4096, v=32000, iters=20):
+    """Evaluation loss of m rows of v-wide bf16 logits (one read of the logits)."""
+    import matmulfreellm_amd.functional as F_
+    g = torch.Generator(device=dev).manual_seed(6)
+    logits = torch.randn(m, v, generator=g, device=dev).bfloat16()
+    targets = torch.randint(0, v, (m,), generator=g, device=dev)
+    lib, rows = F_.L.load(), torch.empty(m, dtype=torch.float32, device=dev)
+    ms = timed(lambda: F_.L.check(lib.mmf_cross_entropy_fwd(logits.data_ptr(), v, targets.data_ptr(), -100, rows.data_ptr(), m, v,
+                                                            F_.L.dtype_id(logits.dtype), F_.L.stream()), "mmf_cross_entropy_fwd"), iters)
+    return {"shape": [m, v], "ms": round(ms, 4), "GBs": round(m * v * 2 / ms / 1e6, 1)}
+
+
 def sampler_bench(model, dev, n_new=256):
     """Top-p sampling as the reference's generate.py asks for it (top_p 0.4, temperature 0.6): the sampling kernel
     alone on one 32000-wide row, and generate() end to end (128-token prompt, prefill included) against greedy."""
@@ -328,6 +340,7 @@ def main():
         extra["hgrn_scan"] = scan_bench(dev)
         extra["norms"] = norm_bench(dev)
         extra["sampling"] = sampler_bench(model, dev)
+        extra["cross_entropy"] = loss_bench(dev)
         result["extra"] = extra
         del model, eng, eng1
         torch.cuda.empty_cache()
