@@ -373,13 +373,13 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
         choose = None
         if do_sample:
             temperature = max(float(temperature), 1e-6)
+            # every uniform number of the run is drawn here, so the random stream does not depend on the path taken
+            g_dev = generator.device if generator is not None else input_ids.device
+            uniforms = torch.rand(max_new_tokens, B, generator=generator, device=g_dev).to(input_ids.device)
             if logits.shape[-1] <= F_.sample_top_p_max_vocab():
-                # every uniform number of the run is drawn here, so the random stream does not depend on the path taken
-                g_dev = generator.device if generator is not None else input_ids.device
-                uniforms = torch.rand(max_new_tokens, B, generator=generator, device=g_dev).to(input_ids.device)
                 choose = lambda lg, step, out=None: F_.sample_top_p(lg, top_p, temperature, uniforms[step], out=out)
             else:
-                choose = lambda lg, step, out=None: _sample_top_p(lg.float(), top_p, temperature, generator, out)
+                choose = lambda lg, step, out=None: _sample_top_p(lg.float(), top_p, temperature, uniforms[step], out)
         first = choose(logits, 0) if do_sample else F_.argmax(logits)
         if engine is not None:
             pick = (lambda step: choose(engine.logits, step, engine.tok)) if do_sample else None
@@ -435,15 +435,17 @@ def _self_feeding(engine, first, max_new_tokens, eos_token_id, pad_token_id, chu
     return seq.contiguous()
 
 
-def _sample_top_p(logits, top_p, temperature, generator, out=None):
-    """Vocabularies wider than the sampling kernel holds: the same nucleus with library calls."""
-    probs = torch.softmax(logits / max(temperature, 1e-6), dim=-1)
+def _sample_top_p(logits, top_p, temperature, u, out=None):
+    """Vocabularies wider than the sampling kernel holds: the same nucleus and the same inverse CDF (kept tokens in
+    index order, one uniform number per row) with library calls in fp32."""
+    probs = torch.softmax(logits / temperature, dim=-1)
     sp, si = torch.sort(probs, dim=-1, descending=True)
-    keep = (sp.cumsum(-1) - sp) < top_p
-    sp = sp * keep
-    sp = sp / sp.sum(-1, keepdim=True)
-    choice = torch.multinomial(sp, 1, generator=generator)
-    tok = si.gather(-1, choice).squeeze(-1)
+    keep_sorted = (sp.cumsum(-1) - sp) < max(float(top_p), 0.0)
+    keep_sorted[..., 0] = True                                   # at least the most probable token
+    keep = torch.zeros_like(keep_sorted).scatter_(-1, si, keep_sorted)
+    cdf = (probs * keep).cumsum(-1)
+    target = u.to(cdf.dtype).clamp(0.0, 1.0).reshape(-1, 1) * cdf[..., -1:]
+    tok = torch.searchsorted(cdf, target, right=True).squeeze(-1).clamp_(max=logits.shape[-1] - 1)
     if out is not None:
         out.copy_(tok)
         return out

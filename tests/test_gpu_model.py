@@ -534,3 +534,28 @@ def test_long_prompt_with_the_swiglu_in_the_contraction_epilogue(dev, tiny_bf16,
     monkeypatch.setattr(F_, "SWIGLU_EPILOGUE_MIN_M", 1 << 30)
     out2 = model(input_ids=ids.to(dev), use_cache=True, logits_to_keep=1)
     assert torch.equal(out2.logits, out.logits)
+
+
+def test_wide_vocabulary_sampling_fallback(dev, tiny_bf16, monkeypatch):
+    """Vocabularies beyond the sampling kernel's width take library calls with the same nucleus rule and the same
+    inverse CDF of the same uniform numbers.  On peaked rows the two agree except where a draw lands within fp32
+    rounding of a boundary (library sums in fp32 against exact integer masses); forced on a 32000-wide model, the
+    fallback gives the same tokens through the decode graph and through the module path."""
+    import matmulfreellm_amd.functional as F_
+    from matmulfreellm_amd.modeling_hgrn_bit import _sample_top_p
+    g = torch.Generator(device=dev).manual_seed(71)
+    logits = (torch.randn(64, 2000, generator=g, device=dev) * 3).bfloat16()
+    u = torch.rand(64, generator=g, device=dev)
+    a = F_.sample_top_p(logits, 0.9, 0.8, u)
+    b = _sample_top_p(logits.float(), 0.9, 0.8, u)
+    assert (a == b).sum().item() >= 62, (a != b).nonzero().flatten().tolist()
+    model = build(tiny_bf16, torch.bfloat16, dev)
+    torch.manual_seed(70)
+    ids = torch.randint(0, V, (3, 8), device=dev)
+    kw = dict(max_new_tokens=10, do_sample=True, top_p=0.4, temperature=0.6)
+    monkeypatch.setattr(F_, "sample_top_p_max_vocab", lambda: 0)
+    outs = [model.generate(ids, generator=torch.Generator(device=dev).manual_seed(5), use_graph=use_graph, **kw)
+            for use_graph in (True, False)]
+    assert outs[0].shape == (3, 18) and torch.equal(outs[0], outs[1])
+    cpu_gen = model.generate(ids, generator=torch.Generator().manual_seed(5), **kw)      # a CPU generator is accepted too
+    assert cpu_gen.shape == (3, 18)
