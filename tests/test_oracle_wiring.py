@@ -1,0 +1,258 @@
+"""Known-answer pin of the oracle's MODEL WIRING whose expected values do not come from ``oracle/``.
+
+``reference_forward`` below is a straight-line float64 numpy restatement written from the reference's text only:
+  HGRNBitAttention.forward   mmfreelm/layers/hgrn_bit.py:110-140
+  HGRNBitMLP.forward         mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py:55-59
+  HGRNBitBlock.forward       modeling_hgrn_bit.py:97-109
+  HGRNBitModel.forward       modeling_hgrn_bit.py:212, 231-238, 262
+  lm_head                    modeling_hgrn_bit.py:386
+  BitLinear                  mmfreelm/ops/fusedbitnet.py:556-581 with activation_quant :26-28, weight_quant :43-45
+  RMSNorm                    mmfreelm/modules/layernorm.py:73-87
+  gated norm                 mmfreelm/modules/fused_norm_gate.py:123-128 (y = norm(x) * w * o * sigmoid(o))
+  swiglu                     mmfreelm/modules/activations.py:115-119
+  recurrence                 mmfreelm/ops/hgrn/naive.py:22-28
+It imports nothing from ``oracle`` and shares no helper with it.  The model is tiny and hand-built: every latent
+weight matrix is c * T with T a known ternary matrix, so weight_quant gives back exactly T with step c * (share of
+non-zeros) and every BitLinear is ``codes . T^T * deq * wdeq`` by hand; g_norm / block norm / inner norm weights are
+non-trivial and differ from each other; lower_bounds are non-zero; L = 3.
+
+float64 against the oracle's fp32: the two agree to ~1e-5 unless an int8 code sits on a rounding tie, so the
+restatement also reports the smallest distance of any pre-rounding value to a tie and the test requires a margin.
+
+``test_mutants_of_the_oracle_are_caught`` rewrites the oracle's forward with first-order wiring mistakes (operand
+order, a dropped or misplaced residual, wrong norm input, shifted lower-bound schedule ...) and requires this
+known answer to reject each of them.
+"""
+import inspect
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import model as om
+
+V, H, I, L = 24, 8, 16, 3
+RMS_EPS, BL_EPS = 1e-6, 1e-8
+
+
+# ------------------------------------------------------------------ the independent restatement (numpy float64)
+def _sigmoid(v):
+    return 1.0 / (1.0 + np.exp(-v))
+
+
+def _rms_norm(x, w, eps):
+    return x / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + eps) * w
+
+
+class _Margin:
+    """Smallest distance of a value about to be rounded from the nearest tie (k + 0.5)."""
+    def __init__(self):
+        self.value = 1.0
+
+    def see(self, v):
+        self.value = min(self.value, float(np.min(np.abs(np.abs(v - np.floor(v)) - 0.5))))
+
+
+def _bit_linear(x, latent, norm_w, margin):
+    """x [..., K], latent [N, K]: RMSNorm(eps 1e-8) -> activation_quant -> weight_quant -> linear."""
+    y = _rms_norm(x, norm_w, BL_EPS)
+    s = 127.0 / np.maximum(np.max(np.abs(y), axis=-1, keepdims=True), 1e-5)
+    margin.see(y * s)
+    q = np.clip(np.rint(y * s), -128, 127)                      # int8 codes
+    ws = 1.0 / max(float(np.mean(np.abs(latent))), 1e-5)
+    t = np.clip(np.rint(latent * ws), -1, 1)                    # ternary codes
+    return (q @ t.T) / s / ws
+
+
+def reference_forward(p, ids, margin, states=None):
+    """ids [B, T] -> (logits [B, T, V], final recurrent states [L][B, H])."""
+    n_layers = p["model.lower_bounds"].shape[0]
+    h = p["model.embeddings.weight"][ids]                       # modeling_hgrn_bit.py:212
+    lbs = np.exp(p["model.lower_bounds"])
+    lbs = lbs / lbs.sum(axis=0, keepdims=True)                  # softmax over LAYERS (:232)
+    lbs = np.cumsum(lbs, axis=0) - lbs[0]                       # :233
+    finals = []
+    for li in range(n_layers):
+        b = f"model.layers.{li}."
+        residual = h                                            # :97
+        x = _rms_norm(h, p[b + "attn_norm.weight"], RMS_EPS)    # :98
+        # ---- attention, layers/hgrn_bit.py:110-140
+        i = _bit_linear(x, p[b + "attn.i_proj.weight"], p[b + "attn.i_proj.norm.weight"], margin)
+        f = _bit_linear(x, p[b + "attn.f_proj.weight"], p[b + "attn.f_proj.norm.weight"], margin)
+        f = _sigmoid(f)                                         # :113
+        if li > 0:                                              # :115
+            f = lbs[li] + (1 - lbs[li]) * f
+        i = i * _sigmoid(i) * (1 - f)                           # swiglu(i, 1 - f), :117
+        state = np.zeros_like(i[:, 0]) if states is None else states[li]
+        o = np.empty_like(i)
+        for t in range(i.shape[1]):                             # naive.py:25-27
+            state = f[:, t] * state + i[:, t]
+            o[:, t] = state
+        finals.append(state)
+        g = _bit_linear(x, p[b + "attn.g_proj.weight"], p[b + "attn.g_proj.norm.weight"], margin)
+        o = _rms_norm(g, p[b + "attn.g_norm.weight"], RMS_EPS) * o * _sigmoid(o)      # g_norm(g_proj(x), o), :139
+        a = _bit_linear(o, p[b + "attn.o_proj.weight"], p[b + "attn.o_proj.norm.weight"], margin)   # :140
+        # ---- block, modeling_hgrn_bit.py:107-109
+        residual = a + residual                                 # mlp_norm(h, residual, prenorm=True)
+        x = _rms_norm(residual, p[b + "mlp_norm.weight"], RMS_EPS)
+        y = _bit_linear(x, p[b + "mlp.gate_proj.weight"], p[b + "mlp.gate_proj.norm.weight"], margin)   # :56
+        gate, up = y[..., :y.shape[-1] // 2], y[..., y.shape[-1] // 2:]                                  # :57
+        z = _bit_linear(gate * _sigmoid(gate) * up, p[b + "mlp.down_proj.weight"],
+                        p[b + "mlp.down_proj.norm.weight"], margin)                                      # :58
+        h = residual + z                                        # :109
+    h = _rms_norm(h, p["model.norm.weight"], RMS_EPS)           # :262
+    return _bit_linear(h, p["lm_head.weight"], p["lm_head.norm.weight"], margin), finals   # :386
+
+
+# ------------------------------------------------------------------ the hand-built model
+def _ternary(rng, n, k, c):
+    """c * T with T in {-1, 0, 1}; every row and column keeps a non-zero."""
+    t = rng.integers(-1, 2, size=(n, k)).astype(np.float64)
+    for r in range(n):
+        t[r, (r * 3 + 1) % k] = 1.0 if r % 2 else -1.0
+    for col in range(k):
+        if not t[:, col].any():
+            t[col % n, col] = 1.0
+    return c * t, t
+
+
+def build(seed):
+    rng = np.random.default_rng(seed)
+    p, tern = {}, {}
+
+    def vec(n):
+        return rng.uniform(0.5, 1.5, size=n) * rng.choice([-1.0, 1.0], size=n, p=[0.2, 0.8])
+
+    def lin(name, n, k):
+        c = float(rng.uniform(0.15, 0.6))     # large enough that a layer moves the residual stream visibly
+        p[name + ".weight"], tern[name] = _ternary(rng, n, k, c)
+        p[name + ".norm.weight"] = vec(k)
+
+    p["model.embeddings.weight"] = rng.normal(size=(V, H))
+    p["model.lower_bounds"] = rng.normal(size=(L, H)) * 1.5
+    for li in range(L):
+        b = f"model.layers.{li}."
+        p[b + "attn_norm.weight"] = vec(H)
+        for name in ("i_proj", "f_proj", "g_proj", "o_proj"):
+            lin(b + "attn." + name, H, H)
+        p[b + "attn.g_norm.weight"] = vec(H)
+        p[b + "mlp_norm.weight"] = vec(H)
+        lin(b + "mlp.gate_proj", 2 * I, H)
+        lin(b + "mlp.down_proj", H, I)
+    p["model.norm.weight"] = vec(H)
+    lin("lm_head", V, H)
+    ids = rng.integers(0, V, size=(2, 5))
+    return p, tern, ids
+
+
+def _torch_params(p):
+    return {k: torch.from_numpy(np.ascontiguousarray(v)).to(torch.float32) for k, v in p.items()}
+
+
+SEED = 40          # a seed whose model keeps every pre-rounding value >= 1e-3 away from a tie (checked below)
+_MARGIN_NEEDED = 1e-3
+
+
+def _case():
+    p, tern, ids = build(SEED)
+    margin = _Margin()
+    want, finals = reference_forward(p, ids, margin)
+    return p, tern, ids, want, finals, margin.value
+
+
+def _rel(a, b):
+    return float(np.max(np.abs(a - b)) / np.max(np.abs(b)))
+
+
+# ------------------------------------------------------------------ tests
+def test_weight_quant_of_c_times_ternary_is_that_ternary():
+    """weight_quant(c * T) = T * (c * share of non-zeros): the closed form that makes the model hand-computable."""
+    from oracle.quant import ternary_codes, weight_quant_literal
+    p, tern, _ = build(SEED)
+    for name, t in tern.items():
+        w = torch.from_numpy(p[name + ".weight"]).float()
+        codes, wdeq = ternary_codes(w)
+        assert np.array_equal(codes.numpy(), t), name
+        c = np.abs(p[name + ".weight"]).max()
+        assert abs(float(wdeq) - c * np.abs(t).mean()) < 1e-6 * c, name
+        assert np.allclose(weight_quant_literal(w).numpy(), t * c * np.abs(t).mean(), rtol=1e-5, atol=0)
+
+
+def test_the_case_has_a_rounding_margin():
+    *_, margin = _case()
+    assert margin >= _MARGIN_NEEDED, margin
+
+
+@pytest.mark.parametrize("mode", ["spec", "literal"])
+def test_oracle_forward_matches_the_independent_restatement(mode):
+    p, _, ids, want, finals, _ = _case()
+    got, states = om.forward(_torch_params(p), torch.from_numpy(ids), L, mode=mode, rms_norm_eps=RMS_EPS,
+                             bitlinear_eps=BL_EPS)
+    assert _rel(got.double().numpy(), want) < 2e-4
+    for li in range(L):
+        assert _rel(states[li].double().numpy(), finals[li]) < 2e-4
+    assert np.array_equal(got.argmax(-1).numpy(), want.argmax(-1))
+
+
+def test_oracle_decode_with_carried_state_matches_the_restatement():
+    """Prefill 3 tokens, then 2 single-token steps with the carried state == the 5-token known answer."""
+    p, _, ids, want, _, _ = _case()
+    tp, tids = _torch_params(p), torch.from_numpy(ids)
+    _, st = om.forward(tp, tids[:, :3], L)
+    for t in (3, 4):
+        lg, st = om.forward(tp, tids[:, t:t + 1], L, states=st)
+        assert _rel(lg[:, 0].double().numpy(), want[:, t]) < 2e-4
+
+
+def test_restatement_continues_from_a_state_like_the_full_sequence():
+    """The restatement's own state carry (so the decode check above compares like with like)."""
+    p, _, ids, want, _, _ = _case()
+    m = _Margin()
+    _, st = reference_forward(p, ids[:, :3], m)
+    tail, _ = reference_forward(p, ids[:, 3:], m, states=st)
+    assert _rel(tail, want[:, 3:]) < 1e-12
+
+
+# first-order wiring mistakes: (name, text in oracle.model.forward, replacement)
+MUTANTS = [
+    ("g_norm operands swapped", "ops.gated_norm(gg, o.reshape(B, T, H),", "ops.gated_norm(o.reshape(B, T, H), gg,"),
+    ("closing residual add dropped", 'b + "mlp.down_proj", residual_add=residual)', 'b + "mlp.down_proj")'),
+    ("mlp_norm sees the un-summed residual", "residual=residual, prenorm=True)",
+     "residual=torch.zeros_like(residual), prenorm=True)"),
+    ("attn_norm output used as the residual", "        ii = ops.bitlinear(hn,", "        residual = hn\n        ii = ops.bitlinear(hn,"),
+    ("swiglu(1 - f, i)", "x_in, gate = ops.gate(ii, ff,", "x_in, gate = ops.gate(ff, ii,"),
+    ("lower-bound schedule shifted by a layer", "lbs[i] if lbs is not None", "lbs[(i + 1) % num_layers] if lbs is not None"),
+    ("lower bounds not applied", "lbs[i] if lbs is not None else None", "None"),
+    ("f_proj and g_proj exchanged", 'ff = ops.bitlinear(hn, params, b + "attn.f_proj")',
+     'ff = ops.bitlinear(hn, params, b + "attn.g_proj")'),
+    ("o_proj reads the block norm output", "a = ops.bitlinear(o2,", "a = ops.bitlinear(hn,"),
+    ("gate and up halves exchanged", "g1, y1 = y.chunk(2, -1)", "y1, g1 = y.chunk(2, -1)"),
+    ("final norm skipped", 'hN = ops.rmsnorm(h, params["model.norm.weight"], rms_norm_eps)', "hN = h"),
+    ("scan gate and input exchanged", "ops.scan(x_in.reshape(B, 1, T, H), gate.reshape(B, 1, T, H), h0)",
+     "ops.scan(gate.reshape(B, 1, T, H), x_in.reshape(B, 1, T, H), h0)"),
+    ("MLP reads the attention output, not its norm", "y = ops.bitlinear(hn2,", "y = ops.bitlinear(a,"),
+]
+
+
+@pytest.mark.parametrize("name,old,new", MUTANTS, ids=[m[0] for m in MUTANTS])
+def test_mutants_of_the_oracle_are_caught(name, old, new):
+    """Each mutated copy of oracle.model.forward must disagree with the known answer by far more than the
+    tolerance of the positive test (2e-4)."""
+    src = inspect.getsource(om.forward)
+    assert src.count(old) == 1, f"oracle.model.forward no longer contains {old!r}: update MUTANTS"
+    scope = dict(vars(om))
+    exec(compile(src.replace(old, new), f"<mutant: {name}>", "exec"), scope)
+    p, _, ids, want, _, _ = _case()
+    for mode in ("spec", "literal"):
+        got, _ = scope["forward"](_torch_params(p), torch.from_numpy(ids), L, mode=mode, rms_norm_eps=RMS_EPS,
+                                  bitlinear_eps=BL_EPS)
+        assert _rel(got.double().numpy(), want) > 1e-2, (name, mode)
+
+
+def test_lower_bound_of_layer_0_is_exactly_zero():
+    """cumsum(softmax)[0] - softmax[0] = 0 for any parameter value, so applying the bound at layer 0 (dropping the
+    reference's ``layer_idx > 0`` test, layers/hgrn_bit.py:115) changes nothing: that mutant is equivalent and is
+    not in the list above."""
+    lb = om.lower_bound_rows(torch.randn(5, 9) * 3)
+    assert torch.equal(lb[0], torch.zeros(9))
+    assert (lb[1:] > 0).all() and (lb < 1).all()
