@@ -215,12 +215,23 @@ class DecodeEngine:
         """False once a wait inside the resident layer chain ran out of polling rounds (host synchronisation)."""
         return not self.resident or int(self.err.item()) == 0
 
+    def _reset_resident(self):
+        """Bring the hand-off words back to their initial state.  A launch whose wait timed out may have had a late
+        workgroup read the tag base after workgroup 0 advanced it (the base is only published safely when every poll
+        succeeded), and so have left words that carry tags of the NEXT launch; a later launch would accept them as its
+        own.  With every word, the tag base and the error word zero the next launch starts like the first one.  The
+        caller has synchronised with the device (it has read the error word)."""
+        self._words.zero_()
+        self.am_words.zero_()
+        self.epoch.zero_()
+        self.err.zero_()
+
     def check(self):
         """Raise if a wait inside the resident layer chain timed out since the engine was built: its workgroups were
         not all resident at once (other work held CUs), so the steps since then are invalid.  One host synchronisation;
-        callers run it once per generation, not per step."""
+        callers run it once per generation, not per step.  The engine is reset and can be used again."""
         if not self.resident_ok():
-            self.err.zero_()
+            self._reset_resident()
             raise L.MMFError("DecodeEngine: a wait inside the resident layer chain timed out (were other kernels running "
                              "on this device?); the tokens of this generation are invalid. Build the engine with "
                              "resident=False to decode with one launch per BitLinear.")
@@ -368,7 +379,7 @@ class DecodeEngine:
             warnings.warn("DecodeEngine: the resident layer chain timed out waiting for its workgroups; "
                           "falling back to one launch per BitLinear")
             self.resident = False
-            self.err.zero_()
+            self._reset_resident()
             for e, sv in zip(self.layers, saved):
                 e["state"].copy_(sv)
             self.tok.copy_(tok)

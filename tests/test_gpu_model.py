@@ -418,6 +418,44 @@ def test_resident_layer_chain_timeout_is_reported_and_recoverable(dev, tiny_bf16
     eng.check()
 
 
+def test_resident_engine_is_clean_after_a_timed_out_launch(dev, tiny_bf16):
+    """After a timed-out launch a late workgroup may have stored words tagged for the NEXT launch (it read the tag base
+    after workgroup 0 advanced it).  Such words are planted here from the host, with the tags the next launch expects
+    and a wrong value; check() must leave an engine whose next steps equal the launch chain's."""
+    import matmulfreellm_amd._lib as L_
+    from matmulfreellm_amd.decode import DecodeEngine
+    model = build(tiny_bf16, torch.bfloat16, dev)
+    torch.manual_seed(35)
+    ids = torch.randint(0, V, (1, 12), device=dev)
+    out = model(input_ids=ids, use_cache=True, logits_to_keep=1)
+    states = [c[-1] for c in out.past_key_values]
+    tok = out.logits[:, -1].argmax(-1)
+    eng = DecodeEngine(model, 1, use_graph=False, resident=True)
+    ref = DecodeEngine(model, 1, use_graph=False, resident=False)
+    eng.SPIN = 1
+    eng.load_state(states)
+    eng.step(tok)
+    torch.cuda.synchronize()
+    assert not eng.resident_ok()
+    e = int(eng.epoch.item())
+    h0, h1, ob, gb, ab, rb, zb = eng.words
+    wrong = 0x3F80 << 16                                         # bf16 1.0 in the value half
+    for buf, link in ((ob, 0), (gb, 0), (ab, 1), (rb, 2), (zb, 2), (h0, 3)):
+        buf.fill_(wrong | ((e + link + 1) & 0xFFFF))
+    with pytest.raises(L_.MMFError):
+        eng.check()
+    assert int(eng.epoch.item()) == 0 and int(eng._words.abs().max().item()) == 0
+    eng.SPIN = DecodeEngine.SPIN
+    eng.load_state(states)
+    ref.load_state(states)
+    for _ in range(3):
+        a = eng.step(tok).clone()
+        b = ref.step(tok).clone()
+        assert torch.equal(a, b)
+        tok = b.argmax(-1)
+    eng.check()
+
+
 def test_resident_launch_at_the_full_1p3b_shape(dev):
     """The benchmarked configuration itself (hidden 2048, 24 layers, vocabulary 32000, random weights on the device):
     16 self-feeding greedy steps through the one-launch decode step and through the launch chain give the same
