@@ -31,9 +31,13 @@ def bitlinear_fused_literal(x, weight, norm_weight, bias=None, eps=1e-6):
 def contract_exact(q, deq, t, wdeq, out_dtype, bias=None):
     """out[m,n] = dtype( fp32(acc[m,n]) * deq[m] * wdeq (+ bias[n]) ),
     acc = sum_k q[m,k] * t[n,k] in exact integers (|acc| <= 128*K < 2**24)."""
-    # fp64 BLAS matmul of small integers: every product and partial sum is an integer
-    # below 2**53, so the result is the exact integer accumulator (and fast).
-    acc = (q.to(torch.float64) @ t.to(torch.float64).t())
+    # BLAS matmul of small integers held as floats: every product and partial sum is an integer of magnitude
+    # <= 128 * K, exactly representable below 2**53 in fp64 (and below 2**24 in fp32), so whatever the summation
+    # order the result is the exact integer accumulator (and fast).  t may come in already converted (fp32 or
+    # fp64, the caller's choice under that bound); int8 codes are converted to fp64 here.
+    ft = t.dtype if t.is_floating_point() else torch.float64
+    assert 128 * q.shape[-1] < (2 ** 24 if ft == torch.float32 else 2 ** 53)
+    acc = (q.to(ft) @ t.to(ft).t())
     out = (acc.to(_F) * deq.reshape(-1, 1)) * wdeq
     if bias is not None:
         out = out + bias.to(_F)

@@ -79,7 +79,10 @@ class _Ops:
             key = prefix
             if key not in self._tern:
                 from .quant import ternary_codes
-                self._tern[key] = ternary_codes(w)
+                t, wdeq = ternary_codes(w)
+                # kept as floats for the BLAS contraction (exact: see contract_exact); fp32 holds every partial sum
+                # of a row of K codes exactly while 128 * K < 2**24
+                self._tern[key] = (t.to(_F if 128 * t.shape[1] < 2 ** 24 else torch.float64), wdeq)
             t, wdeq = self._tern[key]
             shp = x.shape
             q, deq, _, _ = on.rms_norm_quant_spec(x.reshape(-1, shp[-1]), nw, eps=self.bl_eps)

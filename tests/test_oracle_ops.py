@@ -93,6 +93,26 @@ def test_bitlinear_integer_identity():
     assert rel(out, dense) < 1e-6
 
 
+def test_contraction_on_fp32_codes_is_the_exact_accumulator():
+    """The model oracle keeps the ternary codes as fp32 for a BLAS contraction: at the widest row of the
+    benchmarked shapes (K = 6912, worst-case codes +-128 / +-1) every partial sum stays below 2**24, so the fp32
+    result is the int64 one."""
+    torch.manual_seed(8)
+    k = 6912
+    q = torch.randint(-128, 128, (5, k), dtype=torch.int8)
+    q[0] = -128
+    q[1] = 127
+    t = torch.randint(-1, 2, (33, k), dtype=torch.int8)
+    t[0] = 1
+    t[1] = -1
+    deq = torch.rand(5) + 0.5
+    wdeq = torch.tensor(0.0123)
+    out32, acc32 = ob.contract_exact(q, deq, t.float(), wdeq, torch.bfloat16)
+    out64, acc64 = ob.contract_exact(q, deq, t, wdeq, torch.bfloat16)
+    assert torch.equal(acc32.to(torch.int64), q.to(torch.int64) @ t.to(torch.int64).t())
+    assert torch.equal(acc32, acc64) and torch.equal(out32, out64)
+
+
 # ---------------------------------------------------------------- scans
 def test_scan_closed_forms():
     B, H, T, D = 2, 1, 50, 8
