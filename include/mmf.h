@@ -52,6 +52,17 @@ int64_t mmf_packed_bytes(int64_t N, int64_t K);
 int64_t mmf_ternarize_workspace_bytes(void);
 int mmf_ternarize_pack(const void* w, int w_dtype, int64_t N, int64_t K, void* packed, float* wdeq,
                        void* workspace, void* stream);
+/* mmf_ternarize_pack_noalloc: mmf_ternarize_pack without the workspace argument, for callers that cannot allocate
+ * device memory (code under HIP graph capture, tight serving loops that re-pack updated weights, harnesses that
+ * forbid hipMalloc).  It has no counterpart in the reference.  The 8 KiB of partial sums live in a file-scope device
+ * array of the library (one copy per GPU, held until the process ends; its address is looked up on the first call
+ * on each GPU, which should therefore happen outside a graph capture).  Same kernels, same results as
+ * mmf_ternarize_pack.  Nothing is allocated, freed or synchronised.  N * K above
+ * mmf_ternarize_pack_noalloc_max_elements() (2^31): MMF_ERR_WIDE.  Every call on a GPU uses that GPU's one array:
+ * calls that overlap on one GPU (different streams or threads) race; calls on one stream are ordered and safe.
+ * Nothing in the array needs clearing between calls: a call writes every partial sum it later reads. */
+int64_t mmf_ternarize_pack_noalloc_max_elements(void);
+int mmf_ternarize_pack_noalloc(const void* w, int w_dtype, int64_t N, int64_t K, void* packed, float* wdeq, void* stream);
 /* packed -> int8 codes [N, K] in {-1, 0, 1} (inspection / tests). */
 int mmf_unpack_ternary(const void* packed, int64_t N, int64_t K, int8_t* codes, void* stream);
 

@@ -24,6 +24,8 @@ SIGNATURES = {
     "mmf_packed_bytes": (_i64, [_i64, _i64]),
     "mmf_ternarize_workspace_bytes": (_i64, []),
     "mmf_ternarize_pack": (_i32, [_ptr, _i32, _i64, _i64, _ptr, _ptr, _ptr, _ptr]),
+    "mmf_ternarize_pack_noalloc_max_elements": (_i64, []),
+    "mmf_ternarize_pack_noalloc": (_i32, [_ptr, _i32, _i64, _i64, _ptr, _ptr, _ptr]),
     "mmf_unpack_ternary": (_i32, [_ptr, _i64, _i64, _ptr, _ptr]),
     "mmf_rmsnorm": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _f32, _i32, _i32, _i32, _ptr]),
     "mmf_rmsnorm_swishgate": (_i32, [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _f32, _i32, _i32, _i32, _ptr]),

@@ -111,6 +111,33 @@ int launch_pack(const void* w, int64_t N, int64_t K, void* packed, float* wdeq, 
     return 0;
 }
 
+// Scratch of mmf_ternarize_pack_noalloc: the partial sums live in the library's own device memory (one copy per GPU,
+// held until the process ends) instead of a caller-provided workspace.
+static __device__ __align__(256) double scratch[kPartials];
+
+constexpr int kMaxDevices = 64;
+double* scratch_ptr[kMaxDevices];          // device address of `scratch` on each GPU, looked up on first use
+
+// The address of this GPU's copy of `scratch` (the array's name is only a host-side handle: kernels must be given
+// the address hipGetSymbolAddress returns for the current device).
+int scratch_of_current_device(double** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return MMF_ERR_ARG;
+    double* p = __atomic_load_n(&scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (!p) {
+        void* sym = nullptr;
+        e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!sym) return MMF_ERR_ARG;
+        p = static_cast<double*>(sym);
+        __atomic_store_n(&scratch_ptr[dev], p, __ATOMIC_RELEASE);   // every thread would store the same address
+    }
+    *out = p;
+    return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -128,6 +155,23 @@ int mmf_ternarize_pack(const void* w, int w_dtype, int64_t N, int64_t K, void* p
         case MMF_F32: return launch_pack<float>(w, N, K, packed, wdeq, workspace, stream);
         case MMF_BF16: return launch_pack<bf16_t>(w, N, K, packed, wdeq, workspace, stream);
         case MMF_F16: return launch_pack<f16_t>(w, N, K, packed, wdeq, workspace, stream);
+    }
+    return MMF_ERR_ARG;
+}
+
+int64_t mmf_ternarize_pack_noalloc_max_elements(void) { return (int64_t)1 << 31; }
+
+int mmf_ternarize_pack_noalloc(const void* w, int w_dtype, int64_t N, int64_t K, void* packed, float* wdeq, void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (N <= 0 || K <= 0 || !w || !packed || !wdeq) return MMF_ERR_ARG;
+    if (N > mmf_ternarize_pack_noalloc_max_elements() / K) return MMF_ERR_WIDE;   // more than 2^31 weights
+    if (reinterpret_cast<uintptr_t>(packed) & 15u) return MMF_ERR_ALIGN;
+    double* ws = nullptr;
+    if (const int rc = scratch_of_current_device(&ws)) return rc;
+    switch (w_dtype) {
+        case MMF_F32: return launch_pack<float>(w, N, K, packed, wdeq, ws, stream);
+        case MMF_BF16: return launch_pack<bf16_t>(w, N, K, packed, wdeq, ws, stream);
+        case MMF_F16: return launch_pack<f16_t>(w, N, K, packed, wdeq, ws, stream);
     }
     return MMF_ERR_ARG;
 }
