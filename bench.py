@@ -1,21 +1,29 @@
 #!/usr/bin/env python3
 """Headline benchmark: greedy decode tok/s of the 1.3B-shape HGRNBit model on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--only LEG[,LEG...]]
 
 One step = one decode step of the whole model (24 layers, ternary 2-bit packed weights,
 bf16 activations, fp32 recurrent state) for the whole batch, replayed as one HIP graph with
 inputs resident in HBM.  Prints ONE JSON line:
   value        decode tokens/s at --batch (default 1)
-  roofline     the dominant kernel at batch 1, the fused BitLinear GEMV: algorithmic bytes of
-               the 97 GEMV launches of one step / their average launch time, timed live with
-               HIP events on the launch stream (a graph holding only those launches, with the
-               model's own 325 MB of packed weights so HBM, not a cache, is measured)
+  roofline     the dominant kernel at batch 1: the resident launch that is the whole decode step
+               (decode_layers_kernel: embedding row, the 4L fused BitLinears, lm_head, argmax) --
+               its algorithmic bytes (every 2-bit weight once + each link's activations, norm
+               weights and state) / its launch time, timed live with HIP events on the launch
+               stream; with --launch-chain the fused BitLinear GEMV launches of one step instead.
+               The model's own 325 MB of packed weights exceed the 256 MB last-level cache, so
+               HBM, not a cache, is measured.
   cpu_baseline the reference's PyTorch formulation (oracle, literal mode, weights
-               re-quantised per call as the reference does) timed on this host's cores on a
-               bounded sample (2 of the 24 layers + head, scaled to 24)
-  extra        batch-64 decode, prompt prefill (8 x 512 tokens), prefill-sized BitLinear on the int8
-               matrix cores (TOP/s and fraction of 5.0 POP/s), HGRN scan and norm bandwidths.
+               re-quantised per call as the reference does) timed on this host's cores on bounded
+               samples: 1.3B-shape decode (2 of 24 layers + head, scaled), the tiny config end to
+               end, single BitLinears and the scan
+  extra        batch-64 decode, prompt prefill (8 x 512 and 8 x 2048 tokens, with the whole forward's
+               int8 TOP/s against 5.0 POP/s), prefill-sized BitLinear on the int8 matrix cores,
+               HGRN scan, norm and loss bandwidths (cache-cold: the legs rotate through buffer sets
+               of more than 512 MB in total; counted HBM traffic from rocprofv3 beside each).
+--only runs the named legs only (decode, bs64, prefill, mfma, scan, norms, sampling, loss, cpu): the
+profiles under profiles/ are made that way.
 Synthetic data: random-init N(0, 0.02) weights, uniform random token ids.
 """
 import argparse
@@ -163,18 +171,50 @@ def mfma_bench(dev, m=4096, k=2048, n=11264, iters=20):
             "int8_TOPs": round(tops, 1), "frac_of_5POPs": round(tops / INT8_PEAK_TOPS, 4)}
 
 
-def scan_bench(dev, b=8, t=2048, d=2048, iters=10):
+def _rotating(make_set, set_bytes, min_total=512 << 20, min_sets=3):
+    """Independent buffer sets whose total exceeds the 256 MB last-level cache twice over, and a counter to walk them:
+    by the time a set comes round again the others have pushed it out, so every launch reads from HBM."""
+    n = max(min_sets, -(-min_total // set_bytes) + 1)
+    sets = [make_set() for _ in range(n)]
+    state = {"i": 0}
+
+    def nxt():
+        state["i"] = (state["i"] + 1) % n
+        return sets[state["i"]]
+    return nxt, n
+
+
+# HBM bytes per launch of the bandwidth-bound kernels at the shapes below, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/hbm_traffic_scan_norm_loss.txt; same calibration copy as the decode kernels).
+COUNTED_TRAFFIC = {"hgrn_recurrent": 201466341, "hgrn_chunk": 201478277, "rmsnorm": 134308657, "rmsnorm_swishgate": 201466176,
+                   "cross_entropy": 263075006}
+
+
+def scan_bench(dev, b=8, t=2048, d=2048, iters=12):
     import matmulfreellm_amd.functional as F_
     g = torch.Generator(device=dev).manual_seed(3)
-    z = torch.randn(b, 1, t, d, generator=g, device=dev) + 2
-    x = torch.randn(b, 1, t, d, generator=g, device=dev).bfloat16()
-    glog = torch.nn.functional.logsigmoid(z).bfloat16()
-    glin = torch.sigmoid(z).bfloat16()
+
+    def make():
+        z = torch.randn(b, 1, t, d, generator=g, device=dev) + 2
+        x = torch.randn(b, 1, t, d, generator=g, device=dev).bfloat16()
+        return x, torch.nn.functional.logsigmoid(z).bfloat16(), torch.sigmoid(z).bfloat16()
     nbytes = 3 * b * t * d * 2
-    ms_r = timed(lambda: F_.hgrn_recurrent(x, glin), iters)
-    ms_c = timed(lambda: F_.hgrn_chunk(x, glog, chunk_size=64), iters)
-    return {"shape": [b, t, d], "recurrent_ms": round(ms_r, 4), "recurrent_GBs": round(nbytes / ms_r / 1e6, 1),
-            "chunk64_ms": round(ms_c, 4), "chunk64_GBs": round(nbytes / ms_c / 1e6, 1)}
+    nxt, nsets = _rotating(make, 4 * b * t * d * 2)
+
+    def rec():
+        x, _, glin = nxt()
+        F_.hgrn_recurrent(x, glin)
+
+    def chk():
+        x, glog, _ = nxt()
+        F_.hgrn_chunk(x, glog, chunk_size=64)
+    ms_r = timed(rec, iters, warmup=nsets)
+    ms_c = timed(chk, iters, warmup=nsets)
+    return {"shape": [b, t, d], "buffer_sets": nsets, "recurrent_ms": round(ms_r, 4), "recurrent_GBs": round(nbytes / ms_r / 1e6, 1),
+            "recurrent_frac_of_hbm": round(nbytes / ms_r / 1e6 / HBM_PEAK_GBS, 4),
+            "chunk64_ms": round(ms_c, 4), "chunk64_GBs": round(nbytes / ms_c / 1e6, 1),
+            "algorithmic_bytes": nbytes, "counted_traffic_bytes": {"recurrent": COUNTED_TRAFFIC["hgrn_recurrent"],
+                                                                   "chunk64": COUNTED_TRAFFIC["hgrn_chunk"]}}
 
 
 def prefill_bench(model, dev, batch=8, seq=512, iters=5):
@@ -183,31 +223,55 @@ def prefill_bench(model, dev, batch=8, seq=512, iters=5):
     ids = torch.randint(0, model.config.vocab_size, (batch, seq), generator=g, device=dev)
     with torch.no_grad():
         ms = timed(lambda: model(input_ids=ids, use_cache=True, logits_to_keep=1), iters)
-    return {"batch": batch, "seq_len": seq, "ms": round(ms, 3), "tok_s": round(batch * seq / ms * 1e3)}
+    # int8 operations of the whole forward: every row through every layer's ternary weights, the last position of
+    # every sequence through the head
+    layer_w = sum(p.numel() for n, p in model.named_parameters() if n.endswith("proj.weight"))
+    head_w = model.lm_head.weight.numel()
+    ops = 2.0 * (batch * seq * layer_w + batch * head_w)
+    tops = ops / (ms * 1e-3) / 1e12
+    return {"batch": batch, "seq_len": seq, "ms": round(ms, 3), "tok_s": round(batch * seq / ms * 1e3),
+            "int8_TOPs_whole_forward": round(tops, 1), "frac_of_5POPs": round(tops / INT8_PEAK_TOPS, 4)}
 
 
-def norm_bench(dev, m=16384, k=2048, iters=20):
+def norm_bench(dev, m=16384, k=2048, iters=24):
     import matmulfreellm_amd.functional as F_
     g = torch.Generator(device=dev).manual_seed(4)
-    x = torch.randn(m, k, generator=g, device=dev).bfloat16()
-    o = torch.randn(m, k, generator=g, device=dev).bfloat16()
     w = torch.ones(k, device=dev, dtype=torch.bfloat16)
-    ms_n = timed(lambda: F_.rmsnorm(x, w), iters)
-    ms_g = timed(lambda: F_.rmsnorm_swishgate(x, o, w), iters)
-    return {"shape": [m, k], "rmsnorm_GBs": round(2 * m * k * 2 / ms_n / 1e6, 1),
-            "rmsnorm_swishgate_GBs": round(3 * m * k * 2 / ms_g / 1e6, 1)}
+
+    def make():
+        return (torch.randn(m, k, generator=g, device=dev).bfloat16(), torch.randn(m, k, generator=g, device=dev).bfloat16())
+    nxt, nsets = _rotating(make, 3 * m * k * 2)
+
+    def plain():
+        x, _ = nxt()
+        F_.rmsnorm(x, w)
+
+    def gated():
+        x, o = nxt()
+        F_.rmsnorm_swishgate(x, o, w)
+    ms_n = timed(plain, iters, warmup=nsets)
+    ms_g = timed(gated, iters, warmup=nsets)
+    return {"shape": [m, k], "buffer_sets": nsets, "rmsnorm_GBs": round(2 * m * k * 2 / ms_n / 1e6, 1),
+            "rmsnorm_swishgate_GBs": round(3 * m * k * 2 / ms_g / 1e6, 1),
+            "algorithmic_bytes": {"rmsnorm": 2 * m * k * 2, "rmsnorm_swishgate": 3 * m * k * 2},
+            "counted_traffic_bytes": {"rmsnorm": COUNTED_TRAFFIC["rmsnorm"], "rmsnorm_swishgate": COUNTED_TRAFFIC["rmsnorm_swishgate"]}}
 
 
-def loss_bench(dev, m=4096, v=32000, iters=20):
+def loss_bench(dev, m=4096, v=32000, iters=12):
     """Evaluation loss of m rows of v-wide bf16 logits (one read of the logits)."""
     import matmulfreellm_amd.functional as F_
     g = torch.Generator(device=dev).manual_seed(6)
-    logits = torch.randn(m, v, generator=g, device=dev).bfloat16()
     targets = torch.randint(0, v, (m,), generator=g, device=dev)
     lib, rows = F_.L.load(), torch.empty(m, dtype=torch.float32, device=dev)
-    ms = timed(lambda: F_.L.check(lib.mmf_cross_entropy_fwd(logits.data_ptr(), v, targets.data_ptr(), -100, rows.data_ptr(), m, v,
-                                                            F_.L.dtype_id(logits.dtype), F_.L.stream()), "mmf_cross_entropy_fwd"), iters)
-    return {"shape": [m, v], "ms": round(ms, 4), "GBs": round(m * v * 2 / ms / 1e6, 1)}
+    nxt, nsets = _rotating(lambda: torch.randn(m, v, generator=g, device=dev).bfloat16(), m * v * 2)
+
+    def run():
+        logits = nxt()
+        F_.L.check(lib.mmf_cross_entropy_fwd(logits.data_ptr(), v, targets.data_ptr(), -100, rows.data_ptr(), m, v,
+                                             F_.L.dtype_id(logits.dtype), F_.L.stream()), "mmf_cross_entropy_fwd")
+    ms = timed(run, iters, warmup=nsets)
+    return {"shape": [m, v], "buffer_sets": nsets, "ms": round(ms, 4), "GBs": round(m * v * 2 / ms / 1e6, 1),
+            "algorithmic_bytes": m * v * 2, "counted_traffic_bytes": COUNTED_TRAFFIC["cross_entropy"]}
 
 
 def sampler_bench(model, dev, n_new=256):
@@ -231,10 +295,34 @@ def sampler_bench(model, dev, n_new=256):
     return res
 
 
+def _cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _median_s(fn, reps, warm=1):
+    for _ in range(warm):
+        fn()
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    return sorted(ts)[len(ts) // 2]
+
+
 def cpu_baseline(shape="1.3B", budget_s=25.0):
-    """Reference PyTorch formulation (oracle literal mode) on the host cores: batch-1 decode of a
-    1.3B-shape model, timed on 2 of its 24 layers plus the head and scaled to 24 layers."""
+    """The reference's PyTorch formulation (oracle, literal mode; weights re-quantised on every call, as the reference
+    does) on the host cores.  Headline leg: batch-1 decode of a 1.3B-shape model, timed on 2 of its 24 layers plus the
+    head and scaled to 24 layers.  Further legs: the tiny configuration end to end (batch 1, 128 tokens: one forward
+    and greedy steps), single BitLinears at the benchmark's shapes, and the recurrence."""
     from oracle import bitlinear as ob
+    from oracle import hgrn as oh
     from oracle import model as om
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
@@ -252,25 +340,42 @@ def cpu_baseline(shape="1.3B", budget_s=25.0):
     def run_head():
         ob.bitlinear_literal(x, params["lm_head.weight"], params["lm_head.norm.weight"])
 
-    def med(fn, reps):
-        ts = []
-        for _ in range(reps):
-            t0 = time.perf_counter()
-            fn()
-            ts.append(time.perf_counter() - t0)
-        return sorted(ts)[len(ts) // 2]
-
     run_model(); run_head()
-    t_one = med(run_model, 1)
-    reps = max(3, min(15, int(budget_s / 2 / max(t_one, 1e-3))))
-    t_model = med(run_model, reps)
-    t_head = med(run_head, reps)
+    t_one = _median_s(run_model, 1, warm=0)
+    reps = max(3, min(15, int(budget_s / 3 / max(t_one, 1e-3))))
+    t_model = _median_s(run_model, reps, warm=0)
+    t_head = _median_s(run_head, reps, warm=0)
     t_layer = max(t_model - t_head, 1e-9) / Ls
     t_tok = t_layer * Lfull + t_head
+    del params
+
+    legs = {}
+    # tiny configuration, fp32, batch 1, 128-token prompt: forward over the prompt, then greedy steps with carried state
+    tc = SHAPES["tiny"]
+    tp = om.init_params(tc["vocab_size"], tc["hidden_size"], tc["num_hidden_layers"], seed=0, dtype=torch.float32)
+    tids = torch.randint(0, tc["vocab_size"], (1, 128))
+    nl = tc["num_hidden_layers"]
+    t_fwd = _median_s(lambda: om.forward(tp, tids, nl, mode="literal"), 3)
+    _, st = om.forward(tp, tids, nl, mode="literal", last_only=True)
+    t_step = _median_s(lambda: om.forward(tp, tids[:, :1], nl, states=st, mode="literal"), 5)
+    legs["tiny_config_fp32"] = {"prompt_128_forward_ms": round(t_fwd * 1e3, 1), "prompt_tok_s": round(128 / t_fwd, 1),
+                                "greedy_decode_tok_s": round(1.0 / t_step, 2)}
+    del tp
+    # single BitLinear, bf16-valued inputs computed in fp32 (the reference's CPU-runnable path), weights re-quantised per call
+    for name, (m, k, n) in (("bitlinear_4096x2048x11264", (4096, 2048, 11264)), ("bitlinear_4096x5632x2048", (4096, 5632, 2048)),
+                            ("bitlinear_64x2048x11264", (64, 2048, 11264)), ("bitlinear_1x2048x11264", (1, 2048, 11264))):
+        xx, ww, nw = torch.randn(m, k), torch.randn(n, k) * 0.02, torch.ones(k)
+        legs[name + "_ms"] = round(_median_s(lambda: ob.bitlinear_literal(xx, ww, nw), 3) * 1e3, 2)
+    # recurrence, naive loop as the reference's CPU oracle runs it: B = 8, D = 2048, T reduced from 2048 to 512
+    b, t, d = 8, 512, 2048
+    gg = torch.sigmoid(torch.randn(b, 1, t, d) + 2)
+    xs = torch.randn(b, 1, t, d)
+    legs["hgrn_naive_scan_8x512x2048_ms"] = round(_median_s(lambda: oh.naive_recurrent_hgrn_literal(xs, gg), 3) * 1e3, 2)
+    legs["hgrn_scan_note"] = "T reduced from 2048 to 512 (time is linear in T)"
     return {"value": round(1.0 / t_tok, 3), "unit": "tok/s", "cores": cores, "kind": "port",
             "sample": f"batch-1 decode step of a {shape}-shape model in fp32, {Ls} of {Lfull} layers + lm_head timed "
                       f"(median of {reps}), scaled to {Lfull} layers; weights re-quantised on every call as the reference does",
-            "ms_per_token": round(t_tok * 1e3, 2), "torch": torch.__version__}
+            "ms_per_token": round(t_tok * 1e3, 2), "cpu_model": _cpu_model(), "torch": torch.__version__, "legs": legs}
 
 
 def main():
@@ -283,6 +388,8 @@ def main():
     ap.add_argument("--launch-chain", action="store_true",
                     help="batch 1: one launch per fused BitLinear instead of the resident layer chain")
     ap.add_argument("--no-extra", action="store_true", help="skip the batch-64 / matrix-core / scan / norm / CPU legs")
+    ap.add_argument("--only", default="", help="comma-separated legs to run instead of everything: decode, bs64, prefill, mfma, "
+                                               "scan, norms, sampling, loss, cpu (profiling runs)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by)")
     args = ap.parse_args()
@@ -294,9 +401,7 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    model = build_model(args.shape, torch.bfloat16, dev)
-    n_tern = sum(p.numel() for n, p in model.named_parameters() if n.endswith("proj.weight") or n == "lm_head.weight")
-
+    only = {t for t in args.only.split(",") if t}
     if args.calib_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
@@ -304,6 +409,25 @@ def main():
         dst.copy_(src)          # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
+    if only and not (only & {"decode", "bs64", "prefill", "sampling"}):
+        # legs that need no model: run them alone and print what they measured
+        res = {}
+        if "mfma" in only:
+            res["bitlinear_mfma_gate_proj"] = mfma_bench(dev, 4096, 2048, 11264)
+            res["bitlinear_mfma_down_proj"] = mfma_bench(dev, 4096, 5632, 2048)
+        if "scan" in only:
+            res["hgrn_scan"] = scan_bench(dev)
+        if "norms" in only:
+            res["norms"] = norm_bench(dev)
+        if "loss" in only:
+            res["cross_entropy"] = loss_bench(dev)
+        if "cpu" in only:
+            res["cpu_baseline"] = cpu_baseline(args.shape)
+        print(json.dumps({"only": sorted(only), "extra": res}))
+        return
+    model = build_model(args.shape, torch.bfloat16, dev)
+    n_tern = sum(p.numel() for n, p in model.named_parameters() if n.endswith("proj.weight") or n == "lm_head.weight")
+
     ms, eng = decode_bench(model, args.batch, args.steps, args.warmup, dev, resident=False if args.launch_chain else None)
     tok_s = args.batch * 1e3 / ms
     result = {
@@ -328,25 +452,34 @@ def main():
         eng1 = DecodeEngine.for_model(model, 1, use_graph=True, resident=False if args.launch_chain else None)
     result["roofline"] = gemv_roofline(eng1)
 
-    if not args.no_extra:
-        extra = {}
-        other = 64 if args.batch == 1 else 1
+    def want(leg):
+        return (leg in only) if only else not args.no_extra
+
+    extra = {}
+    other = 64 if args.batch == 1 else 1
+    if want("bs64"):
         ms_o, _ = decode_bench(model, other, args.steps, args.warmup, dev)
         extra[f"decode_bs{other}_tok_s"] = round(other * 1e3 / ms_o, 1)
         extra[f"decode_bs{other}_ms_per_step"] = round(ms_o, 4)
+    if want("prefill"):
         extra["prefill_8x512"] = prefill_bench(model, dev, 8, 512)
+        extra["prefill_8x2048"] = prefill_bench(model, dev, 8, 2048, iters=3)
+    if want("mfma"):
         extra["bitlinear_mfma_gate_proj"] = mfma_bench(dev, 4096, 2048, 11264)
         extra["bitlinear_mfma_down_proj"] = mfma_bench(dev, 4096, 5632, 2048)
+    if want("scan"):
         extra["hgrn_scan"] = scan_bench(dev)
+    if want("norms"):
         extra["norms"] = norm_bench(dev)
+    if want("sampling"):
         extra["sampling"] = sampler_bench(model, dev)
+    if want("loss"):
         extra["cross_entropy"] = loss_bench(dev)
+    if extra:
         result["extra"] = extra
-        del model, eng, eng1
-        torch.cuda.empty_cache()
-        result["cpu_baseline"] = cpu_baseline(args.shape)
-    else:
-        result["cpu_baseline"] = None
+    del model, eng, eng1
+    torch.cuda.empty_cache()
+    result["cpu_baseline"] = cpu_baseline(args.shape) if want("cpu") else None
     print(json.dumps(result))
 
 
