@@ -210,7 +210,14 @@ def scan_bench(dev, b=8, t=2048, d=2048, iters=12):
         F_.hgrn_chunk(x, glog, chunk_size=64)
     ms_r = timed(rec, iters, warmup=nsets)
     ms_c = timed(chk, iters, warmup=nsets)
+    # one long sequence: the same bytes as [1, 8 * t, d]; batch * channels alone give 32 workgroups, so the chunked entry
+    # point also splits the time axis over workgroups (the sequential recurrence cannot)
+    ms_r1 = timed(lambda: F_.hgrn_recurrent(*[v.view(1, 1, b * t, d) for v in (lambda s: (s[0], s[2]))(nxt())]), iters, warmup=nsets)
+    ms_c1 = timed(lambda: F_.hgrn_chunk(*[v.view(1, 1, b * t, d) for v in nxt()[:2]], chunk_size=64), iters, warmup=nsets)
+    long_seq = {"shape": [1, b * t, d], "recurrent_ms": round(ms_r1, 4), "recurrent_GBs": round(nbytes / ms_r1 / 1e6, 1),
+                "chunk64_ms": round(ms_c1, 4), "chunk64_GBs": round(nbytes / ms_c1 / 1e6, 1)}
     return {"shape": [b, t, d], "buffer_sets": nsets, "recurrent_ms": round(ms_r, 4), "recurrent_GBs": round(nbytes / ms_r / 1e6, 1),
+            "one_long_sequence": long_seq,
             "recurrent_frac_of_hbm": round(nbytes / ms_r / 1e6 / HBM_PEAK_GBS, 4),
             "chunk64_ms": round(ms_c, 4), "chunk64_GBs": round(nbytes / ms_c / 1e6, 1),
             "algorithmic_bytes": nbytes, "counted_traffic_bytes": {"recurrent": COUNTED_TRAFFIC["hgrn_recurrent"],

@@ -173,16 +173,20 @@ int mmf_bitlinear_mfma_swiglu(const int8_t* codes_tiled, const float* deq, const
  * mmf_hgrn_recurrent replaces fused_recurrent_hgrn, mmfreelm/ops/hgrn/recurrent_fuse.py:
  *   176-185 (kernel :32-68): h = g*h + x with g the decay itself.
  * mmf_hgrn_chunk replaces chunk_hgrn, mmfreelm/ops/hgrn/chunk.py:287-296 (kernels :49-116):
- *   h = exp(g)*h + x with g the log decay.  The reference's two-pass chunked evaluation is a
- *   reassociation of this recurrence; here it is run step by step, so the result agrees with
- *   the reference's to rounding and does not depend on `chunk` (kept for the reference's
- *   signature; 1 <= chunk <= 64 is still checked).
+ *   h = exp(g)*h + x with g the log decay, evaluated as the reference's chunked form: per chunk of `chunk` steps
+ *   (1 <= chunk <= 64; the reference fixes 128) a scan from zero (the first chunk from h0) with the running sum gc of
+ *   the log gates, then o_t += exp(gc_t) * (last output of the chunk before).  One pass over x and g with the chunk in
+ *   registers (no fp32 [B,H,T,D] scratch tensors).  When BH * ceil(D / 64) < 256 the time axis is also cut into
+ *   segments that run in parallel (a first launch leaves each segment's (decay product, end state from zero) pair in
+ *   `workspace`, mmf_hgrn_chunk_workspace_bytes(BH, T, D, chunk) bytes, 4-byte aligned, may be NULL when that is 0).
+ *   exp is the hardware one: results agree with the reference's within rounding, not bit for bit.
  * The final state is fp32 in both (the reference rounds the recurrent one to x's dtype).
  * MMF_ERR_WIDE when 64 rows of D elements reach 2 GiB. */
 int mmf_hgrn_recurrent(const void* x, const void* g, const float* h0, void* o, float* ht, int64_t BH,
                        int64_t T, int64_t D, int dtype, void* stream);
+int64_t mmf_hgrn_chunk_workspace_bytes(int64_t BH, int64_t T, int64_t D, int chunk);
 int mmf_hgrn_chunk(const void* x, const void* g, const float* h0, void* o, float* ht, int64_t BH,
-                   int64_t T, int64_t D, int chunk, int dtype, void* stream);
+                   int64_t T, int64_t D, int chunk, int dtype, void* workspace, void* stream);
 
 /* Gate math of HGRNBitAttention.forward, mmfreelm/layers/hgrn_bit.py:113-120, fused:
  *   g_out = T(lb + (1 - lb) * sigmoid(f))  (lower_bound NULL: T(sigmoid(f)))

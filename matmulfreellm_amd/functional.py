@@ -400,9 +400,13 @@ def hgrn_chunk(x, g, initial_state=None, output_final_state=False, chunk_size=64
     o = torch.empty_like(xc)
     h0 = _state32(initial_state, b * h, d, dev)
     ht = torch.empty(b, h, d, dtype=torch.float32, device=dev) if output_final_state else None
+    if not 1 <= chunk_size <= 64:
+        raise ValueError("chunk_size must lie in [1, 64]")
+    nws = lib.mmf_hgrn_chunk_workspace_bytes(b * h, t, d, chunk_size)
+    ws = torch.empty(nws // 4, dtype=torch.float32, device=dev) if nws else None    # per-segment carries (few KB)
     with torch.cuda.device(dev):
         L.check(lib.mmf_hgrn_chunk(xc.data_ptr(), gc.data_ptr(), L.ptr(h0), o.data_ptr(), L.ptr(ht), b * h, t, d,
-                                   chunk_size, L.dtype_id(x.dtype), L.stream()), "mmf_hgrn_chunk")
+                                   chunk_size, L.dtype_id(x.dtype), L.ptr(ws), L.stream()), "mmf_hgrn_chunk")
     return o, ht
 
 

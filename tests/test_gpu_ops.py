@@ -264,8 +264,9 @@ def test_hgrn_recurrent(dev, dtype, bhtd, with_h0):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("bhtd", [(2, 1, 64, 128), (1, 2, 200, 100), (2, 1, 1, 64), (1, 1, 1030, 256)])
-@pytest.mark.parametrize("chunk", [64, 16, 7])
+@pytest.mark.parametrize("bhtd", [(2, 1, 64, 128), (1, 2, 200, 100), (2, 1, 1, 64), (1, 1, 1030, 256), (1, 1, 4100, 192),
+                                  (2, 2, 777, 64), (1, 1, 16384, 128)])
+@pytest.mark.parametrize("chunk", [64, 16, 7, 48, 1])
 def test_hgrn_chunk(dev, dtype, bhtd, chunk):
     torch.manual_seed(11)
     b, h, t, d = bhtd
@@ -273,10 +274,21 @@ def test_hgrn_chunk(dev, dtype, bhtd, chunk):
     g = torch.nn.functional.logsigmoid(z).to(dtype)
     x = torch.randn(b, h, t, d).to(dtype)
     h0 = torch.randn(b, h, d)
+    if t > 5000 and chunk < 16:
+        pytest.skip("the oracle's chunk loop is slow for many tiny chunks")
     o_ref, ht_ref = oh.chunk_hgrn_spec(x, g, h0, True, chunk=chunk)
     o, ht = F().hgrn_chunk(x.to(dev), g.to(dev), h0.to(dev), True, chunk_size=chunk)
     assert_same(o, o_ref, tol_of(dtype), f"chunk {dtype} {bhtd} c{chunk}")
     assert rel_err(ht, ht_ref) <= 1e-3
+    # the time axis is cut into parallel segments exactly when batch * channel blocks leave CUs idle
+    lib = F().L.load()
+    nws = lib.mmf_hgrn_chunk_workspace_bytes(b * h, t, d, chunk)
+    assert (nws > 0) == (b * h * -(-d // 64) < 256 and t // (4 * min(64 // chunk, 8) * chunk) >= 2)
+    # without an initial state, and without asking for the final one
+    o2, none = F().hgrn_chunk(x.to(dev), g.to(dev), None, False, chunk_size=chunk)
+    o2_ref, _ = oh.chunk_hgrn_spec(x, g, None, False, chunk=chunk)
+    assert none is None
+    assert_same(o2, o2_ref, tol_of(dtype), f"chunk without state {dtype} {bhtd} c{chunk}")
     # the chunked and the sequential form agree (g_lin = exp(g_log))
     o_seq, _ = oh.recurrent_hgrn_spec(x, g.float().exp().to(dtype) if dtype == torch.float32 else g.float().exp(), h0, True) \
         if dtype == torch.float32 else (None, None)

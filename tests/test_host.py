@@ -42,7 +42,7 @@ def test_argument_errors_are_codes_not_crashes():
     lib = _lib.load()
     assert lib.mmf_rmsnorm(None, None, None, None, None, 4, 64, 1e-6, 1, 1, 1, None) == -1       # null x
     assert lib.mmf_rmsnorm(None, None, None, None, None, 0, 64, 1e-6, 1, 1, 1, None) == 0        # empty is fine
-    assert lib.mmf_hgrn_chunk(None, None, None, None, None, 0, 0, 64, 100, 1, None) == -1        # chunk > 64
+    assert lib.mmf_hgrn_chunk(None, None, None, None, None, 0, 0, 64, 100, 1, None, None) == -1        # chunk > 64
     assert lib.mmf_bitlinear_mfma(None, None, None, None, None, 32, None, None, None, 8, 4, 64, 16, 1, -1, None) == -1
 
 
