@@ -22,7 +22,7 @@ inputs resident in HBM.  Prints ONE JSON line:
                int8 TOP/s against 5.0 POP/s), prefill-sized BitLinear on the int8 matrix cores,
                HGRN scan, norm and loss bandwidths (cache-cold: the legs rotate through buffer sets
                of more than 512 MB in total; counted HBM traffic from rocprofv3 beside each).
---only runs the named legs only (decode, bs64, prefill, mfma, scan, norms, sampling, loss, cpu): the
+--only runs the named legs only (decode, bs64, prefill, mfma, scan, norms, sampling, loss, cpu, link_trace): the
 profiles under profiles/ are made that way.
 Synthetic data: random-init N(0, 0.02) weights, uniform random token ids.
 """
@@ -153,6 +153,33 @@ def gemv_roofline(eng, iters=20):
             "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH if counted else None,
             "launches_per_step": n, "algorithmic_bytes_per_launch": total_bytes // n,
             "avg_launch_us": round(us_per_launch, 3)}
+
+
+def link_trace_bench(model, dev):
+    """Where a link of the resident batch-1 launch spends its cycles: the kernel's own cycle stamps (thread 0 of three
+    workgroups, ten points per link), averaged per kind of link over the layers of one decode step."""
+    import numpy as np
+    from matmulfreellm_amd.decode import DecodeEngine
+    eng = DecodeEngine.for_model(model, 1, use_graph=True)
+    if not eng.resident:
+        return None
+    for _ in range(4):
+        eng._launch_layers(True)
+    t = eng.link_trace().numpy().astype(np.float64)
+    assert eng.resident_ok()
+    names = ["i/f/g", "o_proj", "gate/up", "down"]
+    stages = ["row arrives", "block norm", "sum of squares", "rstd", "absmax", "codes -> LDS", "dot", "partials meet", "epilogue"]
+    out = {"unit": "shader clock cycles (s_memtime), mean over layers 2.. of one step", "stages": stages, "workgroups": {}}
+    nl = 4 * eng.L
+    for slot, wg in enumerate((0, 37, 200)):
+        per = {}
+        for kind in range(4):
+            rows = t[slot, kind:nl:4, :10][2:]
+            per[names[kind]] = {"stages": [round(float(v)) for v in np.diff(rows, axis=1).mean(axis=0)],
+                                "link_total": round(float((rows[:, 9] - rows[:, 0]).mean()))}
+        per["whole_chain_cycles"] = int(t[slot, nl - 1, 9] - t[slot, 0, 0])
+        out["workgroups"][str(wg)] = per
+    return out
 
 
 def mfma_bench(dev, m=4096, k=2048, n=11264, iters=20):
@@ -416,7 +443,7 @@ def main():
         dst.copy_(src)          # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
-    if only and not (only & {"decode", "bs64", "prefill", "sampling"}):
+    if only and not (only & {"decode", "bs64", "prefill", "sampling", "link_trace"}):
         # legs that need no model: run them alone and print what they measured
         res = {}
         if "mfma" in only:
@@ -478,6 +505,8 @@ def main():
         extra["hgrn_scan"] = scan_bench(dev)
     if want("norms"):
         extra["norms"] = norm_bench(dev)
+    if "link_trace" in only:
+        extra["link_trace"] = link_trace_bench(model, dev)
     if want("sampling"):
         extra["sampling"] = sampler_bench(model, dev)
     if want("loss"):

@@ -256,13 +256,18 @@ int mmf_sample_top_p(const void* logits, int64_t ld, int64_t rows, int64_t V, fl
  *     K = H, N = vocabulary size); the launch then also writes the logits [N] (activation dtype), and the greedy token
  *     (lowest index of the largest logit; NaNs never win) to *tok_out, which may be the buffer `tok` points to.
  *     am_words: 256 uint64 scratch words, zero-initialised once.  With head == null the three pointers are ignored.
+ *   trace: null, or mmf_decode_layers_trace_words() int64 words (zeroed by the caller): thread 0 of workgroups 0, 37 and
+ *     200 stores the shader clock at ten points of each of the first 128 links, [workgroup][link][12]: 0 link entered,
+ *     1 input row arrived, 2 block norm applied, 3 sum of squares reduced, 4 rstd, 5 absmax reduced, 6 codes in LDS,
+ *     7 dot products done, 8 partial sums met, 9 epilogue stored (a measuring aid; costs a few scalar branches).
  *   Requires D == H, H, I multiples of 128, H <= 4096, I <= 8192 (else MMF_ERR_WIDE), 16-bit activations (dtype 1 or 2), batch 1.
  *   Calls on one device must not overlap (they share the scratch words). */
 int mmf_decode_layers_phase_bytes(void);
+int mmf_decode_layers_trace_words(void);
 int mmf_decode_layers(const void* phases, int n_layers, const void* table, const int64_t* tok, int64_t vocab,
                       uint32_t* h0, uint32_t* h1, uint32_t* o, uint32_t* g, uint32_t* attn, uint32_t* res, uint32_t* z,
                       void* h_out, const void* head, void* logits, uint64_t* am_words, int64_t* tok_out, uint32_t* epoch, int* err,
-                      int H, int D, int I, int spin, int dtype, void* stream);
+                      int64_t* trace, int H, int D, int I, int spin, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -35,8 +35,9 @@ SIGNATURES = {
     "mmf_rmsnorm_quant_fused": (_i32, [_i32, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _f32, _ptr, _f32, _ptr, _ptr, _ptr, _ptr,
                                        _ptr, _i64, _i64, _i32, _i32, _ptr]),
     "mmf_decode_layers_phase_bytes": (_i32, []),
+    "mmf_decode_layers_trace_words": (_i32, []),
     "mmf_decode_layers": (_i32, [_ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
-                                 _ptr, _ptr, _ptr, _i32, _i32, _i32, _i32, _i32, _ptr]),
+                                 _ptr, _ptr, _ptr, _ptr, _i32, _i32, _i32, _i32, _i32, _ptr]),
     "mmf_bitlinear_gemv_max_k": (_i64, []),
     "mmf_bitlinear_gemv": (_i32, [_ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _i64, _i64, _f32, _i32, _i32, _ptr]),
     "mmf_bitlinear_gemv_fused": (_i32, [_i32, _i32, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _f32, _ptr, _f32, _ptr, _ptr, _i64, _ptr,

@@ -63,8 +63,20 @@ struct LayersArgs {
     int64_t* tok_out;         // head: the greedy token
     uint32_t* epoch;          // tag base; advanced by 4 * n_layers at the end of the launch
     int* err;                 // set to 1 when a poll ran out of rounds
+    long long* trace;         // null, or kTraceWGs * kTraceLinks * kTraceStamps cycle stamps (see MMF_STAMP)
     int n_layers, H, D, I, spin;
 };
+
+// Optional cycle trace: thread 0 of three workgroups notes the shader clock at ten points of every link (entry, row
+// arrived, block norm done, sum of squares, rstd, absmax, codes in LDS, dot done, partials met, epilogue done).
+constexpr int kTraceWGs = 3, kTraceLinks = 128, kTraceStamps = 12;
+#define MMF_STAMP(i)                                                                                              \
+    do {                                                                                                          \
+        if (a.trace && threadIdx.x == 0 && tr_link < kTraceLinks) {                                               \
+            const int slot_ = blockIdx.x == 0 ? 0 : blockIdx.x == 37 ? 1 : blockIdx.x == 200 ? 2 : -1;            \
+            if (slot_ >= 0) a.trace[(slot_ * kTraceLinks + tr_link) * kTraceStamps + (i)] = __builtin_amdgcn_s_memtime(); \
+        }                                                                                                         \
+    } while (0)
 
 // A row as a phase reads it: plain elements (layer 0 reads the embedding row) or tagged words.
 struct RowSrc {
@@ -127,7 +139,8 @@ __device__ __forceinline__ float word_finish1(uint32_t w, const uint32_t* p, uin
 template <typename T, int NV, int PRO, int EPI, int S, bool PF = false>
 __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, Smem& sm, const RowSrc& xs, const RowSrc& auxs,
                                           const uint32_t* add_words, uint32_t add_tag, uint32_t* res_words,
-                                          uint32_t* out_words, uint32_t* g_words, T* plain_out, uint32_t tag_out, Best* am = nullptr) {
+                                          uint32_t* out_words, uint32_t* g_words, T* plain_out, uint32_t tag_out, int tr_link,
+                                          Best* am = nullptr) {
     constexpr int R = EPI == EPI_STEP ? 3 : EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int BPW = 2 * NV;
     constexpr int GMAX = NV * kNW / 2;
@@ -137,6 +150,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
     constexpr bool HAS_W1 = PRO >= PRO_NORM;
     constexpr int NWREG = S == 1 ? R * BPW : ITEMS;
 
+    MMF_STAMP(0);
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int K = ph.K, KB = (K + 127) >> 7, Kp = KB << 7;
     const int Nseg = ph.N / R;
@@ -275,6 +289,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
         }
     }
 
+    MMF_STAMP(1);
     // ---- prologue stage 1
     if constexpr (PRO == PRO_RESNORM) {
 #pragma unroll
@@ -313,6 +328,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
         }
     }
 
+    MMF_STAMP(2);
     // ---- prologue stage 2: the BitLinear's own norm, absmax int8 codes into LDS
     double ss = 0.0;
 #pragma unroll
@@ -320,7 +336,9 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
 #pragma unroll
         for (int i = 0; i < 4; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
     ss = mmf_block_sum_once<kNW>(ss, sm.red_b);
+    MMF_STAMP(3);
     const float rstd = mmf_rstd(ss, K, ph.inv_K, ph.eps);
+    MMF_STAMP(4);
     float amax = 0.0f;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
@@ -334,6 +352,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
         }
     }
     amax = mmf_block_max_once<kNW>(amax, sm.red_f);
+    MMF_STAMP(5);
     const float scale = __fdiv_rn(127.0f, fmaxf(amax, 1e-5f));
     const float deq = __fdiv_rn(1.0f, scale);                 // needed by the epilogue only: computed here, in the shadow of the barriers
     int qs = 0;
@@ -352,6 +371,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
         }
     }
     __syncthreads();
+    MMF_STAMP(6);
     qs = mmf_wave_sum(qs);
     if (lane == 0) sm.red_q[wave] = qs;
 
@@ -386,7 +406,9 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
                 }
             }
         }
+        MMF_STAMP(7);
         __syncthreads();
+        MMF_STAMP(8);
         const int ch = nb * 32 + sub * CHN + (lane & (CHN - 1));
         if constexpr (EPI == EPI_STEP && S == 4) {
             // Lanes 0-7 take the i rows, 8-15 the f rows, 16-23 the g rows of the same 8 channels, so the two exp /
@@ -469,6 +491,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
                 ll_st4(out_words + ch, make_word<T>(__fdiv_rn(__fmul_rn(g, u), __fadd_rn(1.0f, mmf_exp(-g))), tag_out));
             }
         }
+        MMF_STAMP(9);
         __syncthreads();                                        // part[] and the wave-0 registers are reused by the next block
     };
 #pragma unroll
@@ -505,27 +528,27 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
         {
             const Phase p = ph[0];
             if ((p.N / 3 + 31) / 32 <= 64)
-                run_phase<T, NVH, PRO_NORM, EPI_STEP, 4>(p, a, sm, h_in, none, nullptr, 0u, nullptr, a.ob, a.gb, nullptr, tag_of(4 * l));
+                run_phase<T, NVH, PRO_NORM, EPI_STEP, 4>(p, a, sm, h_in, none, nullptr, 0u, nullptr, a.ob, a.gb, nullptr, tag_of(4 * l), 4 * l);
             else
-                run_phase<T, NVH, PRO_NORM, EPI_STEP, 1>(p, a, sm, h_in, none, nullptr, 0u, nullptr, a.ob, a.gb, nullptr, tag_of(4 * l));
+                run_phase<T, NVH, PRO_NORM, EPI_STEP, 1>(p, a, sm, h_in, none, nullptr, 0u, nullptr, a.ob, a.gb, nullptr, tag_of(4 * l), 4 * l);
         }
         // gated norm -> o_proj
         {
             const Phase p = ph[1];
             const RowSrc g_in{nullptr, a.gb, tag_of(4 * l)}, o_in{nullptr, a.ob, tag_of(4 * l)};
             if ((p.N + 31) / 32 <= 64)
-                run_phase<T, NVH, PRO_GATEDNORM, EPI_PLAIN, 4>(p, a, sm, g_in, o_in, nullptr, 0u, nullptr, a.ab, nullptr, nullptr, tag_of(4 * l + 1));
+                run_phase<T, NVH, PRO_GATEDNORM, EPI_PLAIN, 4>(p, a, sm, g_in, o_in, nullptr, 0u, nullptr, a.ab, nullptr, nullptr, tag_of(4 * l + 1), 4 * l + 1);
             else
-                run_phase<T, NVH, PRO_GATEDNORM, EPI_PLAIN, 1>(p, a, sm, g_in, o_in, nullptr, 0u, nullptr, a.ab, nullptr, nullptr, tag_of(4 * l + 1));
+                run_phase<T, NVH, PRO_GATEDNORM, EPI_PLAIN, 1>(p, a, sm, g_in, o_in, nullptr, 0u, nullptr, a.ab, nullptr, nullptr, tag_of(4 * l + 1), 4 * l + 1);
         }
         // residual + norm -> gate_proj -> swiglu
         {
             const Phase p = ph[2];
             const RowSrc a_in{nullptr, a.ab, tag_of(4 * l + 1)};
             if ((p.N / 2 + 31) / 32 <= 64)
-                run_phase<T, NVH, PRO_RESNORM, EPI_SWIGLU, 4>(p, a, sm, a_in, h_in, nullptr, 0u, a.rb, a.zb, nullptr, nullptr, tag_of(4 * l + 2));
+                run_phase<T, NVH, PRO_RESNORM, EPI_SWIGLU, 4>(p, a, sm, a_in, h_in, nullptr, 0u, a.rb, a.zb, nullptr, nullptr, tag_of(4 * l + 2), 4 * l + 2);
             else
-                run_phase<T, NVH, PRO_RESNORM, EPI_SWIGLU, 1>(p, a, sm, a_in, h_in, nullptr, 0u, a.rb, a.zb, nullptr, nullptr, tag_of(4 * l + 2));
+                run_phase<T, NVH, PRO_RESNORM, EPI_SWIGLU, 1>(p, a, sm, a_in, h_in, nullptr, 0u, a.rb, a.zb, nullptr, nullptr, tag_of(4 * l + 2), 4 * l + 2);
         }
         // down_proj + residual
         {
@@ -533,9 +556,9 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
             const RowSrc z_in{nullptr, a.zb, tag_of(4 * l + 2)};
             T* plain = last ? static_cast<T*>(a.h_out) : nullptr;
             if ((p.N + 31) / 32 <= 64)
-                run_phase<T, NVI, PRO_PLAIN, EPI_PLAIN, 4>(p, a, sm, z_in, none, a.rb, tag_of(4 * l + 2), nullptr, a.hb[l & 1], nullptr, plain, tag_of(4 * l + 3));
+                run_phase<T, NVI, PRO_PLAIN, EPI_PLAIN, 4>(p, a, sm, z_in, none, a.rb, tag_of(4 * l + 2), nullptr, a.hb[l & 1], nullptr, plain, tag_of(4 * l + 3), 4 * l + 3);
             else
-                run_phase<T, NVI, PRO_PLAIN, EPI_PLAIN, 1>(p, a, sm, z_in, none, a.rb, tag_of(4 * l + 2), nullptr, a.hb[l & 1], nullptr, plain, tag_of(4 * l + 3));
+                run_phase<T, NVI, PRO_PLAIN, EPI_PLAIN, 1>(p, a, sm, z_in, none, a.rb, tag_of(4 * l + 2), nullptr, a.hb[l & 1], nullptr, plain, tag_of(4 * l + 3), 4 * l + 3);
         }
     }
     if (a.head) {
@@ -546,7 +569,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
         const uint32_t tag_h = tag_of(4 * L);
         Best best{0.0f, kNone};
         run_phase<T, NVH, PRO_NORM, EPI_PLAIN, 1, true>(p, a, sm, h_last, none, nullptr, 0u, nullptr, nullptr, nullptr,
-                                                  static_cast<T*>(a.logits), tag_h, &best);
+                                                  static_cast<T*>(a.logits), tag_h, 4 * L, &best);
         const int lane = threadIdx.x & 63;
         if (threadIdx.x < 64) {                                  // wave 0 holds the candidates of its 32 epilogue lanes
 #pragma unroll
@@ -606,10 +629,12 @@ extern "C" {
 
 int mmf_decode_layers_phase_bytes(void) { return (int)sizeof(Phase); }
 
+int mmf_decode_layers_trace_words(void) { return kTraceWGs * kTraceLinks * kTraceStamps; }
+
 int mmf_decode_layers(const void* phases, int n_layers, const void* table, const int64_t* tok, int64_t vocab,
                       uint32_t* h0, uint32_t* h1, uint32_t* o, uint32_t* g, uint32_t* attn, uint32_t* res, uint32_t* z,
                       void* h_out, const void* head, void* logits, uint64_t* am_words, int64_t* tok_out, uint32_t* epoch, int* err,
-                      int H, int D, int I, int spin, int dtype, void* stream_) {
+                      int64_t* trace, int H, int D, int I, int spin, int dtype, void* stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (!phases || n_layers <= 0 || !table || !tok || vocab <= 0 || !h0 || !h1 || !o || !g || !attn || !res || !z || !h_out ||
         !epoch || !err || H <= 0 || D <= 0 || I <= 0 || spin <= 0)
@@ -629,7 +654,7 @@ int mmf_decode_layers(const void* phases, int n_layers, const void* table, const
     a.phases = static_cast<const Phase*>(phases); a.n_layers = n_layers; a.table = table; a.tok = tok; a.vocab = vocab;
     a.hb[0] = h0; a.hb[1] = h1; a.ob = o; a.gb = g; a.ab = attn; a.rb = res; a.zb = z; a.h_out = h_out; a.head = static_cast<const Phase*>(head); a.logits = logits; a.am_words = am_words; a.tok_out = tok_out;
     a.epoch = epoch;
-    a.err = err; a.H = H; a.D = D; a.I = I; a.spin = spin;
+    a.err = err; a.trace = reinterpret_cast<long long*>(trace); a.H = H; a.D = D; a.I = I; a.spin = spin;
     switch (dtype) {
         case MMF_BF16: return launch_layers<bf16_t>(a, stream);
         case MMF_F16: return launch_layers<f16_t>(a, stream);

@@ -200,13 +200,22 @@ class DecodeEngine:
         self.epoch = torch.zeros(1, dtype=torch.int32, device=self.dev)
         self.err = torch.zeros(1, dtype=torch.int32, device=self.dev)
 
-    def _launch_layers(self, with_head: bool):
+    def _launch_layers(self, with_head: bool, trace: Optional[torch.Tensor] = None):
         w = [t.data_ptr() for t in self.words]
         head = self.phases.data_ptr() + 4 * self.L * ctypes.sizeof(_Phase) if with_head else None
         L.check(self.lib.mmf_decode_layers(self.phases.data_ptr(), self.L, self.table.data_ptr(), self.tok.data_ptr(), self.V,
                                            *w, self.h.data_ptr(), head, self.logits.data_ptr(), self.am_words.data_ptr(),
-                                           self.tok.data_ptr(), self.epoch.data_ptr(), self.err.data_ptr(), self.H, self.D,
-                                           self.I, self.SPIN, self.dt_id, L.stream()), "mmf_decode_layers")
+                                           self.tok.data_ptr(), self.epoch.data_ptr(), self.err.data_ptr(), L.ptr(trace),
+                                           self.H, self.D, self.I, self.SPIN, self.dt_id, L.stream()), "mmf_decode_layers")
+
+    def link_trace(self) -> torch.Tensor:
+        """One resident step with the kernel's cycle trace on: int64 [3 workgroups, 128 links, 12 stamps] (see
+        mmf_decode_layers in include/mmf.h), on the host."""
+        assert self.resident
+        t = torch.zeros(self.lib.mmf_decode_layers_trace_words(), dtype=torch.int64, device=self.dev)
+        self._launch_layers(True, trace=t)
+        torch.cuda.synchronize(self.dev)
+        return t.view(3, 128, 12).cpu()
 
     def _launch_step_resident(self):
         self._launch_layers(True)       # the whole step: final norm, lm_head and argmax are the launch's last two links

@@ -191,15 +191,16 @@ def test_rejected_shapes_and_pointers_return_their_code_before_any_launch():
     assert lib.mmf_hgrn_gate(P, 32, P, 64, None, None, P, P, 2, 64, 1, None) == -1
     # resident layer chain: D must equal H, rows are whole k-blocks, 16-bit activations only, bounded widths, aligned rows
     layers = lambda h, d, i, dtype=1, h0=P, spin=100: lib.mmf_decode_layers(P, 2, P, P, 1000, h0, P, P, P, P, P, P, P, None, None, None,
-                                                                          None, P, P, h, d, i, spin, dtype, None)
+                                                                          None, P, P, None, h, d, i, spin, dtype, None)
     assert layers(512, 256, 1536) == -1 and layers(500, 500, 1536) == -1 and layers(512, 512, 1500) == -1
     assert layers(512, 512, 1536, dtype=0) == -1 and layers(512, 512, 1536, spin=0) == -1
     assert layers(4224, 4224, 4096) == -2 and layers(2048, 2048, 8320) == -2
     assert layers(512, 512, 1536, h0=P + 4) == -3
-    assert lib.mmf_decode_layers(None, 2, P, P, 1000, P, P, P, P, P, P, P, P, None, None, None, None, P, P, 512, 512, 1536,
+    assert lib.mmf_decode_layers(None, 2, P, P, 1000, P, P, P, P, P, P, P, P, None, None, None, None, P, P, None, 512, 512, 1536,
                                  100, 1, None) == -1
-    assert lib.mmf_decode_layers(P, 2, P, P, 1000, P, P, P, P, P, P, P, P, P, None, P, P, P, P, 512, 512, 1536, 100, 1,
+    assert lib.mmf_decode_layers(P, 2, P, P, 1000, P, P, P, P, P, P, P, P, P, None, P, P, P, P, None, 512, 512, 1536, 100, 1,
                                  None) == -1                      # a head record without its logits buffer
+    assert lib.mmf_decode_layers_trace_words() == 3 * 128 * 12
     assert lib.mmf_decode_layers_phase_bytes() == 80
 
 
