@@ -219,6 +219,55 @@ int mmf_argmax(const void* logits, int64_t ld, int64_t rows, int64_t V, int64_t*
 int mmf_cross_entropy_fwd(const void* logits, int64_t ld, const int64_t* labels, int64_t ignore_index, float* loss,
                           int64_t rows, int64_t V, int dtype, void* stream);
 
+/* ---- training side: backward kernels and the fused loss ------------------------------------------
+ * Gradients are fp32 arithmetic (hardware exp / log), compared with autograd through the reference formulation to a
+ * tolerance.  Sums over rows (norm weight, lower bound) are accumulated per workgroup, written as [groups, K] fp32
+ * partials (groups = mmf_backward_groups(rows); the caller provides the buffer) and added in a fixed order.
+ *
+ * mmf_rmsnorm_bwd replaces the Triton backward kernels of the three norms:
+ *   mode 0  RMSNorm                    mmfreelm/modules/layernorm.py:245-330 (LayerNormFn.backward :484-531)
+ *   mode 1  RMSNorm * swish gate       mmfreelm/modules/fused_norm_gate.py:210-300 (:462-500); also returns dgate
+ *   mode 2  BitLinear's norm           mmfreelm/ops/fusedbitnet.py:209-317 (LayerNormLinearQuantFn.backward :470-510): the
+ *           gradient passes through the activation quantiser unchanged (straight-through, :571) and y_quant receives the
+ *           de-quantised int8 output recomputed with the forward arithmetic, for the weight gradient dout^T y (:498)
+ *   x [M, K] (row stride ldx) is what the norm normalised (the summed residual where the forward added one); rstd is
+ *   recomputed from it.  dx = (w dy - xhat mean(xhat w dy)) rstd (+ dresidual, the gradient arriving through a prenorm
+ *   residual output); dweight [K] (weight dtype) = sum over rows of dy xhat, needs dw_partial [groups, K] fp32. */
+int mmf_backward_groups(int64_t rows);
+int mmf_rmsnorm_bwd(int mode, const void* x, int64_t ldx, const void* gate, int64_t ldg, const void* weight, const void* dy,
+                    int64_t lddy, const void* dresidual, void* dx, void* dgate, void* y_quant, float* dw_partial, void* dweight,
+                    int64_t M, int64_t K, float eps, int x_dtype, int weight_dtype, void* stream);
+/* mmf_swiglu_bwd replaces swiglu_bwd, mmfreelm/modules/activations.py:121-126: with s = sigmoid(x),
+ *   dx = s (1 + x (1 - s)) g y,  dy = x s g; every operand may be a column slice (leading dimensions in elements). */
+int mmf_swiglu_bwd(const void* x, int64_t ldx, const void* y, int64_t ldy, const void* g, int64_t ldg, void* dx, int64_t lddx,
+                   void* dy, int64_t lddy, int64_t rows, int64_t cols, int dtype, void* stream);
+/* mmf_hgrn_gate_bwd: gradient of the gate math mmf_hgrn_gate fuses (what autograd derives for
+ *   mmfreelm/layers/hgrn_bit.py:113-120): from grad_x, grad_g [rows, D] to di, df (leading dimensions lddi, lddf) and, with a
+ *   lower bound, dlb [D] fp32 = sum over rows of (grad_g - grad_x i sigmoid(i)) (1 - sigmoid(f)) (dlb_partial: [groups, D]). */
+int mmf_hgrn_gate_bwd(const void* i_in, int64_t ldi, const void* f_in, int64_t ldf, const float* lower_bound, const uint8_t* mask,
+                      const void* grad_x, const void* grad_g, void* di, int64_t lddi, void* df, int64_t lddf, float* dlb_partial,
+                      float* dlb, int64_t rows, int64_t D, int dtype, void* stream);
+/* mmf_hgrn_recurrent_bwd replaces fused_recurrent_hgrn_bwd_kernel, mmfreelm/ops/hgrn/recurrent_fuse.py:89-133 (backward
+ *   :158-173): time runs backwards, dh += do_t; dx_t = dh; dg_t = dh h_{t-1}; dh *= g_t, with h_{-1} = h0 (or 0).  o is the
+ *   forward output.  log_gates = 1: g holds log decays (chunk_hgrn, mmfreelm/ops/hgrn/chunk.py:137-220): the step uses
+ *   exp(g_t) and dg_t = dh h_{t-1} exp(g_t).  As in the reference the gradient of the final state is not propagated. */
+int mmf_hgrn_recurrent_bwd(const void* g, const void* o, const void* grad_o, const float* h0, void* dx, void* dg, int64_t BH,
+                           int64_t T, int64_t D, int log_gates, int dtype, void* stream);
+/* mmf_cross_entropy_train_fwd / _bwd replace cross_entropy_fwd_kernel / cross_entropy_bwd_kernel,
+ *   mmfreelm/modules/fused_cross_entropy.py:26-98 / :98-160 (CrossEntropyLossFunction :163-310, one device): per row, with
+ *   l = logit_scale * logits, lse = logsumexp(l):
+ *     loss = lse - smoothing mean(l) - (1 - smoothing) l[label] + lse_square_scale lse^2   (0 where label == ignore_index;
+ *            a label outside [0, V) keeps only the smoothing and z terms, as the reference's out-of-range case does);
+ *     z_loss (optional) = lse_square_scale lse^2;  lse is kept for the backward;
+ *     dlogits = dloss logit_scale ( exp(l - lse) (1 + 2 lse_square_scale lse) - onehot (1 - smoothing) - smoothing / V ).
+ *   dlogits may be the logits buffer itself (the reference's inplace_backward). */
+int mmf_cross_entropy_train_fwd(const void* logits, int64_t ld, const int64_t* labels, int64_t ignore_index, float smoothing,
+                                float logit_scale, float lse_square_scale, float* loss, float* lse, float* z_loss, int64_t rows,
+                                int64_t V, int dtype, void* stream);
+int mmf_cross_entropy_train_bwd(const void* logits, int64_t ld, const int64_t* labels, int64_t ignore_index, const float* lse,
+                                const float* dloss, float smoothing, float logit_scale, float lse_square_scale, void* dlogits,
+                                int64_t ldd, int64_t rows, int64_t V, int dtype, void* stream);
+
 /* ---- top-p (nucleus) sampling of the next token -----------------------------------------------
  * mmf_sample_top_p replaces, per decoded token of the loop that mmfreelm's generate.py:11 runs
  *   (model.generate(do_sample=True, top_p=0.4, temperature=0.6)), what transformers' sampling path does with the

@@ -87,6 +87,8 @@ class HGRNBitAttention(nn.Module):
         stacked i/f/g projection instead of running as a launch of its own."""
         B, T, _ = hidden_states.shape
         D = self.input_dim
+        if self.training and torch.is_grad_enabled():
+            return self._forward_train(hidden_states, attention_mask, lower_bound, input_norm), None, past_key_values
         last_state = past_key_values[self.layer_idx] if use_cache else None
 
         stacked = self._stacked_ifg()
@@ -125,6 +127,22 @@ class HGRNBitAttention(nn.Module):
         # g_norm (layers/hgrn_bit.py:138) folded into o_proj
         o = self.o_proj.forward_fused(g, ("gatednorm", o.reshape(g.shape), self.g_norm.weight, self.g_norm.eps))
         return o, None, past_key_values
+
+    def _forward_train(self, hidden_states, attention_mask, lower_bound, input_norm):
+        """The layer as the reference composes it (mmfreelm/layers/hgrn_bit.py:110-140), one autograd Function per op;
+        no state cache (training runs whole sequences)."""
+        from .autograd import HGRNGateFn
+        from .hgrn import fused_recurrent_hgrn
+        B, T, _ = hidden_states.shape
+        D = self.input_dim
+        if input_norm is not None:
+            hidden_states = input_norm(hidden_states)
+        i, f, g = self.i_proj(hidden_states), self.f_proj(hidden_states), self.g_proj(hidden_states)
+        lb = lower_bound if (lower_bound is not None and self.layer_idx > 0) else None
+        x_in, gate = HGRNGateFn.apply(i, f, lb, attention_mask)
+        o, _ = fused_recurrent_hgrn(x_in.view(B, 1, T, D), gate.view(B, 1, T, D))
+        o = self.g_norm(g, o.view(B, T, D))
+        return self.o_proj(o)
 
     def init_state(self, batch_size: int) -> Tuple[torch.Tensor]:
         """Zero recurrent state [B, num_heads, head_dim], kept in fp32."""

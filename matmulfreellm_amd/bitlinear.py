@@ -55,6 +55,11 @@ def layer_norm_linear_quant_fn(x, norm_weight, norm_bias, linear_weight, linear_
     if not is_rms_norm or norm_bias is not None:
         raise NotImplementedError("only is_rms_norm=True with norm_bias=None is implemented "
                                   "(the only form FusedBitLinear uses, fusedbitnet.py:602-610)")
+    from .autograd import BitLinearFn, needs_grad
+    if needs_grad(x, norm_weight, linear_weight, linear_bias, residual):
+        if linear_weight.is_meta:
+            raise RuntimeError("this BitLinear holds packed codes only: there is no latent weight to train")
+        return BitLinearFn.apply(x, norm_weight, linear_weight, linear_bias, eps, residual, prenorm, residual_in_fp32, packed)
     pw = packed if packed is not None else F_.ternarize_pack(linear_weight)
     return F_.bitlinear(x, norm_weight, pw, bias=linear_bias, eps=eps, residual=residual, prenorm=prenorm,
                         residual_in_fp32=residual_in_fp32)

@@ -9,6 +9,11 @@ def rms_norm_swish_gate_fn(x, o, weight, bias, residual=None, prenorm=False, res
     """mmfreelm/modules/fused_norm_gate.py:510 (there named rms_norm_fn)."""
     if bias is not None:
         raise NotImplementedError("bias is not on the MatMul-free LM path (reference registers bias=None)")
+    from .autograd import RMSNormSwishGateFn, needs_grad
+    if needs_grad(x, o, weight, residual):
+        if residual is not None or prenorm:
+            raise NotImplementedError("the gated norm's backward takes no residual (the model never gives it one)")
+        return RMSNormSwishGateFn.apply(x, o, weight, eps)
     return F_.rmsnorm_swishgate(x, o, weight, residual=residual, eps=eps, prenorm=prenorm,
                                 residual_in_fp32=residual_in_fp32)
 

@@ -13,6 +13,9 @@ def fused_recurrent_hgrn(x: torch.Tensor, g: torch.Tensor, initial_state: Option
     The final state is returned in fp32 (the reference returns it in x.dtype)."""
     if initial_state is not None:
         initial_state = initial_state.detach()
+    from .autograd import FusedRecurrentHGRNFn, needs_grad
+    if needs_grad(x, g):
+        return FusedRecurrentHGRNFn.apply(x, g, initial_state, output_final_state)
     return F_.hgrn_recurrent(x, g, initial_state, output_final_state)
 
 
@@ -21,4 +24,7 @@ def chunk_hgrn(x: torch.Tensor, g: torch.Tensor, initial_state: Optional[torch.T
     """h_t = exp(g_t) * h_{t-1} + x_t with g the LOG decay (<= 0).  Same shapes; fp32 final state."""
     if initial_state is not None:
         initial_state = initial_state.detach()
+    from .autograd import ChunkHGRNFn, needs_grad
+    if needs_grad(x, g):
+        return ChunkHGRNFn.apply(x, g, initial_state, output_final_state, chunk_size)
     return F_.hgrn_chunk(x, g, initial_state, output_final_state, chunk_size)

@@ -9,6 +9,9 @@ def rms_norm_fn(x, weight, bias, residual=None, prenorm=False, residual_in_fp32=
     """Same signature as mmfreelm/modules/layernorm.py:534.  bias must be None (the model never sets one)."""
     if bias is not None:
         raise NotImplementedError("RMSNorm bias is not on the MatMul-free LM path (reference registers bias=None)")
+    from .autograd import RMSNormFn, needs_grad
+    if needs_grad(x, weight, residual):
+        return RMSNormFn.apply(x, weight, residual, eps, prenorm, residual_in_fp32)
     return F_.rmsnorm(x, weight, residual=residual, eps=eps, prenorm=prenorm, residual_in_fp32=residual_in_fp32)
 
 

@@ -69,6 +69,14 @@ class HGRNBitMLP(nn.Module):
         fused into down_proj's epilogue; with ``pre_norm`` (the block's mlp_norm) x is the attention
         output and the residual add + RMSNorm in front of gate_proj (:107) is folded into gate_proj."""
         inter = self.intermediate_size
+        if self.training and torch.is_grad_enabled():
+            # the reference's composition (:55-59) through the autograd Functions; the block's norm and residual as :107-109
+            from .activations import swiglu
+            if pre_norm is not None:
+                x, residual = pre_norm(x, residual, True)
+            y = self.gate_proj(x)
+            z = self.down_proj(swiglu(y[..., :inter], y[..., inter:]))
+            return z if residual is None else residual + z
         rows = x.numel() // x.shape[-1]
         # long prompts: the tiled gate/up contraction applies the swiglu itself and down_proj quantises its result
         in_epilogue = (self.gate_proj.bias is None and x.is_cuda
@@ -168,12 +176,20 @@ class HGRNBitModel(HGRNBitPreTrainedModel):
             self._lb_key, self._lb = key, lower_bound_schedule(p)
         return self._lb
 
-    @torch.no_grad()
     def forward(self, input_ids: Optional[torch.LongTensor] = None, attention_mask: Optional[torch.Tensor] = None,
                 inputs_embeds: Optional[torch.FloatTensor] = None, past_key_values=None,
                 use_cache: Optional[bool] = None, output_attentions: Optional[bool] = None,
                 output_hidden_states: Optional[bool] = None, return_dict: Optional[bool] = None
                 ) -> Union[Tuple, BaseModelOutputWithPast]:
+        """Training mode with gradients enabled runs the reference's op-by-op composition through the autograd
+        Functions (matmulfreellm_amd/autograd.py); everything else runs the fused inference launches without a graph."""
+        train = self.training and torch.is_grad_enabled()
+        with torch.enable_grad() if train else torch.no_grad():
+            return self._forward(train, input_ids, attention_mask, inputs_embeds, past_key_values, use_cache,
+                                 output_attentions, output_hidden_states, return_dict)
+
+    def _forward(self, train, input_ids, attention_mask, inputs_embeds, past_key_values, use_cache, output_attentions,
+                 output_hidden_states, return_dict):
         if output_attentions:
             warnings.warn("`HGRNBitModel` does not `output_attentions` now, setting it to `False`.")
         output_attentions = False
@@ -192,8 +208,10 @@ class HGRNBitModel(HGRNBitPreTrainedModel):
             raise ValueError("You have to specify either input_ids or inputs_embeds")
 
         if inputs_embeds is None:
-            inputs_embeds = F_.embedding(self.embeddings.weight, input_ids)
+            inputs_embeds = self.embeddings(input_ids) if train else F_.embedding(self.embeddings.weight, input_ids)
         hidden_states = inputs_embeds
+        if train:
+            use_cache = False                                    # whole sequences, no recurrent-state cache
 
         if use_cache:
             if past_key_values is None:
@@ -202,7 +220,13 @@ class HGRNBitModel(HGRNBitPreTrainedModel):
                 past_key_values = RecurrentCache.from_legacy_cache(past_key_values)
 
         all_hidden_states = () if output_hidden_states else None
-        lower_bounds = self.lower_bound_rows() if self.config.use_lower_bound else None
+        if not self.config.use_lower_bound:
+            lower_bounds = None
+        elif train:                                              # differentiable (modeling_hgrn_bit.py:231-233)
+            lower_bounds = self.lower_bounds.float().softmax(0)
+            lower_bounds = lower_bounds.cumsum(0) - lower_bounds[0]
+        else:
+            lower_bounds = self.lower_bound_rows()
         for i, layer in enumerate(self.layers):
             if output_hidden_states:
                 all_hidden_states += (hidden_states,)
@@ -289,12 +313,18 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
             model_inputs["logits_to_keep"] = kwargs["logits_to_keep"]
         return model_inputs
 
-    @torch.no_grad()
     def forward(self, input_ids: torch.LongTensor = None, attention_mask: Optional[torch.Tensor] = None,
                 inputs_embeds: Optional[torch.Tensor] = None, past_key_values=None,
                 labels: Optional[torch.LongTensor] = None, use_cache: Optional[bool] = None,
                 output_attentions: Optional[bool] = None, output_hidden_states: Optional[bool] = None,
                 return_dict: Optional[bool] = None, logits_to_keep: int = 0) -> Union[Tuple, CausalLMOutputWithPast]:
+        train = self.training and torch.is_grad_enabled()
+        with torch.enable_grad() if train else torch.no_grad():
+            return self._forward(train, input_ids, attention_mask, inputs_embeds, past_key_values, labels, use_cache,
+                                 output_attentions, output_hidden_states, return_dict, logits_to_keep)
+
+    def _forward(self, train, input_ids, attention_mask, inputs_embeds, past_key_values, labels, use_cache, output_attentions,
+                 output_hidden_states, return_dict, logits_to_keep):
         if labels is not None:
             logits_to_keep = 0                           # the loss scores every position
         return_dict = return_dict if return_dict is not None else bool(getattr(self.config, "return_dict", True))
@@ -311,7 +341,12 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
             # as mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py:388-397: position t is scored against token t + 1
             labels = labels.to(logits.device)
             targets = torch.cat((labels[..., 1:], torch.full_like(labels[:, :1], -100)), 1)
-            loss = F_.cross_entropy(logits, targets, ignore_index=-100)
+            if train:
+                # FusedCrossEntropyLoss(inplace_backward=True) as :389-391 (nn.CrossEntropyLoss gives the same value)
+                from .autograd import FusedCrossEntropyLoss
+                loss = FusedCrossEntropyLoss(inplace_backward=True)(logits.view(-1, logits.shape[-1]), targets.view(-1))
+            else:
+                loss = F_.cross_entropy(logits, targets, ignore_index=-100)
         if not return_dict:
             return tuple(x for x in (loss, logits, outputs.past_key_values, outputs.hidden_states) if x is not None)
         return CausalLMOutputWithPast(loss=loss, logits=logits, past_key_values=outputs.past_key_values,

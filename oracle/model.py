@@ -7,6 +7,9 @@ mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py wires the fused ones:
   HGRNBitAttention.forward mmfreelm/layers/hgrn_bit.py:83-142, lm_head :386,
   lower bounds :231-238 (softmax over layers, cumsum, minus first row).
 
+``mode="literal_ste"`` is the literal mode with the straight-through estimators of mmfreelm/ops/fusedbitnet.py:571-573 on
+both quantisers, so that torch.autograd differentiates it as the reference's training path does.
+
 ``forward(..., mode="spec")`` uses the *_spec ops (what the HIP path must reproduce bit for
 bit); ``mode="literal"`` uses the *_literal ops in the parameters' dtype (the reference's
 PyTorch formulation: fake-quantised floats, F.linear, torch sigmoid/exp, recurrent state
@@ -91,7 +94,11 @@ class _Ops:
             if residual_add is not None:
                 out = (out.to(_F) + residual_add.to(_F)).to(x.dtype)
             return out
-        out = ob.bitlinear_literal(x, w, nw, eps=self.bl_eps)
+        if self.mode == "literal_ste":
+            from .backward import bitlinear_ste
+            out = bitlinear_ste(x, w, nw, eps=self.bl_eps)
+        else:
+            out = ob.bitlinear_literal(x, w, nw, eps=self.bl_eps)
         return out if residual_add is None else residual_add + out
 
     def rmsnorm(self, x, w, eps, residual=None, prenorm=False):
