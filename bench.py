@@ -21,8 +21,9 @@ inputs resident in HBM.  Prints ONE JSON line:
   extra        batch-64 decode, prompt prefill (8 x 512 and 8 x 2048 tokens, with the whole forward's
                int8 TOP/s against 5.0 POP/s), prefill-sized BitLinear on the int8 matrix cores,
                HGRN scan, norm and loss bandwidths (cache-cold: the legs rotate through buffer sets
-               of more than 512 MB in total; counted HBM traffic from rocprofv3 beside each).
---only runs the named legs only (decode, bs64, prefill, mfma, scan, norms, sampling, loss, cpu, link_trace): the
+               of more than 512 MB in total; counted HBM traffic from rocprofv3 beside each),
+               and one training step (forward + loss + backward) of the same model at 8 x 1024 tokens.
+--only runs the named legs only (decode, bs64, prefill, mfma, scan, norms, sampling, loss, train, cpu, link_trace): the
 profiles under profiles/ are made that way.
 Synthetic data: random-init N(0, 0.02) weights, uniform random token ids.
 """
@@ -329,6 +330,45 @@ def sampler_bench(model, dev, n_new=256):
     return res
 
 
+def train_bench(model, dev, batch=8, seq=1024, iters=3):
+    """One training step of the module path: forward with the fused loss, backward to the gradient of every
+    parameter (no optimiser step), plus the two backward kernels that carry the most bytes, timed alone."""
+    import matmulfreellm_amd as mm
+    g = torch.Generator(device=dev).manual_seed(9)
+    ids = torch.randint(0, model.config.vocab_size, (batch, seq), generator=g, device=dev)
+    model.train()
+
+    def step():
+        for p in model.parameters():
+            p.grad = None
+        model(input_ids=ids, labels=ids).loss.backward()
+    try:
+        ms = timed(step, iters, warmup=2)
+    finally:
+        model.eval()
+        for p in model.parameters():
+            p.grad = None
+    res = {"batch": batch, "seq_len": seq, "ms_per_step": round(ms, 2), "tok_s": round(batch * seq / ms * 1e3),
+           "what": "forward + loss + backward, bf16 parameters, no optimiser step"}
+    b, t, d = 8, 2048, model.config.hidden_size
+    x = torch.randn(b, 1, t, d, generator=g, device=dev).bfloat16().requires_grad_()
+    gt = torch.sigmoid(torch.randn(b, 1, t, d, generator=g, device=dev)).bfloat16().requires_grad_()
+    o, _ = mm.fused_recurrent_hgrn(x, gt)
+    do = torch.randn_like(o)
+    ms_s = timed(lambda: torch.autograd.grad(o, (x, gt), do, retain_graph=True), 10)
+    res["scan_backward"] = {"shape": [b, t, d], "ms": round(ms_s, 4), "GBs": round(5 * b * t * d * 2 / ms_s / 1e6, 1),
+                            "algorithmic_bytes": 5 * b * t * d * 2}
+    m, k = 16384, d
+    xn = torch.randn(m, k, generator=g, device=dev).bfloat16().requires_grad_()
+    norm = mm.RMSNorm(k).to(dev, torch.bfloat16)
+    y = norm(xn)
+    dy = torch.randn_like(y)
+    ms_n = timed(lambda: torch.autograd.grad(y, (xn, norm.weight), dy, retain_graph=True), 10)
+    res["rmsnorm_backward"] = {"shape": [m, k], "ms": round(ms_n, 4), "GBs": round(3 * m * k * 2 / ms_n / 1e6, 1),
+                               "algorithmic_bytes": 3 * m * k * 2}
+    return res
+
+
 def _cpu_model():
     try:
         for line in open("/proc/cpuinfo"):
@@ -423,7 +463,7 @@ def main():
                     help="batch 1: one launch per fused BitLinear instead of the resident layer chain")
     ap.add_argument("--no-extra", action="store_true", help="skip the batch-64 / matrix-core / scan / norm / CPU legs")
     ap.add_argument("--only", default="", help="comma-separated legs to run instead of everything: decode, bs64, prefill, mfma, "
-                                               "scan, norms, sampling, loss, cpu (profiling runs)")
+                                               "scan, norms, sampling, loss, train, cpu, link_trace (profiling runs)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by)")
     args = ap.parse_args()
@@ -443,7 +483,7 @@ def main():
         dst.copy_(src)          # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
-    if only and not (only & {"decode", "bs64", "prefill", "sampling", "link_trace"}):
+    if only and not (only & {"decode", "bs64", "prefill", "sampling", "link_trace", "train"}):
         # legs that need no model: run them alone and print what they measured
         res = {}
         if "mfma" in only:
@@ -511,6 +551,8 @@ def main():
         extra["sampling"] = sampler_bench(model, dev)
     if want("loss"):
         extra["cross_entropy"] = loss_bench(dev)
+    if want("train"):
+        extra["training_step"] = train_bench(model, dev)
     if extra:
         result["extra"] = extra
     del model, eng, eng1

@@ -147,14 +147,37 @@ __global__ __launch_bounds__(kBT) void rmsnorm_bwd_kernel(NormBwdArgs a) {
     }
 }
 
-// out[k] = T(sum_g part[g, k]), groups in index order
+// out[k] = T(sum_g part[g, k]).  A workgroup owns 32 columns; its 32 lanes per column each add every 32nd group in index order and
+// the 32 lane sums are then added in lane order, so the result depends on the shape only.
+constexpr int kColsumCols = 32, kColsumLanes = 32;
 template <typename T>
-__global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ part, int groups, int K, T* __restrict__ out) {
-    const int k = blockIdx.x * 256 + threadIdx.x;
-    if (k >= K) return;
-    float s = 0.0f;
-    for (int g = 0; g < groups; ++g) s += part[(int64_t)g * K + k];
-    out[k] = mmf_from_float<T>(s);
+__global__ __launch_bounds__(kColsumCols * kColsumLanes) void colsum_kernel(const float* __restrict__ part, int groups, int K,
+                                                                            T* __restrict__ out) {
+    __shared__ float lane_sum[kColsumLanes][kColsumCols + 1];
+    const int c = (int)threadIdx.x % kColsumCols, l = (int)threadIdx.x / kColsumCols;
+    const int k = (int)blockIdx.x * kColsumCols + c;
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+    if (k < K) {
+        int g = l;
+        for (; g + 3 * kColsumLanes < groups; g += 4 * kColsumLanes) {
+            const float a0 = part[(int64_t)g * K + k], a1 = part[(int64_t)(g + kColsumLanes) * K + k];
+            const float a2 = part[(int64_t)(g + 2 * kColsumLanes) * K + k], a3 = part[(int64_t)(g + 3 * kColsumLanes) * K + k];
+            s0 += a0; s1 += a1; s2 += a2; s3 += a3;
+        }
+        for (; g < groups; g += kColsumLanes) s0 += part[(int64_t)g * K + k];
+    }
+    lane_sum[l][c] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (l == 0 && k < K) {
+        float s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kColsumLanes; ++i) s += lane_sum[i][c];
+        out[k] = mmf_from_float<T>(s);
+    }
+}
+template <typename T>
+void launch_colsum(const float* part, int groups, int64_t K, T* out, hipStream_t s) {
+    colsum_kernel<T><<<(unsigned)mmf_ceil_div(K, kColsumCols), kColsumCols * kColsumLanes, 0, s>>>(part, groups, (int)K, out);
 }
 
 template <typename T, typename TW, int MODE>
@@ -233,25 +256,63 @@ __global__ __launch_bounds__(256) void hgrn_gate_bwd_kernel(const T* __restrict_
 }
 
 // ------------------------------------------------------------------------------------------ recurrence
-// dh += do_t; dx_t = dh; dg_t = dh * h_{t-1} (* exp(g_t) for log gates); dh *= g_t (exp(g_t)).  A lane owns a channel; time
-// runs backwards in register blocks of 32 steps whose loads are issued together.
+// dh += do_t; dx_t = dh; dg_t = dh * h_{t-1} (* exp(g_t) for log gates); dh *= g_t (exp(g_t)).  A lane owns a channel and a
+// workgroup 64 channels of one sequence; its NW waves split the time axis.  Every wave first walks its segment from a zero carry
+// and keeps the carry L it would hand to the earlier segment and the product P of its gates, then folds the (L, P) of the later
+// segments (carry = L + P * carry, last segment first) into the carry it really starts from, and walks its segment again to
+// write the gradients.  Time runs backwards in register blocks of 32 steps whose loads are issued together.
+constexpr int kScanBwdBlock = 32, kScanBwdMaxWaves = 8;
 template <typename T, bool LOG>
-__global__ __launch_bounds__(64) void hgrn_recurrent_bwd_kernel(const T* __restrict__ g, const T* __restrict__ o,
-                                                                const T* __restrict__ dout, const float* __restrict__ h0,
-                                                                T* __restrict__ dx, T* __restrict__ dg, int64_t Tlen, int64_t D) {
-    constexpr int BL = 32;
-    const int64_t d = (int64_t)blockIdx.x * 64 + threadIdx.x, bh = blockIdx.y;
-    if (d >= D) return;
-    const int64_t base = bh * Tlen * D + d;
-    const float hinit = h0 ? h0[bh * D + d] : 0.0f;
+__global__ __launch_bounds__(64 * kScanBwdMaxWaves) void hgrn_recurrent_bwd_kernel(const T* __restrict__ g, const T* __restrict__ o,
+                                                                                   const T* __restrict__ dout,
+                                                                                   const float* __restrict__ h0, T* __restrict__ dx,
+                                                                                   T* __restrict__ dg, int64_t Tlen, int64_t D,
+                                                                                   int64_t seg) {
+    constexpr int BL = kScanBwdBlock;
+    __shared__ float carry_l[kScanBwdMaxWaves][64], carry_p[kScanBwdMaxWaves][64];
+    const int lane = (int)threadIdx.x & 63, wave = (int)threadIdx.x >> 6, nw = (int)blockDim.x >> 6;
+    const int64_t d = (int64_t)blockIdx.x * 64 + lane, bh = blockIdx.y;
+    const bool live = d < D;
+    const int64_t base = bh * Tlen * D + (live ? d : 0);
+    const int64_t ta = (int64_t)wave * seg, tb = ta + seg < Tlen ? ta + seg : Tlen;   // this wave's steps ta .. tb - 1 (may be none)
     float dh = 0.0f;
-    for (int64_t t1 = Tlen; t1 > 0; t1 -= BL) {
-        const int64_t t0 = t1 - BL;                              // block covers steps max(t0, 0) .. t1 - 1
+    if (nw > 1) {
+        float prod = 1.0f;
+        if (live)
+            for (int64_t t1 = tb; t1 > ta; t1 -= BL) {
+                const int64_t t0 = t1 - BL;
+                float gv[BL], dv[BL];
+#pragma unroll
+                for (int j = 0; j < BL; ++j) {
+                    const int64_t t = t0 + j;
+                    if (t >= ta) {
+                        gv[j] = mmf_to_float(g[base + t * D]);
+                        dv[j] = mmf_to_float(dout[base + t * D]);
+                    }
+                }
+#pragma unroll
+                for (int j = BL - 1; j >= 0; --j)
+                    if (t0 + j >= ta) {
+                        const float gl = LOG ? __expf(gv[j]) : gv[j];
+                        dh = (dh + dv[j]) * gl;
+                        prod *= gl;
+                    }
+            }
+        carry_l[wave][lane] = dh;
+        carry_p[wave][lane] = prod;
+        __syncthreads();
+        dh = 0.0f;
+        for (int w = nw - 1; w > wave; --w) dh = carry_l[w][lane] + carry_p[w][lane] * dh;
+    }
+    if (!live) return;
+    const float hinit = h0 ? h0[bh * D + d] : 0.0f;
+    for (int64_t t1 = tb; t1 > ta; t1 -= BL) {
+        const int64_t t0 = t1 - BL;                              // block covers steps max(t0, ta) .. t1 - 1
         float gv[BL], dv[BL], hv[BL];
 #pragma unroll
         for (int j = 0; j < BL; ++j) {
             const int64_t t = t0 + j;
-            if (t >= 0) {
+            if (t >= ta) {
                 gv[j] = mmf_to_float(g[base + t * D]);
                 dv[j] = mmf_to_float(dout[base + t * D]);
                 hv[j] = t > 0 ? mmf_to_float(o[base + (t - 1) * D]) : hinit;
@@ -260,7 +321,7 @@ __global__ __launch_bounds__(64) void hgrn_recurrent_bwd_kernel(const T* __restr
 #pragma unroll
         for (int j = BL - 1; j >= 0; --j) {
             const int64_t t = t0 + j;
-            if (t >= 0) {
+            if (t >= ta) {
                 const float gl = LOG ? __expf(gv[j]) : gv[j];
                 dh += dv[j];
                 dx[base + t * D] = mmf_from_float<T>(dh);
@@ -377,11 +438,10 @@ int mmf_rmsnorm_bwd(int mode, const void* x, int64_t ldx, const void* gate, int6
         case MMF_F16: rc = wf32 ? dispatch_norm_bwd<f16_t, float>(a, mode, groups, stream) : dispatch_norm_bwd<f16_t, f16_t>(a, mode, groups, stream); break;
     }
     if (rc != 0 || !a.dw_part) return rc;
-    const unsigned gb = (unsigned)mmf_ceil_div(K, 256);
     switch (weight_dtype) {
-        case MMF_F32: colsum_kernel<float><<<gb, 256, 0, stream>>>(dw_partial, groups, (int)K, static_cast<float*>(dweight)); break;
-        case MMF_BF16: colsum_kernel<bf16_t><<<gb, 256, 0, stream>>>(dw_partial, groups, (int)K, static_cast<bf16_t*>(dweight)); break;
-        case MMF_F16: colsum_kernel<f16_t><<<gb, 256, 0, stream>>>(dw_partial, groups, (int)K, static_cast<f16_t*>(dweight)); break;
+        case MMF_F32: launch_colsum(dw_partial, groups, K, static_cast<float*>(dweight), stream); break;
+        case MMF_BF16: launch_colsum(dw_partial, groups, K, static_cast<bf16_t*>(dweight), stream); break;
+        case MMF_F16: launch_colsum(dw_partial, groups, K, static_cast<f16_t*>(dweight), stream); break;
         default: return MMF_ERR_ARG;
     }
     MMF_CHECK_LAUNCH();
@@ -432,7 +492,7 @@ int mmf_hgrn_gate_bwd(const void* i_in, int64_t ldi, const void* f_in, int64_t l
 #undef MMF_GB
     MMF_CHECK_LAUNCH();
     if (part) {
-        colsum_kernel<float><<<(unsigned)mmf_ceil_div(D, 256), 256, 0, stream>>>(part, groups, (int)D, dlb);
+        launch_colsum(part, groups, D, dlb, stream);
         MMF_CHECK_LAUNCH();
     }
     return 0;
@@ -445,8 +505,12 @@ int mmf_hgrn_recurrent_bwd(const void* g, const void* o, const void* grad_o, con
     if (BH == 0 || T == 0) return 0;
     if (!g || !o || !grad_o || !dx || !dg) return MMF_ERR_ARG;
     dim3 grid((unsigned)mmf_ceil_div(D, 64), (unsigned)BH);
-#define MMF_RB(T_, L_) hgrn_recurrent_bwd_kernel<T_, L_><<<grid, 64, 0, stream>>>(static_cast<const T_*>(g), static_cast<const T_*>(o), \
-        static_cast<const T_*>(grad_o), h0, static_cast<T_*>(dx), static_cast<T_*>(dg), T, D)
+    // segments of at least 64 steps, a whole number of register blocks each, at most 8 waves
+    int64_t nw = T / 64 < 1 ? 1 : T / 64 > kScanBwdMaxWaves ? kScanBwdMaxWaves : T / 64;
+    const int64_t seg = mmf_ceil_div(mmf_ceil_div(T, nw), kScanBwdBlock) * kScanBwdBlock;
+    nw = mmf_ceil_div(T, seg);
+#define MMF_RB(T_, L_) hgrn_recurrent_bwd_kernel<T_, L_><<<grid, (unsigned)(64 * nw), 0, stream>>>(static_cast<const T_*>(g), \
+        static_cast<const T_*>(o), static_cast<const T_*>(grad_o), h0, static_cast<T_*>(dx), static_cast<T_*>(dg), T, D, seg)
     switch (dtype) {
         case MMF_F32: if (log_gates) MMF_RB(float, true); else MMF_RB(float, false); break;
         case MMF_BF16: if (log_gates) MMF_RB(bf16_t, true); else MMF_RB(bf16_t, false); break;

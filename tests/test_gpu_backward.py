@@ -165,7 +165,8 @@ def test_gate_math_backward(dev, dtype, use_lb):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("bhtd", [(2, 1, 70, 128), (1, 2, 33, 100), (2, 1, 1, 64)])
+@pytest.mark.parametrize("bhtd", [(2, 1, 70, 128), (1, 2, 33, 100), (2, 1, 1, 64), (1, 2, 130, 100), (1, 1, 301, 64),
+                                  (2, 1, 1000, 192)])   # one wave; 2, 4 and 8 waves along time with ragged last segments
 @pytest.mark.parametrize("with_h0", [False, True])
 def test_recurrent_scan_backward(dev, dtype, bhtd, with_h0):
     import matmulfreellm_amd as mm
@@ -188,7 +189,7 @@ def test_recurrent_scan_backward(dev, dtype, bhtd, with_h0):
 def test_chunk_scan_backward_log_gates(dev):
     import matmulfreellm_amd as mm
     torch.manual_seed(8)
-    b, h, t, d = 2, 1, 130, 64
+    b, h, t, d = 2, 1, 330, 64
     g = torch.nn.functional.logsigmoid(torch.randn(b, h, t, d) + 1)
     x, do, h0 = torch.randn(b, h, t, d), torch.randn(b, h, t, d), torch.randn(b, h, d)
     xc, gc = leaf(x), leaf(g)
