@@ -195,8 +195,41 @@ def mfma_bench(dev, m=4096, k=2048, n=11264, iters=20):
     ms_mm = timed(lambda: F_.bitlinear_mfma(q, deq, qsum, pw, m, torch.bfloat16, out=out), iters)
     ms_q = timed(lambda: F_.rmsnorm_quant(x, nw, eps=1e-8, tiled=True), iters)
     tops = 2.0 * m * k * n / (ms_mm * 1e-3) / 1e12
+    # the clock the part sustains under this kernel: shader-clock ticks over 100 MHz ticks, per workgroup, of one launch
+    lib, wgs = F_.L.load(), (m // 64) * (n // 512)
+    clocks = torch.zeros(wgs, 2, dtype=torch.int64, device=dev)
+    F_.L.check(lib.mmf_bitlinear_mfma_clock_sink(clocks.data_ptr(), wgs), "mmf_bitlinear_mfma_clock_sink")
+    try:
+        F_.bitlinear_mfma(q, deq, qsum, pw, m, torch.bfloat16, out=out)
+        torch.cuda.synchronize()
+    finally:
+        F_.L.check(lib.mmf_bitlinear_mfma_clock_sink(None, 0), "mmf_bitlinear_mfma_clock_sink")
+    c = clocks.double().cpu()
+    ghz = float((c[:, 0] / c[:, 1].clamp(min=1)).median()) * 0.1
+    # a SIMD holds 2 waves of a workgroup, each issuing (k / 32) steps of 4 MFMAs of 32 pipe cycles per tile; two
+    # workgroups share a CU when the launch has more than 256 of them
+    busy = (k // 32) * 4 * 32 * 2 * (2 if wgs > 256 else 1) / float(c[:, 0].median())
     return {"shape": [m, k, n], "contract_ms": round(ms_mm, 4), "quant_prologue_ms": round(ms_q, 4),
-            "int8_TOPs": round(tops, 1), "frac_of_5POPs": round(tops / INT8_PEAK_TOPS, 4)}
+            "int8_TOPs": round(tops, 1), "frac_of_5POPs": round(tops / INT8_PEAK_TOPS, 4),
+            "shader_clock_GHz_in_kernel": round(ghz, 3), "workgroup_cycles_median": int(c[:, 0].median()),
+            "matrix_pipe_busy_frac": round(busy, 3)}
+
+
+def mfma_pipe_bench(dev, steps=512, per_cu=2):
+    """The matrix pipe alone: the tiled kernel's four independent MFMAs per step on register operands, nothing else."""
+    import matmulfreellm_amd.functional as F_
+    lib, wgs = F_.L.load(), 256 * per_cu
+    clocks = torch.zeros(2 * wgs + 1, dtype=torch.int64, device=dev)
+    run = lambda: F_.L.check(lib.mmf_mfma_pipe_probe(steps, wgs, clocks.data_ptr(), F_.L.stream()), "mmf_mfma_pipe_probe")
+    ms = timed(run, 10)
+    c = clocks[:2 * wgs].view(wgs, 2).double().cpu()
+    ghz = float((c[:, 0] / c[:, 1].clamp(min=1)).median()) * 0.1
+    tops = wgs * 8 * steps * 4 * 65536.0 / (ms * 1e-3) / 1e12
+    # a SIMD holds per_cu * 2 waves, each with steps * 4 MFMAs of 32 pipe cycles, against the launch's cycles at that clock
+    busy = steps * 4 * 32 * per_cu * 2 / (ms * 1e-3 * ghz * 1e9)
+    return {"workgroups": wgs, "steps": steps, "ms": round(ms, 4), "int8_TOPs": round(tops, 1),
+            "frac_of_5POPs": round(tops / INT8_PEAK_TOPS, 4), "shader_clock_GHz_in_kernel": round(ghz, 3),
+            "matrix_pipe_busy_frac": round(busy, 3)}
 
 
 def _rotating(make_set, set_bytes, min_total=512 << 20, min_sets=3):
@@ -489,6 +522,7 @@ def main():
         if "mfma" in only:
             res["bitlinear_mfma_gate_proj"] = mfma_bench(dev, 4096, 2048, 11264)
             res["bitlinear_mfma_down_proj"] = mfma_bench(dev, 4096, 5632, 2048)
+            res["matrix_pipe_alone"] = mfma_pipe_bench(dev)
         if "scan" in only:
             res["hgrn_scan"] = scan_bench(dev)
         if "norms" in only:
@@ -541,6 +575,7 @@ def main():
     if want("mfma"):
         extra["bitlinear_mfma_gate_proj"] = mfma_bench(dev, 4096, 2048, 11264)
         extra["bitlinear_mfma_down_proj"] = mfma_bench(dev, 4096, 5632, 2048)
+        extra["matrix_pipe_alone"] = mfma_pipe_bench(dev)
     if want("scan"):
         extra["hgrn_scan"] = scan_bench(dev)
     if want("norms"):

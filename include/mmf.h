@@ -168,6 +168,18 @@ int mmf_bitlinear_mfma_swiglu(const int8_t* codes_tiled, const float* deq, const
                               const float* wdeq, int64_t seg_rows, void* out, int64_t ldo, int64_t M, int64_t K, int64_t N,
                               int out_dtype, void* stream);
 
+/* Measuring aids of the tiled contraction (no counterpart in the reference; bench.py's mfma leg uses them).
+ * mmf_bitlinear_mfma_clock_sink: sink = [workgroups][2] int64 on the device, or NULL to switch off.  While set, thread 0
+ *   of each of the first `workgroups` workgroups of every later tiled launch (mmf_bitlinear_mfma with M > 64,
+ *   mmf_bitlinear_mfma_swiglu) stores the shader-clock ticks (s_memtime) and the 100 MHz ticks (s_memrealtime) it
+ *   spent in the kernel: their ratio is the clock the part sustained under that kernel.  Process-wide, not
+ *   thread-safe; the buffer must outlive the launches.
+ * mmf_mfma_pipe_probe: `workgroups` x 8 waves each issue steps x 4 independent v_mfma_i32_32x32x32_i8 on register
+ *   operands (the tiled kernel's inner step with every load, barrier and LDS read taken away) and store the same two
+ *   tick counts; clocks = [workgroups][2] int64 plus one spare int64. */
+int mmf_bitlinear_mfma_clock_sink(int64_t* sink, int64_t workgroups);
+int mmf_mfma_pipe_probe(int64_t steps, int64_t workgroups, int64_t* clocks, void* stream);
+
 /* ---- HGRN recurrence ------------------------------------------------------------------
  * x, g, o: [BH, T, D] contiguous (BH = batch * heads); h0 / ht: [BH, D] fp32 or NULL.
  * mmf_hgrn_recurrent replaces fused_recurrent_hgrn, mmfreelm/ops/hgrn/recurrent_fuse.py:

@@ -43,7 +43,13 @@ struct MfmaArgs {
     int64_t M, N, Kp, seg_rows, ldo;
     int tiles_m, tiles_n;
     int vec_store;        // outputs can be written as aligned 16-byte vectors
+    long long* clocks;    // null, or [clock_cap][2]: shader-clock and 100 MHz ticks a workgroup spent in the kernel
+    int64_t clock_cap;
 };
+
+// Where the tiled kernel notes its clocks (mmf_bitlinear_mfma_clock_sink); null: nothing is noted.
+long long* g_clock_sink = nullptr;
+int64_t g_clock_cap = 0;
 
 // Pack rounded outputs: two floats -> one dword of bf16/f16 (round to nearest even).
 template <typename T>
@@ -420,6 +426,8 @@ void bitlinear_mfma_dma3_kernel(MfmaArgs p) {
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
+    long long clk0 = 0, wall0 = 0;
+    if (p.clocks) { clk0 = __builtin_amdgcn_s_memtime(); wall0 = __builtin_amdgcn_s_memrealtime(); }
     // Workgroup ids are dealt round-robin to the 8 XCDs.  When the tile rows divide by 8, XCD x owns rows
     // [x*R, (x+1)*R) and walks the columns with the rows running fastest: the R workgroups that share a weight
     // tile run together, and the R activation panels stay in that XCD's L2 for the whole walk.
@@ -544,12 +552,17 @@ void bitlinear_mfma_dma3_kernel(MfmaArgs p) {
     if constexpr (SWI) mfma_epilogue_swiglu<T, WM>(p, acc, sc, smem, lane, wave, wm, mb0, nb0);
     else if constexpr (FAST) mfma_epilogue_fast<T, WM, WN>(p, acc, sc, smem, lane, wave, wm, mb0, nb0);
     else mfma_epilogue<T, WM, WN>(p, acc, sc, smem, lane, wave, wm, mb0, nb0);
+    if (p.clocks && threadIdx.x == 0 && (int64_t)blockIdx.x < p.clock_cap) {
+        p.clocks[2 * blockIdx.x] = __builtin_amdgcn_s_memtime() - clk0;
+        p.clocks[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - wall0;
+    }
 }
 
 // The 64 x 512 tile on the stacked [gate; up] weight with the swiglu epilogue: a tile is 64 rows x 256 channels.
 template <typename T>
 int launch_mfma_dma3_swiglu(MfmaArgs a, hipStream_t s) {
     constexpr int WGM = 1, WGN = 8, WM = 2, WN = 2;
+    a.clocks = g_clock_sink; a.clock_cap = g_clock_cap;
     a.tiles_m = (int)mmf_ceil_div(a.M, WGM * WM * 32);
     a.tiles_n = (int)mmf_ceil_div(a.N / 2, WGN * 32);
     size_t lds = 3u * (WGM * WM) * 4096u;
@@ -570,6 +583,7 @@ int launch_mfma_dma3_swiglu(MfmaArgs a, hipStream_t s) {
 template <typename T, int WGM, int WGN, int WM, int WN>
 int launch_mfma_dma3(MfmaArgs a, hipStream_t s) {
     constexpr int BM = WGM * WM * 32, BN = WGN * WN * 32;
+    a.clocks = g_clock_sink; a.clock_cap = g_clock_cap;
     a.tiles_m = (int)mmf_ceil_div(a.M, BM);
     a.tiles_n = (int)mmf_ceil_div(a.N, BN);
     size_t lds = 3u * (WGM * WM) * 4096u;
@@ -756,9 +770,54 @@ int dispatch_mfma(const MfmaArgs& a, int config, hipStream_t s) {
     return MMF_ERR_ARG;
 }
 
+// The matrix pipe with nothing else to do: every wave issues the tiled kernel's four independent 32x32x32 int8 MFMAs per
+// step on operands that never leave its registers (8 waves per workgroup, 4 waves per SIMD with two workgroups per CU).
+__global__ __launch_bounds__(512, 4) void mfma_pipe_probe_kernel(int64_t steps, long long* clocks, int* sink) {
+    const long long clk0 = __builtin_amdgcn_s_memtime(), wall0 = __builtin_amdgcn_s_memrealtime();
+    v4i a, b;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { a[i] = 0x01010101 * (int)(threadIdx.x & 1); b[i] = 0x01010101; }
+    v16i acc[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[t][r] = 0;
+    for (int64_t s = 0; s < steps; ++s) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, a, acc[t], 0, 0, 0);
+    }
+    int x = 0;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x ^= acc[t][r];
+    if (x == 0x7fffffff) *sink = x;                              // keeps the accumulators live; never true
+    if (threadIdx.x == 0) {
+        clocks[2 * blockIdx.x] = __builtin_amdgcn_s_memtime() - clk0;
+        clocks[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - wall0;
+    }
+}
+
 }  // namespace
 
 extern "C" {
+
+int mmf_bitlinear_mfma_clock_sink(int64_t* sink, int64_t workgroups) {
+    if (workgroups < 0 || (sink && workgroups == 0)) return MMF_ERR_ARG;
+    g_clock_sink = reinterpret_cast<long long*>(sink);
+    g_clock_cap = sink ? workgroups : 0;
+    return 0;
+}
+
+int mmf_mfma_pipe_probe(int64_t steps, int64_t workgroups, int64_t* clocks, void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (steps < 0 || workgroups <= 0 || workgroups > 65535 || !clocks) return MMF_ERR_ARG;
+    // the word after the clocks is the sink of the never-taken store
+    mfma_pipe_probe_kernel<<<(unsigned)workgroups, 512, 0, stream>>>(steps, reinterpret_cast<long long*>(clocks),
+                                                                    reinterpret_cast<int*>(clocks + 2 * workgroups));
+    MMF_CHECK_LAUNCH();
+    return 0;
+}
 
 int mmf_bitlinear_mfma(const int8_t* codes_tiled, const float* deq, const int* qsum, const void* packed,
                        const float* wdeq, int64_t seg_rows, const void* bias, const void* addend, void* out, int64_t ldo,
