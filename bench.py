@@ -215,12 +215,14 @@ def mfma_bench(dev, m=4096, k=2048, n=11264, iters=20):
             "matrix_pipe_busy_frac": round(busy, 3)}
 
 
-def mfma_pipe_bench(dev, steps=512, per_cu=2):
-    """The matrix pipe alone: the tiled kernel's four independent MFMAs per step on register operands, nothing else."""
+def mfma_pipe_bench(dev, random_operands, steps=512, per_cu=2):
+    """The matrix pipe alone: the tiled kernel's four independent MFMAs per step on register operands, nothing else.
+    With constant operands the pipe switches little and draws little power; random int8 codes and ternary weights
+    are what a contraction feeds it."""
     import matmulfreellm_amd.functional as F_
     lib, wgs = F_.L.load(), 256 * per_cu
     clocks = torch.zeros(2 * wgs + 1, dtype=torch.int64, device=dev)
-    run = lambda: F_.L.check(lib.mmf_mfma_pipe_probe(steps, wgs, clocks.data_ptr(), F_.L.stream()), "mmf_mfma_pipe_probe")
+    run = lambda: F_.L.check(lib.mmf_mfma_pipe_probe(steps, wgs, int(random_operands), clocks.data_ptr(), F_.L.stream()), "mmf_mfma_pipe_probe")
     ms = timed(run, 10)
     c = clocks[:2 * wgs].view(wgs, 2).double().cpu()
     ghz = float((c[:, 0] / c[:, 1].clamp(min=1)).median()) * 0.1
@@ -522,7 +524,8 @@ def main():
         if "mfma" in only:
             res["bitlinear_mfma_gate_proj"] = mfma_bench(dev, 4096, 2048, 11264)
             res["bitlinear_mfma_down_proj"] = mfma_bench(dev, 4096, 5632, 2048)
-            res["matrix_pipe_alone"] = mfma_pipe_bench(dev)
+            res["matrix_pipe_alone_random_operands"] = mfma_pipe_bench(dev, True)
+            res["matrix_pipe_alone_constant_operands"] = mfma_pipe_bench(dev, False)
         if "scan" in only:
             res["hgrn_scan"] = scan_bench(dev)
         if "norms" in only:
@@ -575,7 +578,8 @@ def main():
     if want("mfma"):
         extra["bitlinear_mfma_gate_proj"] = mfma_bench(dev, 4096, 2048, 11264)
         extra["bitlinear_mfma_down_proj"] = mfma_bench(dev, 4096, 5632, 2048)
-        extra["matrix_pipe_alone"] = mfma_pipe_bench(dev)
+        extra["matrix_pipe_alone_random_operands"] = mfma_pipe_bench(dev, True)
+        extra["matrix_pipe_alone_constant_operands"] = mfma_pipe_bench(dev, False)
     if want("scan"):
         extra["hgrn_scan"] = scan_bench(dev)
     if want("norms"):

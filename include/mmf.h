@@ -176,9 +176,10 @@ int mmf_bitlinear_mfma_swiglu(const int8_t* codes_tiled, const float* deq, const
  *   thread-safe; the buffer must outlive the launches.
  * mmf_mfma_pipe_probe: `workgroups` x 8 waves each issue steps x 4 independent v_mfma_i32_32x32x32_i8 on register
  *   operands (the tiled kernel's inner step with every load, barrier and LDS read taken away) and store the same two
- *   tick counts; clocks = [workgroups][2] int64 plus one spare int64. */
+ *   tick counts; clocks = [workgroups][2] int64 plus one spare int64.  random_operands != 0: per-lane random int8 codes
+ *   and ternary weights (the switching activity, hence the power draw, of real operands) instead of constant ones. */
 int mmf_bitlinear_mfma_clock_sink(int64_t* sink, int64_t workgroups);
-int mmf_mfma_pipe_probe(int64_t steps, int64_t workgroups, int64_t* clocks, void* stream);
+int mmf_mfma_pipe_probe(int64_t steps, int64_t workgroups, int random_operands, int64_t* clocks, void* stream);
 
 /* ---- HGRN recurrence ------------------------------------------------------------------
  * x, g, o: [BH, T, D] contiguous (BH = batch * heads); h0 / ht: [BH, D] fp32 or NULL.

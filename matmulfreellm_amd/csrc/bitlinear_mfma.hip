@@ -772,11 +772,19 @@ int dispatch_mfma(const MfmaArgs& a, int config, hipStream_t s) {
 
 // The matrix pipe with nothing else to do: every wave issues the tiled kernel's four independent 32x32x32 int8 MFMAs per
 // step on operands that never leave its registers (8 waves per workgroup, 4 waves per SIMD with two workgroups per CU).
-__global__ __launch_bounds__(512, 4) void mfma_pipe_probe_kernel(int64_t steps, long long* clocks, int* sink) {
+// random_operands: int8 codes and ternary weights drawn per lane (the switching activity of real operands) instead of the
+// constant 1s, on which the pipe draws far less power.
+__global__ __launch_bounds__(512, 4) void mfma_pipe_probe_kernel(int64_t steps, int random_operands, long long* clocks, int* sink) {
     const long long clk0 = __builtin_amdgcn_s_memtime(), wall0 = __builtin_amdgcn_s_memrealtime();
-    v4i a, b;
+    auto mix = [](uint32_t x) { x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16; return x; };
+    v4i a[2], b[2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) { a[i] = 0x01010101 * (int)(threadIdx.x & 1); b[i] = 0x01010101; }
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            a[h][i] = random_operands ? (int)mix(threadIdx.x * 16 + h * 4 + i) : 0x01010101 * (int)(threadIdx.x & 1);
+            b[h][i] = random_operands ? (int)(mix(threadIdx.x * 16 + 8 + h * 4 + i) & 0x03030303u) : 0x01010101;
+        }
     v16i acc[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
@@ -784,7 +792,7 @@ __global__ __launch_bounds__(512, 4) void mfma_pipe_probe_kernel(int64_t steps, 
         for (int r = 0; r < 16; ++r) acc[t][r] = 0;
     for (int64_t s = 0; s < steps; ++s) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, a, acc[t], 0, 0, 0);
+        for (int t = 0; t < 4; ++t) acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[t & 1], a[t >> 1], acc[t], 0, 0, 0);
     }
     int x = 0;
 #pragma unroll
@@ -809,11 +817,11 @@ int mmf_bitlinear_mfma_clock_sink(int64_t* sink, int64_t workgroups) {
     return 0;
 }
 
-int mmf_mfma_pipe_probe(int64_t steps, int64_t workgroups, int64_t* clocks, void* stream_) {
+int mmf_mfma_pipe_probe(int64_t steps, int64_t workgroups, int random_operands, int64_t* clocks, void* stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (steps < 0 || workgroups <= 0 || workgroups > 65535 || !clocks) return MMF_ERR_ARG;
     // the word after the clocks is the sink of the never-taken store
-    mfma_pipe_probe_kernel<<<(unsigned)workgroups, 512, 0, stream>>>(steps, reinterpret_cast<long long*>(clocks),
+    mfma_pipe_probe_kernel<<<(unsigned)workgroups, 512, 0, stream>>>(steps, random_operands, reinterpret_cast<long long*>(clocks),
                                                                     reinterpret_cast<int*>(clocks + 2 * workgroups));
     MMF_CHECK_LAUNCH();
     return 0;
