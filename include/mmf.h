@@ -101,6 +101,12 @@ int64_t mmf_codes_bytes(int64_t M, int64_t K, int tiled);
 int mmf_rmsnorm_quant(const void* x, const void* residual, const void* weight, int8_t* q, float* deq,
                       int* qsum, void* residual_out, int64_t M, int64_t K, float eps, int x_dtype,
                       int residual_dtype, int weight_dtype, int tiled, void* stream);
+/* mmf_layernorm_quant: the IS_RMS_NORM = False branch of the same reference kernel (fusedbitnet.py:102-121, reached
+ * through layer_norm_linear_quant_fn(..., is_rms_norm=False), :513-536): mean = fp32(sum x / K), the variance is that of
+ * the fp32 differences x - mean, y = (x - mean) * rstd * weight + bias.  bias: [K] in the weight's dtype, or NULL. */
+int mmf_layernorm_quant(const void* x, const void* residual, const void* weight, const void* bias, int8_t* q,
+                        float* deq, int* qsum, void* residual_out, int64_t M, int64_t K, float eps, int x_dtype,
+                        int residual_dtype, int weight_dtype, int tiled, void* stream);
 
 /* mmf_rmsnorm_quant_fused: the same quantiser (tiled codes) with the elementwise op that precedes a
  * BitLinear in the model folded in, for batches that go to the matrix cores:

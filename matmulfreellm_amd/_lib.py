@@ -32,6 +32,7 @@ SIGNATURES = {
     "mmf_swiglu": (_i32, [_ptr, _i64, _ptr, _i64, _ptr, _i64, _i64, _i32, _ptr]),
     "mmf_codes_bytes": (_i64, [_i64, _i64, _i32]),
     "mmf_rmsnorm_quant": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _f32, _i32, _i32, _i32, _i32, _ptr]),
+    "mmf_layernorm_quant": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _f32, _i32, _i32, _i32, _i32, _ptr]),
     "mmf_rmsnorm_quant_fused": (_i32, [_i32, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _f32, _ptr, _f32, _ptr, _ptr, _ptr, _ptr,
                                        _ptr, _i64, _i64, _i32, _i32, _ptr]),
     "mmf_decode_layers_phase_bytes": (_i32, []),

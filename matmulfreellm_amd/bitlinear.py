@@ -49,13 +49,20 @@ def layer_norm_linear_quant_fn(x, norm_weight, norm_bias, linear_weight, linear_
                                prenorm=False, residual_in_fp32=False, is_rms_norm=False, packed=None):
     """Same positional signature as mmfreelm/ops/fusedbitnet.py:513-536.
 
-    Only the RMSNorm form without a norm bias exists on the MatMul-free LM path; anything
-    else raises.  ``packed`` (a functional.PackedWeight) skips the ternarise+pack pass.
+    is_rms_norm=False selects the LayerNorm form (row mean subtracted, optional norm_bias): forward only, the
+    MatMul-free LM never takes it (FusedBitLinear passes is_rms_norm=True, fusedbitnet.py:602-610).  A norm bias on the
+    RMSNorm form raises.  ``packed`` (a functional.PackedWeight) skips the ternarise+pack pass.
     """
-    if not is_rms_norm or norm_bias is not None:
-        raise NotImplementedError("only is_rms_norm=True with norm_bias=None is implemented "
-                                  "(the only form FusedBitLinear uses, fusedbitnet.py:602-610)")
     from .autograd import BitLinearFn, needs_grad
+    if not is_rms_norm:
+        if needs_grad(x, norm_weight, norm_bias, linear_weight, linear_bias, residual):
+            raise NotImplementedError("the LayerNorm form of layer_norm_linear_quant_fn has no backward here "
+                                      "(call it under torch.no_grad(); the model path is RMSNorm)")
+        pw = packed if packed is not None else F_.ternarize_pack(linear_weight)
+        return F_.bitlinear(x, norm_weight, pw, bias=linear_bias, eps=eps, residual=residual, prenorm=prenorm,
+                            residual_in_fp32=residual_in_fp32, norm_bias=norm_bias, is_rms_norm=False)
+    if norm_bias is not None:
+        raise NotImplementedError("a norm bias exists for the LayerNorm form only (is_rms_norm=False)")
     if needs_grad(x, norm_weight, linear_weight, linear_bias, residual):
         if linear_weight.is_meta:
             raise RuntimeError("this BitLinear holds packed codes only: there is no latent weight to train")

@@ -352,12 +352,15 @@ __device__ __forceinline__ float mmf_block_max_once(float v, float* slot) {
 // inv_K = RN(1 / K) from the host, q0 = sumsq * inv_K is within two ulps, one residual step
 // makes it faithful, and a second one (r exact through the fused multiply-add) lands on the
 // correctly rounded quotient (Markstein's theorem; K is a small integer, 0 <= sumsq < 2^200).
-__device__ __forceinline__ float mmf_rstd(double sumsq, int64_t K, double inv_K, float eps) {
+__device__ __forceinline__ double mmf_quotient_by_count(double sum, int64_t K, double inv_K) {
     const double Kd = (double)K;
-    double q = sumsq * inv_K;
-    q = fma(fma(-q, Kd, sumsq), inv_K, q);
-    q = fma(fma(-q, Kd, sumsq), inv_K, q);
-    const float var = (float)q;
+    double q = sum * inv_K;
+    q = fma(fma(-q, Kd, sum), inv_K, q);
+    q = fma(fma(-q, Kd, sum), inv_K, q);
+    return q;
+}
+__device__ __forceinline__ float mmf_rstd(double sumsq, int64_t K, double inv_K, float eps) {
+    const float var = (float)mmf_quotient_by_count(sumsq, K, inv_K);
     return __fdiv_rn(1.0f, sqrtf(__fadd_rn(var, eps)));   // sqrtf: correctly rounded (__fsqrt_rn is the native approximation)
 }
 

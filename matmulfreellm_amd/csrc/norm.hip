@@ -21,6 +21,8 @@ struct RowArgs {
     const void* residual;   // [M, K] or null            (dtype TR)
     const void* gate;       // [M, K] or null            (ROW_GATE, dtype T)
     const void* weight;     // [K] or null               (dtype TW)
+    const void* bias;       // [K] or null: added after the weight (dtype TW)
+    int center;             // LayerNorm: subtract the row mean before the variance (else RMSNorm)
     void* y;                // [M, K] T                  (ROW_NORM / ROW_GATE)
     void* residual_out;     // [M, K] TR or null
     int8_t* q;              // codes                     (ROW_QUANT)
@@ -80,6 +82,26 @@ __global__ __launch_bounds__(kThreads) void row_kernel(RowArgs a) {
             for (int i = 0; i < 8; ++i) xv[v][i] = 0.0f;
         }
     }
+    if (a.center) {
+        // LayerNorm: mean = fp32(sum / K) with the sum in fp64; the variance is that of the fp32 differences
+        double sx = 0.0;
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sx += (double)xv[v][i];
+        sx = mmf_block_sum<kWaves>(sx, red_d);
+        const float mean = (float)mmf_quotient_by_count(sx, K, a.inv_K);
+        ss = 0.0;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                xv[v][i] = k0 + i < K ? __fsub_rn(xv[v][i], mean) : 0.0f;
+                ss += (double)xv[v][i] * (double)xv[v][i];
+            }
+        }
+    }
     ss = mmf_block_sum<kWaves>(ss, red_d);
     const float rstd = mmf_rstd(ss, K, a.inv_K, a.eps);
 
@@ -88,10 +110,13 @@ __global__ __launch_bounds__(kThreads) void row_kernel(RowArgs a) {
     for (int v = 0; v < NV; ++v) {
         const int64_t k0 = ((int64_t)v * kThreads + threadIdx.x) * 8;
         if (k0 < K) {
+            float bv[8];
+            if (a.bias) mmf_load8<TW>(static_cast<const TW*>(a.bias), k0, K, vec_ok, bv);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 float y = __fmul_rn(xv[v][i], rstd);
                 if (w) y = __fmul_rn(y, wv[v][i]);
+                if (a.bias) y = k0 + i < K ? __fadd_rn(y, bv[i]) : 0.0f;
                 xv[v][i] = y;
                 amax = fmaxf(amax, fabsf(y));
             }
@@ -546,6 +571,22 @@ int mmf_rmsnorm_quant(const void* x, const void* residual, const void* weight, i
         return MMF_ERR_ALIGN;
     RowArgs a{};
     a.x = x; a.residual = residual; a.weight = weight; a.residual_out = residual_out;
+    a.q = q; a.deq = deq; a.qsum = qsum;
+    a.M = M; a.K = K; a.inv_K = 1.0 / (double)K; a.Kp = mmf_round_up(K, 128); a.ldx = K; a.eps = eps; a.q_tiled = tiled;
+    return dispatch_x<ROW_QUANT>(a, x_dtype, residual_dtype, weight_dtype, stream);
+}
+
+int mmf_layernorm_quant(const void* x, const void* residual, const void* weight, const void* bias, int8_t* q, float* deq,
+                        int* qsum, void* residual_out, int64_t M, int64_t K, float eps, int x_dtype, int residual_dtype,
+                        int weight_dtype, int tiled, void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (M < 0 || K <= 0 || (M > 0 && (!x || !q || !deq || !qsum))) return MMF_ERR_ARG;
+    if (bias && !weight) return MMF_ERR_ARG;                     // the bias shares the weight's dtype
+    if (!aligned16(q)) return MMF_ERR_ALIGN;
+    if (K % 8 == 0 && !(aligned16(x) && aligned16(residual) && aligned16(residual_out) && aligned16(weight) && aligned16(bias)))
+        return MMF_ERR_ALIGN;
+    RowArgs a{};
+    a.x = x; a.residual = residual; a.weight = weight; a.bias = bias; a.center = 1; a.residual_out = residual_out;
     a.q = q; a.deq = deq; a.qsum = qsum;
     a.M = M; a.K = K; a.inv_K = 1.0 / (double)K; a.Kp = mmf_round_up(K, 128); a.ldx = K; a.eps = eps; a.q_tiled = tiled;
     return dispatch_x<ROW_QUANT>(a, x_dtype, residual_dtype, weight_dtype, stream);

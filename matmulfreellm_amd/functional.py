@@ -158,13 +158,19 @@ def swiglu(x, y):
     return out
 
 
-def rmsnorm_quant(x, weight, residual=None, eps=1e-8, tiled=False, prenorm=False, residual_in_fp32=False):
+def rmsnorm_quant(x, weight, residual=None, eps=1e-8, tiled=False, prenorm=False, residual_in_fp32=False,
+                  norm_bias=None, is_rms_norm=True):
     """RMSNorm + per-row absmax int8 codes.  Returns (q uint8-storage int8 tensor, deq, qsum[, residual_out]).
 
     q is [M, Kp] (row-major) or the flat tiled buffer when tiled=True; Kp = ceil128(K).
+    is_rms_norm=False: LayerNorm (row mean subtracted first) with an optional norm_bias in the weight's dtype.
     """
     lib = L.load()
     dev, shp, x2, r2, res_dtype, res_out, w = _norm_common(x, residual, weight, prenorm, residual_in_fp32)
+    if not is_rms_norm:
+        return _layernorm_quant(lib, dev, shp, x, x2, r2, res_dtype, res_out, w, norm_bias, eps, tiled, prenorm)
+    if norm_bias is not None:
+        raise ValueError("norm_bias needs is_rms_norm=False (the RMSNorm of the BitLinear path has no bias)")
     m, k = x2.shape
     kp = -(-k // 128) * 128
     nbytes = lib.mmf_codes_bytes(m, k, 1 if tiled else 0)
@@ -178,6 +184,30 @@ def rmsnorm_quant(x, weight, residual=None, eps=1e-8, tiled=False, prenorm=False
                 "mmf_rmsnorm_quant")
     if not tiled:
         q = q.view(m, kp)
+    if prenorm:
+        return q, deq, qsum, (res_out.reshape(shp) if res_out is not None else x)
+    return q, deq, qsum
+
+
+def _layernorm_quant(lib, dev, shp, x, x2, r2, res_dtype, res_out, w, bias, eps, tiled, prenorm):
+    m, k = x2.shape
+    if bias is not None:
+        if w is None:
+            raise ValueError("a norm bias needs a norm weight (they share a dtype)")
+        L.require_gpu(bias)
+        bias = bias.detach().to(w.dtype).contiguous()
+        if bias.shape != (k,):
+            raise ValueError(f"norm bias has shape {tuple(bias.shape)}, expected ({k},)")
+    q = torch.empty(lib.mmf_codes_bytes(m, k, 1 if tiled else 0), dtype=torch.int8, device=dev)
+    deq = torch.empty(m, dtype=torch.float32, device=dev)
+    qsum = torch.empty(m, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        L.check(lib.mmf_layernorm_quant(x2.data_ptr(), L.ptr(r2), L.ptr(w), L.ptr(bias), q.data_ptr(), deq.data_ptr(),
+                                        qsum.data_ptr(), L.ptr(res_out), m, k, eps, L.dtype_id(x2.dtype),
+                                        L.dtype_id(res_dtype), L.dtype_id(w.dtype) if w is not None else 0,
+                                        1 if tiled else 0, L.stream()), "mmf_layernorm_quant")
+    if not tiled:
+        q = q.view(m, -(-k // 128) * 128)
     if prenorm:
         return q, deq, qsum, (res_out.reshape(shp) if res_out is not None else x)
     return q, deq, qsum
@@ -326,8 +356,11 @@ def _check_swiglu_epilogue(epilogue, m, pw, dtype, bias, addend):
 
 
 def bitlinear(x, norm_weight, pw, bias=None, eps=1e-8, residual=None, prenorm=False, residual_in_fp32=False,
-              path=None, addend=None, prologue=None, epilogue=None):
+              path=None, addend=None, prologue=None, epilogue=None, norm_bias=None, is_rms_norm=True):
     """Fused BitLinear forward on x [..., K] -> [..., N] (x.dtype).
+
+    is_rms_norm=False (with an optional norm_bias): the LayerNorm form; it always takes the quantiser + contraction
+    pair of launches.
 
     path: None (by M), "gemv" or "mfma".  With a residual (or prenorm) the two-launch path is used.
     prologue: see _bitlinear_prologue (the elementwise op that produces this BitLinear's input, fused).
@@ -335,8 +368,8 @@ def bitlinear(x, norm_weight, pw, bias=None, eps=1e-8, residual=None, prenorm=Fa
     epilogue (large M only: swiglu_epilogue_fits).
     """
     if prologue is not None:
-        if residual is not None or prenorm or path is not None:
-            raise ValueError("prologue= excludes residual=, prenorm= and path=")
+        if residual is not None or prenorm or path is not None or not is_rms_norm:
+            raise ValueError("prologue= excludes residual=, prenorm=, path= and the LayerNorm form")
         return _bitlinear_prologue(x, norm_weight, pw, bias, eps, addend, prologue, epilogue)
     lib = L.load()
     L.require_gpu(x)
@@ -346,7 +379,9 @@ def bitlinear(x, norm_weight, pw, bias=None, eps=1e-8, residual=None, prenorm=Fa
         raise ValueError(f"input features {k} != weight in_features {pw.k}")
     x2 = _as_2d(x)
     m = x2.shape[0]
-    plain = residual is None and not prenorm
+    plain = residual is None and not prenorm and is_rms_norm
+    if not is_rms_norm and path == "gemv":
+        raise ValueError("the fused GEMV launch has the RMSNorm form only")
     if path is None:
         path = "gemv" if (plain and m <= GEMV_MAX_M and k <= lib.mmf_bitlinear_gemv_max_k()) else "mfma"
     if path == "gemv":
@@ -355,7 +390,7 @@ def bitlinear(x, norm_weight, pw, bias=None, eps=1e-8, residual=None, prenorm=Fa
         out = bitlinear_gemv(x2, norm_weight, pw, eps, bias, addend)
         return out.reshape(*shp[:-1], pw.n)
     res = rmsnorm_quant(x, norm_weight, residual=residual, eps=eps, tiled=True, prenorm=prenorm,
-                        residual_in_fp32=residual_in_fp32)
+                        residual_in_fp32=residual_in_fp32, norm_bias=norm_bias, is_rms_norm=is_rms_norm)
     q, deq, qsum = res[:3]
     if epilogue is not None:
         _check_swiglu_epilogue(epilogue, m, pw, x.dtype, bias, addend)

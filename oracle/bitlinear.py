@@ -2,7 +2,7 @@
 import torch
 import torch.nn.functional as F
 
-from .norms import rms_norm_literal, rms_norm_quant_spec
+from .norms import layer_norm_quant_spec, rms_norm_literal, rms_norm_quant_spec
 from .quant import activation_quant_literal, ternary_codes, weight_quant_literal
 
 _F = torch.float32
@@ -44,12 +44,16 @@ def contract_exact(q, deq, t, wdeq, out_dtype, bias=None):
     return out.to(out_dtype), acc.to(torch.int32)
 
 
-def bitlinear_spec(x, weight, norm_weight, bias=None, eps=1e-8, residual=None):
-    """Integer-exact BitLinear on x [..., K], weight [N, K] -> [..., N] in x.dtype."""
+def bitlinear_spec(x, weight, norm_weight, bias=None, eps=1e-8, residual=None, norm_bias=None, is_rms_norm=True):
+    """Integer-exact BitLinear on x [..., K], weight [N, K] -> [..., N] in x.dtype (is_rms_norm=False: the LayerNorm
+    form of mmfreelm/ops/fusedbitnet.py:513-536)."""
     shp = x.shape
     x2 = x.reshape(-1, shp[-1])
     r2 = residual.reshape(-1, shp[-1]) if residual is not None else None
-    q, deq, _, _ = rms_norm_quant_spec(x2, norm_weight, residual=r2, eps=eps)
+    if is_rms_norm:
+        q, deq, _, _ = rms_norm_quant_spec(x2, norm_weight, residual=r2, eps=eps)
+    else:
+        q, deq, _, _ = layer_norm_quant_spec(x2, norm_weight, norm_bias, residual=r2, eps=eps)
     t, wdeq = ternary_codes(weight)
     out, _ = contract_exact(q, deq, t, wdeq, x.dtype, bias)
     return out.reshape(*shp[:-1], weight.shape[0])

@@ -108,3 +108,37 @@ def rms_norm_quant_spec(x, weight, residual=None, eps=1e-8):
         y = y * weight.to(_F)
     q, deq, qsum = activation_codes(y)
     return q, deq, qsum, xf
+
+
+def layer_norm_quant_literal(x, weight, bias=None, residual=None, eps=1e-8):
+    """mmfreelm/ops/fusedbitnet.py:95-128 with IS_RMS_NORM false, as written there (fp32, torch reductions):
+    mean, variance of x - mean, (x - mean) * rstd * w + b, then the fake quantiser; returns the de-quantised y."""
+    xf = _sum_with_residual(x, residual)
+    mean = xf.sum(dim=-1, keepdim=True) / xf.shape[-1]
+    xbar = xf - mean
+    var = (xbar * xbar).sum(dim=-1, keepdim=True) / xf.shape[-1]
+    rstd = 1 / torch.sqrt(var + eps)
+    y = xbar * rstd
+    if weight is not None:
+        y = y * weight.to(_F)
+    if bias is not None:
+        y = y + bias.to(_F)
+    scale = 127.0 / y.abs().amax(dim=-1, keepdim=True).clamp(min=1e-5)
+    return (y * scale).round().clamp(-128, 127) / scale
+
+
+def layer_norm_quant_spec(x, weight, bias=None, residual=None, eps=1e-8):
+    """The same branch in the device's arithmetic: sum of x in fp64 -> mean in fp32; differences in fp32; their
+    squares and sum in fp64; codes as rms_norm_quant_spec.  Returns (q, deq, qsum, xsum)."""
+    xf = _sum_with_residual(x, residual)
+    k = xf.shape[-1]
+    mean = (xf.to(torch.float64).sum(dim=-1, keepdim=True) / k).to(_F)
+    xbar = xf - mean
+    rstd = _rstd(xbar, eps)
+    y = xbar * rstd
+    if weight is not None:
+        y = y * weight.to(_F)
+    if bias is not None:
+        y = y + bias.to(_F)
+    q, deq, qsum = activation_codes(y)
+    return q, deq, qsum, xf

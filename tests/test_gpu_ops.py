@@ -171,6 +171,51 @@ def test_rmsnorm_quant_ties_and_zero_rows(dev):
         assert q[2].abs().sum().item() == 0
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("mk", [(3, 100), (64, 2048), (33, 5632), (130, 1536)])
+@pytest.mark.parametrize("bias,residual", [(False, False), (True, False), (True, True)])
+def test_layernorm_quant_codes(dev, dtype, mk, bias, residual):
+    """The IS_RMS_NORM = False branch (fusedbitnet.py:102-121): codes, scales and code sums bit for bit."""
+    torch.manual_seed(16)
+    m, k = mk
+    x = (torch.randn(m, k) * 2 + 0.7).to(dtype)
+    w = (1 + 0.1 * torch.randn(k)).to(dtype)
+    b = (0.2 * torch.randn(k)).to(dtype) if bias else None
+    r = torch.randn(m, k).to(dtype) if residual else None
+    q_ref, deq_ref, qsum_ref, xs_ref = on.layer_norm_quant_spec(x, w, b, residual=r, eps=1e-8)
+    got = F().rmsnorm_quant(x.to(dev), w.to(dev), residual=r.to(dev) if residual else None, eps=1e-8, prenorm=residual,
+                            norm_bias=b.to(dev) if bias else None, is_rms_norm=False)
+    q, deq, qsum = got[:3]
+    assert q[:, k:].abs().sum().item() == 0, "padding columns must be zero"
+    nbad = (q[:, :k].cpu() != q_ref).sum().item()
+    assert nbad == 0, f"{nbad} of {q_ref.numel()} int8 codes differ"
+    assert torch.equal(deq.cpu(), deq_ref) and torch.equal(qsum.cpu(), qsum_ref)
+    if residual:
+        assert torch.equal(got[3].cpu(), xs_ref.to(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m", [2, 200])
+def test_layer_norm_linear_quant_fn_layernorm_form(dev, dtype, m):
+    """layer_norm_linear_quant_fn(..., is_rms_norm=False) with a norm bias (fusedbitnet.py:513-536) against the oracle,
+    bit for bit; it has no backward here and says so; a norm bias on the RMSNorm form is refused."""
+    import matmulfreellm_amd as mm
+    from matmulfreellm_amd.bitlinear import layer_norm_linear_quant_fn
+    torch.manual_seed(17)
+    k, n = 512, 192
+    x = (torch.randn(m, k) + 0.5).to(dtype)
+    w = (torch.randn(n, k) * 0.02).to(dtype)
+    nw, nb = (1 + 0.1 * torch.randn(k)).to(dtype), (0.1 * torch.randn(k)).to(dtype)
+    lb = (0.1 * torch.randn(n)).to(dtype)
+    ref = ob.bitlinear_spec(x, w, nw, bias=lb, eps=1e-6, norm_bias=nb, is_rms_norm=False)
+    out = layer_norm_linear_quant_fn(x.to(dev), nw.to(dev), nb.to(dev), w.to(dev), lb.to(dev), eps=1e-6, is_rms_norm=False)
+    assert assert_same(out, ref, tol_of(dtype), f"LayerNorm-form BitLinear {dtype} M={m}") == 0
+    with pytest.raises(NotImplementedError):
+        layer_norm_linear_quant_fn(x.to(dev).requires_grad_(), nw.to(dev), nb.to(dev), w.to(dev), None, is_rms_norm=False)
+    with pytest.raises(NotImplementedError):
+        layer_norm_linear_quant_fn(x.to(dev), nw.to(dev), nb.to(dev), w.to(dev), None, is_rms_norm=True)
+
+
 # ------------------------------------------------------------------ BitLinear
 def _bitlinear_case(dev, dtype, m, k, n, path, bias=False, seed=7):
     torch.manual_seed(seed)

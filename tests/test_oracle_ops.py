@@ -114,6 +114,46 @@ def test_contraction_on_fp32_codes_is_the_exact_accumulator():
 
 
 # ---------------------------------------------------------------- scans
+def test_layernorm_form_of_the_quantiser_against_the_library_layer_norm():
+    """mmfreelm/ops/fusedbitnet.py:102-121 (IS_RMS_NORM false): the normalised row is torch's own layer_norm (a library
+    routine that shares no code with the oracle), the codes are round(y * 127 / max|y|); rows of zero mean without a
+    bias reduce to the RMSNorm form bit for bit; the device-arithmetic form gives the same codes up to rounding ties."""
+    torch.manual_seed(21)
+    m, k = 9, 300
+    x = torch.randn(m, k) * 3 + 1.5                      # a mean far from zero: dropping the centring cannot pass
+    w, b = 1 + 0.2 * torch.randn(k), 0.3 * torch.randn(k)
+    res = torch.randn(m, k)
+    for bias, residual in ((None, None), (b, None), (b, res)):
+        xs = x if residual is None else x + residual
+        y = F.layer_norm(xs.double(), (k,), w.double(), None if bias is None else bias.double(), 1e-8)
+        scale = 127.0 / y.abs().amax(dim=-1, keepdim=True)
+        want_codes = (y * scale).round().clamp(-128, 127)
+        got = on.layer_norm_quant_literal(x, w, bias, residual=residual, eps=1e-8)
+        lit_codes = (got.double() * scale).round()
+        assert (lit_codes - want_codes).abs().max().item() <= 1 and (lit_codes != want_codes).float().mean().item() < 0.01
+        q, deq, qsum, xsum = on.layer_norm_quant_spec(x, w, bias, residual=residual, eps=1e-8)
+        assert (q.double() - want_codes).abs().max().item() <= 1 and (q.double() != want_codes).float().mean().item() < 0.01
+        assert torch.equal(qsum, q.to(torch.int32).sum(dim=-1)) and torch.equal(xsum, xs)
+        assert rel(deq.reshape(-1, 1), 1.0 / scale.float()) < 1e-6
+    # zero-mean rows (every value beside its negative), no bias: centring changes nothing
+    half = torch.randn(m, k // 2)
+    z = torch.cat([half, -half], dim=-1)
+    qa, da, sa, _ = on.layer_norm_quant_spec(z, w, None, eps=1e-8)
+    qb, db, sb, _ = on.rms_norm_quant_spec(z, w, eps=1e-8)
+    assert torch.equal(qa, qb) and torch.equal(da, db) and torch.equal(sa, sb)
+    # and the contraction behind it
+    wt = torch.randn(24, k) * 0.02
+    out = ob.bitlinear_spec(x, wt, w, eps=1e-8, norm_bias=b, is_rms_norm=False)
+    want = (want_codes_for(x, w, b, k) @ oq.weight_quant_literal(wt).double().t()).float()
+    assert rel(out, want) < 5e-3
+
+
+def want_codes_for(x, w, b, k):
+    y = F.layer_norm(x.double(), (k,), w.double(), b.double(), 1e-8)
+    scale = 127.0 / y.abs().amax(dim=-1, keepdim=True)
+    return (y * scale).round().clamp(-128, 127) / scale
+
+
 def test_scan_closed_forms():
     B, H, T, D = 2, 1, 50, 8
     x = torch.full((B, H, T, D), 0.5)
