@@ -353,8 +353,9 @@ def sampler_bench(model, dev, n_new=256):
     u = torch.rand(1, generator=g, device=dev)
     out = torch.empty(1, dtype=torch.int64, device=dev)
     us = timed(lambda: F_.sample_top_p(lg, 0.4, 0.6, u, out=out), 50) * 1e3
+    us_k = timed(lambda: F_.sample_top_p(lg, 0.4, 0.6, u, out=out, top_k=50), 50) * 1e3
     ids = torch.randint(0, model.config.vocab_size, (1, 128), generator=g, device=dev)
-    res = {"sample_top_p_us_per_row_of_32000": round(us, 2)}
+    res = {"sample_top_p_us_per_row_of_32000": round(us, 2), "with_top_k_50_us": round(us_k, 2)}
     for name, kw in (("greedy", {}), ("top_p", dict(do_sample=True, top_p=0.4, temperature=0.6, generator=g))):
         model.generate(ids, max_new_tokens=8, eos_token_id=None, **kw)
         torch.cuda.synchronize()

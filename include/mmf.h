@@ -294,15 +294,19 @@ int mmf_cross_entropy_train_bwd(const void* logits, int64_t ld, const int64_t* l
  *   cumulative sum, nucleus mask, renormalisation and the multinomial draw -- one launch, no sort.
  *   All decisions are made on integer probability masses, so the result does not depend on a summation order:
  *     l_i = logit_i / temperature (NaN counts as -inf);  p_i = 1 if l_i == max l, else exp(l_i - max l) in fp32;
- *     m_i = trunc(p_i * 2^31);  Z = sum m_i;  P = max(1, trunc(double(top_p) * double(Z)))  (top_p clamped to [0, 1]);
+ *     m_i = trunc(p_i * 2^31);
+ *     top_k > 0: m_i = 0 unless m_i >= the top_k-th largest mass (transformers' TopKLogitsWarper runs before the
+ *       top-p one; the reference's call passes no top_k and so gets the default generation parameters' 50;
+ *       equal masses stay together; top_k = 0 or >= V: no limit);
+ *     Z = sum m_i;  P = max(1, trunc(double(top_p) * double(Z)))  (top_p clamped to [0, 1]);
  *     token i is kept iff m_i > 0 and the mass of all tokens with m_j > m_i is below P;
  *     S = mass of the kept tokens;  target = trunc(double(u[r]) * double(S));
  *     out[r] = lowest index whose running sum of kept masses, in index order, exceeds target.
  *   u: one uniform number in [0, 1) per row, drawn by the caller (fp32, device memory); out: int64 [rows].
- *   temperature <= 0 or NaN: MMF_ERR_ARG;  V > mmf_sample_top_p_max_vocab() (65536): MMF_ERR_WIDE. */
+ *   temperature <= 0 or NaN, top_k < 0: MMF_ERR_ARG;  V > mmf_sample_top_p_max_vocab() (65536): MMF_ERR_WIDE. */
 int64_t mmf_sample_top_p_max_vocab(void);
 int mmf_sample_top_p(const void* logits, int64_t ld, int64_t rows, int64_t V, float temperature, float top_p,
-                     const float* u, int64_t* out, int dtype, void* stream);
+                     int64_t top_k, const float* u, int64_t* out, int dtype, void* stream);
 
 /* ---- all layers of one batch-1 decode step in one persistent launch ---------------------------
  * mmf_decode_layers replaces, for one token, the loop over HGRNBitBlock.forward in HGRNBitModel.forward

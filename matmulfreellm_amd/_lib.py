@@ -65,7 +65,7 @@ SIGNATURES = {
     "mmf_cross_entropy_train_fwd": (_i32, [_ptr, _i64, _ptr, _i64, _f32, _f32, _f32, _ptr, _ptr, _ptr, _i64, _i64, _i32, _ptr]),
     "mmf_cross_entropy_train_bwd": (_i32, [_ptr, _i64, _ptr, _i64, _ptr, _ptr, _f32, _f32, _f32, _ptr, _i64, _i64, _i64, _i32, _ptr]),
     "mmf_sample_top_p_max_vocab": (_i64, []),
-    "mmf_sample_top_p": (_i32, [_ptr, _i64, _i64, _i64, _f32, _f32, _ptr, _ptr, _i32, _ptr]),
+    "mmf_sample_top_p": (_i32, [_ptr, _i64, _i64, _i64, _f32, _f32, _i64, _ptr, _ptr, _i32, _ptr]),
 }
 
 _lib = None

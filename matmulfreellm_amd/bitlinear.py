@@ -105,11 +105,12 @@ class FusedBitLinear(BitLinear):
     """mmfreelm/ops/fusedbitnet.py:584-610.  Same math as BitLinear here: both run the fused kernels.
 
     ``eps``: the reference's fused forward does not pass the norm's eps and so runs with
-    layer_norm_linear_quant_fn's default 1e-6 (fusedbitnet.py:602-610 vs :520); its un-fused
-    BitLinear uses the norm's 1e-8.  The default here is the norm's 1e-8; set
-    ``fused_eps=1e-6`` to reproduce the fused reference path exactly."""
+    layer_norm_linear_quant_fn's default 1e-6 (fusedbitnet.py:602-610 vs :520), while its un-fused
+    BitLinear uses the norm's 1e-8.  HGRNBitAttention, HGRNBitMLP and the lm_head are FusedBitLinear there
+    (layers/hgrn_bit.py:19, modeling_hgrn_bit.py:24), so 1e-6 is what a reference checkpoint was trained and runs
+    with: it is the default here.  ``fused_eps=None`` falls back to the inner norm's own eps."""
 
-    def __init__(self, in_features, out_features, bias=False, fused_eps=None):
+    def __init__(self, in_features, out_features, bias=False, fused_eps=1e-6):
         super().__init__(in_features, out_features, bias=bias)
         self.fused_eps = fused_eps
 

@@ -10,6 +10,8 @@
 //   l_i   = logit_i / temperature                      (fp32 division; NaN counts as -inf)
 //   p_i   = 1 if l_i == max l, else exp(l_i - max l)   (the deterministic fp32 exp of mmf_common.h)
 //   m_i   = trunc(p_i * 2^31)                          (uint32 probability mass; the row maximum has 2^31)
+//   top_k > 0:  m_i = 0 unless m_i >= the top_k-th largest mass        (transformers' TopKLogitsWarper, which the
+//               reference's call gets from the default generation parameters, top_k = 50; equal masses stay together)
 //   Z     = sum m_i,  P = max(1, trunc(double(top_p) * double(Z)))
 //   keep i  iff  m_i > 0 and  sum{ m_j : m_j > m_i } < P     (the smallest set of most probable tokens whose mass
 //                                                             reaches top_p; tokens of equal mass stay together)
@@ -20,7 +22,8 @@
 // registers.  The nucleus threshold (the smallest kept mass) is found by a radix descent over the 32-bit mass, 8 bits
 // a pass: a 256-bin histogram of mass (LDS atomics on 64-bit integers, 16 interleaved copies of every bin so that
 // neighbouring lanes hit different banks; a thread merges runs of equal bins before it touches LDS), a suffix scan of
-// the bins by one wave, and the digit whose bin straddles P.
+// the bins by one wave, and the digit whose bin straddles P.  The top_k-th largest mass comes from the same descent on
+// token counts instead of masses.
 #include "mmf_common.h"
 
 namespace {
@@ -34,6 +37,7 @@ struct SampleArgs {
     int64_t ld;
     int V;
     float temperature, top_p;
+    int top_k;              // 0: no limit
     const float* u;
     int64_t* out;
 };
@@ -47,67 +51,13 @@ __device__ __forceinline__ u64 samp_shfl_up(u64 v, int o) {
     return ((u64)hi << 32) | lo;
 }
 
-template <typename T, int NPT>
-__global__ __launch_bounds__(kSampThreads) void sample_top_p_kernel(SampleArgs a) {
-    __shared__ u64 hist[kSampBins * kSampCopies];                // 32 KiB
-    __shared__ u64 hsum[kSampBins];
-    __shared__ u64 wtot[kSampWaves], wtot2[kSampWaves];
-    __shared__ u64 sel[2];
-    __shared__ float wmax[kSampWaves];
-    __shared__ int wcand[kSampWaves];
+// Radix descent over the 32-bit masses, 8 bits a pass.  With W(S) the mass (COUNT false) or the number (COUNT true) of
+// the non-zero entries in S, returns the lowest v with W({m > v}) < limit: the smallest kept mass of the nucleus, or the
+// limit-th largest mass.  prefix = the high digits found so far, above = W of everything larger than any mass with that prefix.
+template <bool COUNT, int NPT>
+__device__ __forceinline__ unsigned samp_descent(const unsigned (&m)[NPT], u64 limit, u64* hist, u64* hsum, u64* sel) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int V = a.V;
-    const T* row = static_cast<const T*>(a.logits) + (int64_t)blockIdx.x * a.ld;
-    const int base = t * NPT;
-    const bool vec_ok = (V % 8) == 0 && (a.ld % 8) == 0 && (reinterpret_cast<uintptr_t>(a.logits) & 15u) == 0;
-
-    Raw8<T> raw[NPT / 8];
-#pragma unroll
-    for (int c = 0; c < NPT / 8; ++c) raw[c] = mmf_load8_raw<T>(row, (int64_t)base + c * 8, V, vec_ok);
-#pragma unroll
-    for (int i = 0; i < kSampBins * kSampCopies / kSampThreads; ++i) hist[i * kSampThreads + t] = 0;
-
-    float l[NPT];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int c = 0; c < NPT / 8; ++c) {
-        float v[8];
-        mmf_unpack8<T>(raw[c], v);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int idx = base + c * 8 + i;
-            float x = v[i];
-            x = (idx < V && x == x) ? __fdiv_rn(x, a.temperature) : -INFINITY;
-            l[c * 8 + i] = x;
-            mx = fmaxf(mx, x);
-        }
-    }
-    mx = mmf_wave_max(mx);
-    if (lane == 0) wmax[wave] = mx;
-    __syncthreads();                                              // also publishes the zeroed histogram
-#pragma unroll
-    for (int w = 0; w < kSampWaves; ++w) mx = fmaxf(mx, wmax[w]);
-
-    unsigned m[NPT];
-    u64 zs = 0;
-#pragma unroll
-    for (int j = 0; j < NPT; ++j) {
-        const float p = l[j] == mx ? 1.0f : mmf_exp(__fsub_rn(l[j], mx));
-        m[j] = base + j < V ? (unsigned)__fmul_rn(p, 2147483648.0f) : 0u;
-        zs += m[j];
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) zs += samp_shfl_down(zs, o);
-    if (lane == 0) wtot[wave] = zs;
-    __syncthreads();
-    u64 Z = 0;
-#pragma unroll
-    for (int w = 0; w < kSampWaves; ++w) Z += wtot[w];
-    u64 P = (u64)((double)a.top_p * (double)Z);
-    if (P < 1) P = 1;
-
-    // ---- radix descent: prefix = the high digits of the smallest kept mass, above = mass of everything larger than
-    // any mass with that prefix
+    const u64 P = limit;
     unsigned prefix = 0;
     u64 above = 0;
 #pragma unroll
@@ -126,7 +76,7 @@ __global__ __launch_bounds__(kSampThreads) void sample_top_p_kernel(SampleArgs a
                     cur = b;
                     acc = 0;
                 }
-                acc += mj;
+                acc += COUNT ? 1u : mj;
             }
         }
         if (cur >= 0) atomicAdd(&hist[cur * kSampCopies + (lane & (kSampCopies - 1))], acc);
@@ -171,7 +121,76 @@ __global__ __launch_bounds__(kSampThreads) void sample_top_p_kernel(SampleArgs a
         above = sel[0];
         prefix = (prefix << 8) | (unsigned)sel[1];
     }
-    const unsigned thr = prefix;                                  // the smallest kept mass (>= 1)
+    return prefix;
+}
+
+template <typename T, int NPT>
+__global__ __launch_bounds__(kSampThreads) void sample_top_p_kernel(SampleArgs a) {
+    __shared__ u64 hist[kSampBins * kSampCopies];                // 32 KiB
+    __shared__ u64 hsum[kSampBins];
+    __shared__ u64 wtot[kSampWaves], wtot2[kSampWaves];
+    __shared__ u64 sel[2];
+    __shared__ float wmax[kSampWaves];
+    __shared__ int wcand[kSampWaves];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int V = a.V;
+    const T* row = static_cast<const T*>(a.logits) + (int64_t)blockIdx.x * a.ld;
+    const int base = t * NPT;
+    const bool vec_ok = (V % 8) == 0 && (a.ld % 8) == 0 && (reinterpret_cast<uintptr_t>(a.logits) & 15u) == 0;
+
+    Raw8<T> raw[NPT / 8];
+#pragma unroll
+    for (int c = 0; c < NPT / 8; ++c) raw[c] = mmf_load8_raw<T>(row, (int64_t)base + c * 8, V, vec_ok);
+#pragma unroll
+    for (int i = 0; i < kSampBins * kSampCopies / kSampThreads; ++i) hist[i * kSampThreads + t] = 0;
+
+    float l[NPT];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < NPT / 8; ++c) {
+        float v[8];
+        mmf_unpack8<T>(raw[c], v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int idx = base + c * 8 + i;
+            float x = v[i];
+            x = (idx < V && x == x) ? __fdiv_rn(x, a.temperature) : -INFINITY;
+            l[c * 8 + i] = x;
+            mx = fmaxf(mx, x);
+        }
+    }
+    mx = mmf_wave_max(mx);
+    if (lane == 0) wmax[wave] = mx;
+    __syncthreads();                                              // also publishes the zeroed histogram
+#pragma unroll
+    for (int w = 0; w < kSampWaves; ++w) mx = fmaxf(mx, wmax[w]);
+
+    unsigned m[NPT];
+#pragma unroll
+    for (int j = 0; j < NPT; ++j) {
+        const float p = l[j] == mx ? 1.0f : mmf_exp(__fsub_rn(l[j], mx));
+        m[j] = base + j < V ? (unsigned)__fmul_rn(p, 2147483648.0f) : 0u;
+    }
+    if (a.top_k > 0 && a.top_k < V) {
+        const unsigned kth = samp_descent<true, NPT>(m, (u64)a.top_k, hist, hsum, sel);
+#pragma unroll
+        for (int j = 0; j < NPT; ++j) m[j] = m[j] >= kth ? m[j] : 0u;
+    }
+    u64 zs = 0;
+#pragma unroll
+    for (int j = 0; j < NPT; ++j) zs += m[j];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) zs += samp_shfl_down(zs, o);
+    if (lane == 0) wtot[wave] = zs;
+    __syncthreads();
+    u64 Z = 0;
+#pragma unroll
+    for (int w = 0; w < kSampWaves; ++w) Z += wtot[w];
+    u64 P = (u64)((double)a.top_p * (double)Z);
+    if (P < 1) P = 1;
+
+    // ---- the nucleus: the smallest kept mass
+    const unsigned thr = samp_descent<false, NPT>(m, P, hist, hsum, sel);
 
     // ---- the draw: inverse CDF over the kept masses in index order
     u64 s = 0;
@@ -231,9 +250,9 @@ extern "C" {
 int64_t mmf_sample_top_p_max_vocab(void) { return kSampMaxV; }
 
 int mmf_sample_top_p(const void* logits, int64_t ld, int64_t rows, int64_t V, float temperature, float top_p,
-                     const float* u, int64_t* out, int dtype, void* stream_) {
+                     int64_t top_k, const float* u, int64_t* out, int dtype, void* stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    if (rows < 0 || V <= 0 || ld < V || rows > 0x7fffffff) return MMF_ERR_ARG;
+    if (rows < 0 || V <= 0 || ld < V || rows > 0x7fffffff || top_k < 0) return MMF_ERR_ARG;
     if (!(temperature > 0.0f) || !(top_p == top_p)) return MMF_ERR_ARG;
     if (rows == 0) return 0;
     if (!logits || !u || !out) return MMF_ERR_ARG;
@@ -241,6 +260,7 @@ int mmf_sample_top_p(const void* logits, int64_t ld, int64_t rows, int64_t V, fl
     SampleArgs a{};
     a.logits = logits; a.ld = ld; a.V = (int)V; a.temperature = temperature;
     a.top_p = top_p < 0.0f ? 0.0f : top_p > 1.0f ? 1.0f : top_p;
+    a.top_k = top_k >= V ? 0 : (int)top_k;
     a.u = u; a.out = out;
     switch (dtype) {
         case MMF_F32: return launch_sample<float>(a, rows, stream);

@@ -529,8 +529,9 @@ def argmax(logits):
     return out.reshape(logits.shape[:-1])
 
 
-def sample_top_p(logits, top_p, temperature, u, out=None):
-    """One top-p (nucleus) draw per row; logits [..., V], u fp32 [...] uniform in [0, 1) -> int64 [...].
+def sample_top_p(logits, top_p, temperature, u, out=None, top_k=0):
+    """One top-k / top-p (nucleus) draw per row; logits [..., V], u fp32 [...] uniform in [0, 1) -> int64 [...].
+    top_k > 0 keeps the top_k most probable tokens before the nucleus is taken (0: no limit).
 
     What transformers' sampling path does per token for the reference's generate.py:11 (temperature, softmax,
     sort, cumulative sum, nucleus mask, multinomial), as one launch: integer probability masses decide the nucleus
@@ -550,8 +551,8 @@ def sample_top_p(logits, top_p, temperature, u, out=None):
     elif not (out.dtype == torch.int64 and out.device == dev and out.numel() == rows and out.is_contiguous()):
         raise L.MMFError("sample_top_p: out must be a contiguous int64 tensor with one element per row")
     with torch.cuda.device(dev):
-        L.check(lib.mmf_sample_top_p(l2.data_ptr(), l2.stride(0), rows, v, float(temperature), float(top_p), u.data_ptr(),
-                                     out.data_ptr(), L.dtype_id(l2.dtype), L.stream()), "mmf_sample_top_p")
+        L.check(lib.mmf_sample_top_p(l2.data_ptr(), l2.stride(0), rows, v, float(temperature), float(top_p), int(top_k),
+                                     u.data_ptr(), out.data_ptr(), L.dtype_id(l2.dtype), L.stream()), "mmf_sample_top_p")
     return out.reshape(logits.shape[:-1])
 
 

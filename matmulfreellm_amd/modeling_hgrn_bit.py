@@ -356,7 +356,8 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
     @torch.no_grad()
     def generate(self, input_ids: Optional[torch.LongTensor] = None, attention_mask: Optional[torch.Tensor] = None,
                  max_new_tokens: Optional[int] = None, max_length: Optional[int] = None, do_sample: bool = False,
-                 top_p: float = 1.0, temperature: float = 1.0, eos_token_id: Optional[int] = None,
+                 top_p: float = 1.0, temperature: float = 1.0, top_k: Optional[int] = None,
+                 eos_token_id: Optional[int] = None,
                  pad_token_id: Optional[int] = None, use_graph: bool = True, resident: Optional[bool] = None,
                  generator: Optional[torch.Generator] = None, **kwargs) -> torch.LongTensor:
         """Greedy (default) or top-p sampling; returns [B, T + new] token ids like HF's generate.
@@ -367,13 +368,14 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
         on the step's logits and feeds it back without a host round trip; the uniform numbers of the whole run are
         drawn up front from `generator` (torch.rand), and the logits are bit-identical to the module path's, so a
         seeded generator gives the same tokens either way (not the tokens torch.multinomial would draw from the
-        same seed).  Rows that
+        same seed).  top_k, when not given, is the generation config's, else transformers' default of 50 (what the
+        reference's call, which passes none, samples with); top_k=0 switches the limit off.  Rows that
         have produced eos_token_id (default: the generation config's) are filled with pad_token_id (eos_token_id
         when not given); generation ends early once every row has.  At batch 1 the whole decode step is one resident
         launch when the model fits it; resident=False keeps one launch per fused BitLinear.
 
         Any further keyword (num_beams, repetition_penalty, logits_processor, stopping_criteria, streamer,
-        generation_config, top_k, return_dict_in_generate, ...) sends the whole call to
+        generation_config, return_dict_in_generate, ...) sends the whole call to
         transformers' GenerationMixin.generate, which steps the module path through
         prepare_inputs_for_generation and the RecurrentCache."""
         gen_cfg = getattr(self, "generation_config", None)
@@ -385,7 +387,8 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
             hf = dict(kwargs)
             for name, value, default in (("attention_mask", attention_mask, None), ("max_new_tokens", max_new_tokens, None),
                                          ("max_length", max_length, None), ("top_p", top_p, 1.0),
-                                         ("temperature", temperature, 1.0), ("eos_token_id", eos_token_id, None),
+                                         ("temperature", temperature, 1.0), ("top_k", top_k, None),
+                                         ("eos_token_id", eos_token_id, None),
                                          ("pad_token_id", pad_token_id, None)):
                 if value is not None and not (isinstance(default, float) and value == default):
                     hf[name] = value
@@ -408,13 +411,19 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
         choose = None
         if do_sample:
             temperature = max(float(temperature), 1e-6)
+            if top_k is None:
+                top_k = getattr(gen_cfg, "top_k", None)
+                top_k = 50 if top_k is None else top_k               # transformers' default generation parameter
+            top_k = max(int(top_k), 0)
             # every uniform number of the run is drawn here, so the random stream does not depend on the path taken
             g_dev = generator.device if generator is not None else input_ids.device
             uniforms = torch.rand(max_new_tokens, B, generator=generator, device=g_dev).to(input_ids.device)
             if logits.shape[-1] <= F_.sample_top_p_max_vocab():
-                choose = lambda lg, step, out=None: F_.sample_top_p(lg, top_p, temperature, uniforms[step], out=out)
+                choose = lambda lg, step, out=None: F_.sample_top_p(lg, top_p, temperature, uniforms[step], out=out,
+                                                                    top_k=top_k)
             else:
-                choose = lambda lg, step, out=None: _sample_top_p(lg.float(), top_p, temperature, uniforms[step], out)
+                choose = lambda lg, step, out=None: _sample_top_p(lg.float(), top_p, temperature, uniforms[step], out,
+                                                                  top_k=top_k)
         first = choose(logits, 0) if do_sample else F_.argmax(logits)
         if engine is not None:
             pick = (lambda step: choose(engine.logits, step, engine.tok)) if do_sample else None
@@ -470,10 +479,14 @@ def _self_feeding(engine, first, max_new_tokens, eos_token_id, pad_token_id, chu
     return seq.contiguous()
 
 
-def _sample_top_p(logits, top_p, temperature, u, out=None):
-    """Vocabularies wider than the sampling kernel holds: the same nucleus and the same inverse CDF (kept tokens in
+def _sample_top_p(logits, top_p, temperature, u, out=None, top_k=0):
+    """Vocabularies wider than the sampling kernel holds: the same top-k limit, nucleus and inverse CDF (kept tokens in
     index order, one uniform number per row) with library calls in fp32."""
-    probs = torch.softmax(logits / temperature, dim=-1)
+    logits = logits / temperature
+    if 0 < top_k < logits.shape[-1]:
+        kth = torch.topk(logits, top_k, dim=-1).values[..., -1:]
+        logits = logits.masked_fill(logits < kth, float("-inf"))
+    probs = torch.softmax(logits, dim=-1)
     sp, si = torch.sort(probs, dim=-1, descending=True)
     keep_sorted = (sp.cumsum(-1) - sp) < max(float(top_p), 0.0)
     keep_sorted[..., 0] = True                                   # at least the most probable token

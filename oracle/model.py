@@ -134,7 +134,7 @@ def _literal_prenorm(x, w, residual, eps):
 
 
 def forward(params, input_ids, num_layers, states=None, attention_mask=None, mode="spec", rms_norm_eps=1e-6,
-            bitlinear_eps=1e-8, use_lower_bound=True, last_only=False, ops=None):
+            bitlinear_eps=1e-6, use_lower_bound=True, last_only=False, ops=None):
     """input_ids [B, T] -> (logits [B, T or 1, V], states list of [B, D])."""
     ops = ops or _Ops(mode, bitlinear_eps)
     h = params["model.embeddings.weight"][input_ids]
@@ -175,7 +175,7 @@ def argmax_lowest(logits):
 
 def greedy(params, input_ids, num_layers, max_new_tokens, mode="spec", **kw):
     """Prefill + greedy decode with carried state; returns ([B, new] tokens, list of per-step logits [B, V])."""
-    ops = _Ops(mode, kw.get("bitlinear_eps", 1e-8))
+    ops = _Ops(mode, kw.get("bitlinear_eps", 1e-6))
     logits, states = forward(params, input_ids, num_layers, mode=mode, last_only=True, ops=ops, **kw)
     toks, all_logits = [], []
     for _ in range(max_new_tokens):

@@ -1,9 +1,10 @@
 """Top-p (nucleus) sampling: CPU restatement used by the tests only (test infrastructure, never the product path).
 
 The reference samples through transformers (generate.py:11: ``model.generate(..., do_sample=True, top_p=0.4,
-temperature=0.6)``): TemperatureLogitsWarper (scores / temperature), TopPLogitsWarper (sort ascending, softmax,
-cumulative sum, drop the tokens whose cumulative probability is <= 1 - top_p, keep at least one) and a multinomial
-draw from the softmax of what is left.  transformers is a third-party dependency of the reference (not vendored);
+temperature=0.6)``): TemperatureLogitsWarper (scores / temperature), TopKLogitsWarper (the call passes no top_k, so
+the default generation parameters' 50 applies: scores below the 50th largest become -inf), TopPLogitsWarper (sort
+ascending, softmax, cumulative sum, drop the tokens whose cumulative probability is <= 1 - top_p, keep at least one)
+and a multinomial draw from the softmax of what is left.  transformers is a third-party dependency of the reference (not vendored);
 ``nucleus_literal`` restates that published algorithm in float64, and tests compare it with the installed
 transformers' own TopPLogitsWarper.
 
@@ -31,6 +32,14 @@ def masses(logits, temperature):
     return m.numpy().astype(np.uint64)
 
 
+def top_k_spec(m, top_k):
+    """Masses with everything below the top_k-th largest mass set to 0 (equal masses stay together); 0: no limit."""
+    if top_k <= 0 or top_k >= m.shape[0]:
+        return m
+    kth = np.sort(m)[-top_k]
+    return np.where(m >= kth, m, np.uint64(0))
+
+
 def nucleus_spec(m, top_p):
     """bool [V]: kept iff m_i > 0 and the mass of all strictly heavier tokens is below P = max(1, trunc(top_p * Z))."""
     top_p = np.float32(min(max(float(top_p), 0.0), 1.0))
@@ -45,9 +54,9 @@ def nucleus_spec(m, top_p):
     return keep
 
 
-def sample_top_p_spec(logits, temperature, top_p, u):
-    """One row: (token, keep mask, masses).  u is the caller's uniform number in [0, 1) (fp32)."""
-    m = masses(logits, temperature)
+def sample_top_p_spec(logits, temperature, top_p, u, top_k=0):
+    """One row: (token, keep mask, masses after the top-k limit).  u is the caller's uniform number in [0, 1) (fp32)."""
+    m = top_k_spec(masses(logits, temperature), top_k)
     keep = nucleus_spec(m, top_p)
     cum = np.cumsum(np.where(keep, m.astype(np.int64), 0))
     s = int(cum[-1])
@@ -57,9 +66,12 @@ def sample_top_p_spec(logits, temperature, top_p, u):
     return int(np.searchsorted(cum, target, side="right")), keep, m
 
 
-def nucleus_literal(logits, temperature, top_p):
-    """bool [V]: what TemperatureLogitsWarper + TopPLogitsWarper(top_p, min_tokens_to_keep=1) leave, in float64."""
+def nucleus_literal(logits, temperature, top_p, top_k=0):
+    """bool [V]: what TemperatureLogitsWarper + TopKLogitsWarper(top_k) + TopPLogitsWarper(top_p, min_tokens_to_keep=1)
+    leave, in float64 (top_k = 0: no TopKLogitsWarper)."""
     s = np.asarray(logits, dtype=np.float64) / float(temperature)
+    if 0 < top_k < s.shape[0]:
+        s = np.where(s < np.sort(s)[-top_k], -np.inf, s)
     order = np.argsort(s, kind="stable")                       # ascending
     e = np.exp(s[order] - s.max())
     cum = np.cumsum(e / e.sum())

@@ -96,7 +96,7 @@ def test_bitlinear_backward(dev, dtype, mkn, bias):
     dout = torch.randn(m, n).to(dtype)
     xc, wc, nwc = leaf(x.float()), leaf(w.float()), leaf(nw.float())
     bc = leaf(b.float()) if bias else None
-    (obw.bitlinear_ste(xc, wc, nwc, bc, eps=1e-8, weight_dtype=dtype) * dout.float()).sum().backward()
+    (obw.bitlinear_ste(xc, wc, nwc, bc, eps=1e-6, weight_dtype=dtype) * dout.float()).sum().backward()
     lin = mm.FusedBitLinear(k, n, bias=bias).to(dev, dtype)
     with torch.no_grad():
         lin.weight.copy_(w)

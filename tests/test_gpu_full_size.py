@@ -113,7 +113,7 @@ class _Case:
         self.params = {k: v.detach().cpu() for k, v in self.model.state_dict().items()}
         self.L = self.model.config.num_hidden_layers
         self.V = self.model.config.vocab_size
-        self.ops = om._Ops("spec", 1e-8)
+        self.ops = om._Ops("spec", 1e-6)
         self.dev = dev
 
     def oracle_greedy(self, ids, n_new):

@@ -262,12 +262,14 @@ def test_sampled_tokens_equal_the_oracle_driven_by_the_same_uniform_numbers(dev,
         torch.manual_seed(40 + batch)
         ids = torch.randint(0, V, (batch, 12))
         u = torch.rand(n_new, batch, generator=torch.Generator(device=dev).manual_seed(77), device=dev).cpu()
-        ops = om._Ops("spec", 1e-8)
+        ops = om._Ops("spec", 1e-6)
         logits, states = om.forward(tiny_bf16, ids, L, mode="spec", last_only=True, ops=ops)
         want = []
         for step in range(n_new):
             lg = logits[:, -1, :].float().numpy()
-            nxt = torch.tensor([osamp.sample_top_p_spec(lg[b], temperature, top_p, float(u[step, b]))[0] for b in range(batch)])
+            # generate() is given no top_k, so transformers' default of 50 applies
+            nxt = torch.tensor([osamp.sample_top_p_spec(lg[b], temperature, top_p, float(u[step, b]), top_k=50)[0]
+                                for b in range(batch)])
             want.append(nxt)
             logits, states = om.forward(tiny_bf16, nxt.reshape(-1, 1), L, states=states, mode="spec", ops=ops)
         want = torch.stack(want, dim=1)
@@ -587,6 +589,11 @@ def test_wide_vocabulary_sampling_fallback(dev, tiny_bf16, monkeypatch):
     a = F_.sample_top_p(logits, 0.9, 0.8, u)
     b = _sample_top_p(logits.float(), 0.9, 0.8, u)
     assert (a == b).sum().item() >= 62, (a != b).nonzero().flatten().tolist()
+    flat = torch.randn(64, 2000, generator=g, device=dev) * 0.6  # the top-k limit decides on flatter rows (fp32: no ties)
+    a = F_.sample_top_p(flat, 0.9, 0.8, u, top_k=50)
+    b = _sample_top_p(flat, 0.9, 0.8, u, top_k=50)
+    assert (a == b).sum().item() >= 62, (a != b).nonzero().flatten().tolist()
+    assert (a != F_.sample_top_p(flat, 0.9, 0.8, u)).any()
     model = build(tiny_bf16, torch.bfloat16, dev)
     torch.manual_seed(70)
     ids = torch.randint(0, V, (3, 8), device=dev)

@@ -14,9 +14,10 @@ def F():
     return F_
 
 
-def _check_rows(dev, logits, temperature, top_p, u, what):
-    got = F().sample_top_p(logits.to(dev), top_p, temperature, u.to(dev)).cpu()
-    want = [S.sample_top_p_spec(logits[r].float().numpy(), temperature, top_p, float(u[r]))[0] for r in range(logits.shape[0])]
+def _check_rows(dev, logits, temperature, top_p, u, what, top_k=0):
+    got = F().sample_top_p(logits.to(dev), top_p, temperature, u.to(dev), top_k=top_k).cpu()
+    want = [S.sample_top_p_spec(logits[r].float().numpy(), temperature, top_p, float(u[r]), top_k=top_k)[0]
+            for r in range(logits.shape[0])]
     bad = [(r, int(got[r]), want[r]) for r in range(len(want)) if int(got[r]) != want[r]]
     print(f"{what}: {len(want)} rows, {len(bad)} differ", flush=True)
     assert not bad, (what, bad[:5])
@@ -32,6 +33,31 @@ def test_tokens_equal_the_integer_restatement_at_vocabulary_32000(dev, dtype):
     u = torch.rand(rows, generator=g)
     for temperature, top_p in ((0.6, 0.4), (1.0, 0.9), (0.25, 0.05), (1.3, 1.0)):
         _check_rows(dev, logits, temperature, top_p, u, f"{dtype} T={temperature} top_p={top_p}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_top_k_limit_before_the_nucleus(dev, dtype):
+    """transformers' default top_k = 50 (what the reference's generate.py samples with) and other limits, on flat rows
+    (where the nucleus alone would hold hundreds of tokens, so the limit decides), peaked rows, rows of equal logits
+    (ties at the limit stay together), ragged and two-pass vocabularies, and limits of V or more (no limit)."""
+    g = torch.Generator().manual_seed(31)
+    rows = 32
+    sharp = torch.tensor([0.05, 0.3, 1.0, 4.0]).repeat(rows // 4)[:, None]
+    logits = (torch.randn(rows, 32000, generator=g) * sharp).to(dtype)
+    logits[5] = 0.25                                              # every token ties
+    logits[6, 100:] = -3.0                                        # 100 random heads, then one big tie
+    u = torch.rand(rows, generator=g)
+    for top_k, temperature, top_p in ((50, 0.6, 0.4), (50, 1.0, 1.0), (1, 0.7, 0.9), (7, 1.0, 0.95), (1000, 0.6, 0.999),
+                                      (32000, 0.6, 0.4), (40000, 0.6, 0.4)):
+        _check_rows(dev, logits, temperature, top_p, u, f"{dtype} top_k={top_k} T={temperature} top_p={top_p}", top_k=top_k)
+    # the limit bites on the flat rows: fewer tokens can be drawn than without it
+    flat = logits[0].float().numpy()
+    assert S.sample_top_p_spec(flat, 0.6, 0.4, 0.0, top_k=50)[1].sum() < S.sample_top_p_spec(flat, 0.6, 0.4, 0.0)[1].sum()
+    for v in (3, 33, 4097, 50257):
+        lg = (torch.randn(6, v, generator=g) * 0.5).to(dtype)
+        _check_rows(dev, lg, 0.8, 0.9, u[:6], f"{dtype} V={v} top_k=50", top_k=50)
+    with pytest.raises(Exception):
+        F().sample_top_p(logits.to(dev), 0.5, 1.0, u.to(dev), top_k=-1)
 
 
 def test_ragged_vocabularies_strided_rows_and_two_passes_per_thread(dev):

@@ -96,9 +96,11 @@ def test_config_and_module_tree_mirror_the_reference():
 def test_layer_norm_linear_quant_fn_rejects_unsupported_forms():
     import matmulfreellm_amd as mm
     x, w = torch.randn(2, 64), torch.randn(8, 64)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(NotImplementedError):           # the LayerNorm form has no backward
+        mm.layer_norm_linear_quant_fn(x.clone().requires_grad_(), torch.ones(64), None, w, None, is_rms_norm=False)
+    with pytest.raises(RuntimeError):                  # and, like every op here, no CPU path
         mm.layer_norm_linear_quant_fn(x, torch.ones(64), None, w, None, is_rms_norm=False)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(NotImplementedError):           # a norm bias exists for the LayerNorm form only
         mm.layer_norm_linear_quant_fn(x, torch.ones(64), torch.zeros(64), w, None, is_rms_norm=True)
     with pytest.raises(NotImplementedError):
         mm.HGRNBitAttention(hidden_size=64, num_heads=1, use_short_conv=True)

@@ -51,6 +51,47 @@ def test_nucleus_is_the_one_transformers_keeps(top_p):
         assert (spec == hf_keep).all()
 
 
+@pytest.mark.parametrize("top_k,top_p", [(50, 0.4), (50, 0.999), (5, 0.9), (1, 1.0), (300, 0.95)])
+def test_top_k_then_nucleus_is_what_transformers_keeps(top_k, top_p):
+    """The reference's generate.py passes no top_k, so transformers applies its default of 50 before the nucleus:
+    TemperatureLogitsWarper -> TopKLogitsWarper -> TopPLogitsWarper.  On flat rows (where the nucleus alone would hold
+    more than top_k tokens) the limit changes the kept set: both restatements must keep what the installed warpers keep."""
+    from transformers.generation.logits_process import TemperatureLogitsWarper, TopKLogitsWarper, TopPLogitsWarper
+    rng = np.random.default_rng(12)
+    limited = 0
+    for case in range(6):
+        sharp = (0.3, 1.0, 3.0)[case % 3]
+        lg = (rng.standard_normal(4000) * sharp).astype(np.float32)
+        t = 0.6
+        scores = TemperatureLogitsWarper(t)(None, torch.from_numpy(lg)[None])
+        scores = TopPLogitsWarper(top_p=top_p)(None, TopKLogitsWarper(top_k=top_k)(None, scores))[0]
+        hf_keep = torch.isfinite(scores).numpy()
+        lit = S.nucleus_literal(lg, t, top_p, top_k)
+        m = S.top_k_spec(S.masses(lg, t), top_k)
+        spec = S.nucleus_spec(m, top_p)
+        assert (lit == hf_keep).all()
+        assert (spec == hf_keep).all()
+        assert int((m > 0).sum()) == top_k
+        limited += int(hf_keep.sum() < S.nucleus_literal(lg, t, top_p).sum())
+    assert limited > 0 or top_k >= 300, "no case where the top-k limit bites: the test would not see it dropped"
+
+
+def test_top_k_closed_forms():
+    lg = np.log(np.array([0.1, 0.4, 0.2, 0.3], dtype=np.float32))
+    # top_k 2 keeps tokens 1 and 3 (0.4, 0.3), renormalised 4/7 and 3/7; top_p 1.0 then keeps both
+    tok = [S.sample_top_p_spec(lg, 1.0, 1.0, u, top_k=2)[0] for u in (0.0, 0.57, 0.58, 0.99)]
+    assert tok == [1, 1, 3, 3]
+    assert S.sample_top_p_spec(lg, 1.0, 1.0, 0.0, top_k=2)[1].tolist() == [False, True, False, True]
+    # the nucleus is taken of the limited set: 0.4 / 0.7 = 0.571 >= 0.5, so top_p 0.5 keeps token 1 only
+    assert S.sample_top_p_spec(lg, 1.0, 0.5, 0.9, top_k=2)[1].tolist() == [False, True, False, False]
+    # without the limit 0.4 < 0.5 and the second token stays
+    assert S.sample_top_p_spec(lg, 1.0, 0.5, 0.9, top_k=0)[1].tolist() == [False, True, False, True]
+    # equal masses at the limit stay together; a limit of V or more is no limit
+    flat = np.zeros(6, dtype=np.float32)
+    assert S.sample_top_p_spec(flat, 1.0, 1.0, 0.0, top_k=2)[1].all()
+    assert S.sample_top_p_spec(lg, 1.0, 1.0, 0.0, top_k=4)[1].all() and S.sample_top_p_spec(lg, 1.0, 1.0, 0.0, top_k=9)[1].all()
+
+
 def test_the_draw_realises_the_renormalised_distribution():
     rng = np.random.default_rng(3)
     lg = (rng.standard_normal(50) * 2).astype(np.float32)

@@ -32,7 +32,8 @@ import torch
 from oracle import model as om
 
 V, H, I, L = 24, 8, 16, 3
-RMS_EPS, BL_EPS = 1e-6, 1e-8
+RMS_EPS, BL_EPS = 1e-6, 1e-6   # block norms: config rms_norm_eps; projections: FusedBitLinear.forward passes no eps
+                               # and runs with layer_norm_linear_quant_fn's default (fusedbitnet.py:602-610, :520)
 
 
 # ------------------------------------------------------------------ the independent restatement (numpy float64)
@@ -149,7 +150,7 @@ def _torch_params(p):
     return {k: torch.from_numpy(np.ascontiguousarray(v)).to(torch.float32) for k, v in p.items()}
 
 
-SEED = 40          # a seed whose model keeps every pre-rounding value >= 1e-3 away from a tie (checked below)
+SEED = 78          # a seed whose model keeps every pre-rounding value >= 1e-3 away from a tie (checked below)
 _MARGIN_NEEDED = 1e-3
 
 
