@@ -249,8 +249,8 @@ def _rotating(make_set, set_bytes, min_total=512 << 20, min_sets=3):
 
 # HBM bytes per launch of the bandwidth-bound kernels at the shapes below, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/hbm_traffic_scan_norm_loss.txt; same calibration copy as the decode kernels).
-COUNTED_TRAFFIC = {"hgrn_recurrent": 201466341, "hgrn_chunk": 201478277, "rmsnorm": 134308657, "rmsnorm_swishgate": 201466176,
-                   "cross_entropy": 263075006}
+COUNTED_TRAFFIC = {"hgrn_recurrent": 201453786, "hgrn_chunk": 201465919, "rmsnorm": 134330432,
+                   "rmsnorm_swishgate": 201482279, "cross_entropy": 263065702}
 
 
 def scan_bench(dev, b=8, t=2048, d=2048, iters=12):

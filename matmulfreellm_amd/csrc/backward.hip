@@ -56,7 +56,9 @@ struct NormBwdArgs {
     double inv_K;
 };
 
-template <typename T, typename TW, int NV, int MODE>
+// VEC: K, the row strides and the base addresses allow 4-element vector accesses (a thread's 4 channels are then all inside
+// the row or all outside it).
+template <typename T, typename TW, int NV, int MODE, bool VEC>
 __global__ __launch_bounds__(kBT) void rmsnorm_bwd_kernel(NormBwdArgs a) {
     __shared__ double red_d[kBT / 64];
     __shared__ float red_f[kBT / 64];
@@ -79,16 +81,34 @@ __global__ __launch_bounds__(kBT) void rmsnorm_bwd_kernel(NormBwdArgs a) {
         const T* dr = a.dres ? static_cast<const T*>(a.dres) + row * (int64_t)K : nullptr;
         float xv[NV][4], dv[NV][4], gv[MODE == BWD_GATED ? NV : 1][4], rv[NV][4];
         double ss = 0.0;
+        // every load of the row is issued before anything is converted
+        Raw4<T> xr[NV], dyr[NV], gr[MODE == BWD_GATED ? NV : 1], rr[NV];
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int k0 = (v * kBT + (int)threadIdx.x) * 4;
+            if (k0 < K) {
+                xr[v] = raw4_load<T, VEC>(x, k0, K);
+                dyr[v] = raw4_load<T, VEC>(dy, k0, K);
+                if constexpr (MODE == BWD_GATED) gr[v] = raw4_load<T, VEC>(gt, k0, K);
+                if (dr) rr[v] = raw4_load<T, VEC>(dr, k0, K);
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int k0 = (v * kBT + (int)threadIdx.x) * 4;
+            if (k0 < K) {
+                raw4_unpack<T>(xr[v], xv[v]);
+                raw4_unpack<T>(dyr[v], dv[v]);
+                if constexpr (MODE == BWD_GATED) raw4_unpack<T>(gr[v], gv[v]);
+                if (dr) raw4_unpack<T>(rr[v], rv[v]);
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const bool in = k0 + i < K;
-                xv[v][i] = in ? mmf_to_float(x[k0 + i]) : 0.0f;
-                dv[v][i] = in ? mmf_to_float(dy[k0 + i]) : 0.0f;
-                if constexpr (MODE == BWD_GATED) gv[v][i] = in ? mmf_to_float(gt[k0 + i]) : 0.0f;
-                rv[v][i] = (dr && in) ? mmf_to_float(dr[k0 + i]) : 0.0f;
+                xv[v][i] = in ? xv[v][i] : 0.0f;
+                dv[v][i] = in ? dv[v][i] : 0.0f;
+                if constexpr (MODE == BWD_GATED) gv[v][i] = in ? gv[v][i] : 0.0f;
+                rv[v][i] = (dr && in) ? rv[v][i] : 0.0f;
                 ss += (double)xv[v][i] * (double)xv[v][i];
             }
         }
@@ -116,12 +136,11 @@ __global__ __launch_bounds__(kBT) void rmsnorm_bwd_kernel(NormBwdArgs a) {
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int k0 = (v * kBT + (int)threadIdx.x) * 4;
+            float o[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (k0 + i < K) {
-                    dx[k0 + i] = mmf_from_float<T>((wdy[v][i] - xh[v][i] * c1) * rstd + rv[v][i]);
-                    if constexpr (MODE == BWD_GATED) static_cast<T*>(a.dgate)[row * (int64_t)K + k0 + i] = mmf_from_float<T>(gv[v][i]);
-                }
+            for (int i = 0; i < 4; ++i) o[i] = (wdy[v][i] - xh[v][i] * c1) * rstd + rv[v][i];
+            raw4_store<T, VEC>(dx, k0, K, o);
+            if constexpr (MODE == BWD_GATED) raw4_store<T, VEC>(static_cast<T*>(a.dgate) + row * (int64_t)K, k0, K, gv[v]);
         }
         if constexpr (MODE == BWD_QUANT) {
             amax = mmf_block_max<kBT / 64>(amax, red_f);
@@ -130,9 +149,10 @@ __global__ __launch_bounds__(kBT) void rmsnorm_bwd_kernel(NormBwdArgs a) {
 #pragma unroll
             for (int v = 0; v < NV; ++v) {
                 const int k0 = (v * kBT + (int)threadIdx.x) * 4;
+                float o[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (k0 + i < K) y[k0 + i] = mmf_from_float<T>(__fmul_rn((float)mmf_code(__fmul_rn(xh[v][i], wv[v][i]), scale), deq));
+                for (int i = 0; i < 4; ++i) o[i] = __fmul_rn((float)mmf_code(__fmul_rn(xh[v][i], wv[v][i]), scale), deq);
+                raw4_store<T, VEC>(y, k0, K, o);
             }
         }
     }
@@ -180,15 +200,23 @@ void launch_colsum(const float* part, int groups, int64_t K, T* out, hipStream_t
     colsum_kernel<T><<<(unsigned)mmf_ceil_div(K, kColsumCols), kColsumCols * kColsumLanes, 0, s>>>(part, groups, (int)K, out);
 }
 
-template <typename T, typename TW, int MODE>
-int launch_norm_bwd(const NormBwdArgs& a, int groups, hipStream_t s) {
+template <typename T, typename TW, int MODE, bool VEC>
+int launch_norm_bwd_v(const NormBwdArgs& a, int groups, hipStream_t s) {
     const int nv = (int)mmf_ceil_div(a.K, kBT * 4);
-    if (nv <= 1) rmsnorm_bwd_kernel<T, TW, 1, MODE><<<groups, kBT, 0, s>>>(a);
-    else if (nv <= 2) rmsnorm_bwd_kernel<T, TW, 2, MODE><<<groups, kBT, 0, s>>>(a);
-    else if (nv <= 4) rmsnorm_bwd_kernel<T, TW, 4, MODE><<<groups, kBT, 0, s>>>(a);
+    if (nv <= 1) rmsnorm_bwd_kernel<T, TW, 1, MODE, VEC><<<groups, kBT, 0, s>>>(a);
+    else if (nv <= 2) rmsnorm_bwd_kernel<T, TW, 2, MODE, VEC><<<groups, kBT, 0, s>>>(a);
+    else if (nv <= 4) rmsnorm_bwd_kernel<T, TW, 4, MODE, VEC><<<groups, kBT, 0, s>>>(a);
     else return MMF_ERR_WIDE;
     MMF_CHECK_LAUNCH();
     return 0;
+}
+template <typename T, typename TW, int MODE>
+int launch_norm_bwd(const NormBwdArgs& a, int groups, hipStream_t s) {
+    const uintptr_t al = 4 * sizeof(T) - 1;
+    auto ok = [&](const void* p) { return (reinterpret_cast<uintptr_t>(p) & al) == 0; };
+    const bool vec = a.K % 4 == 0 && a.ldx % 4 == 0 && a.ldg % 4 == 0 && a.lddy % 4 == 0 && ok(a.x) && ok(a.gate) && ok(a.dy) &&
+                     ok(a.dres) && ok(a.dx) && ok(a.dgate) && ok(a.y);
+    return vec ? launch_norm_bwd_v<T, TW, MODE, true>(a, groups, s) : launch_norm_bwd_v<T, TW, MODE, false>(a, groups, s);
 }
 template <typename T, typename TW>
 int dispatch_norm_bwd(const NormBwdArgs& a, int mode, int groups, hipStream_t s) {
@@ -217,7 +245,7 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ x
 
 // ------------------------------------------------------------------------------------------ gate math
 // forward: s = sigmoid(f); g = lb + (1 - lb) s; x = i sigmoid(i) (1 - g), 0 on masked rows.  A thread owns 4 channels and walks rows.
-template <typename T>
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void hgrn_gate_bwd_kernel(const T* __restrict__ i_in, int64_t ldi, const T* __restrict__ f_in,
                                                             int64_t ldf, const float* __restrict__ lb,
                                                             const uint8_t* __restrict__ mask, const T* __restrict__ gx,
@@ -225,6 +253,7 @@ __global__ __launch_bounds__(256) void hgrn_gate_bwd_kernel(const T* __restrict_
                                                             T* __restrict__ df, int64_t lddf, float* __restrict__ dlb_part,
                                                             int64_t rows, int D) {
     const int d0 = ((int)blockIdx.x * 256 + (int)threadIdx.x) * 4;
+    if (d0 >= D) return;
     float lbv[4], acc[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -233,20 +262,24 @@ __global__ __launch_bounds__(256) void hgrn_gate_bwd_kernel(const T* __restrict_
     }
     for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
         const bool keep = !(mask && mask[r] == 0);
+        float iv4[4], fv4[4], dx4[4], dg4[4], di4[4], df4[4];
+        const Raw4<T> ir = raw4_load<T, VEC>(i_in + r * ldi, d0, D), fr = raw4_load<T, VEC>(f_in + r * ldf, d0, D);
+        const Raw4<T> xr = raw4_load<T, VEC>(gx + r * (int64_t)D, d0, D), gr = raw4_load<T, VEC>(gg + r * (int64_t)D, d0, D);
+        raw4_unpack<T>(ir, iv4); raw4_unpack<T>(fr, fv4); raw4_unpack<T>(xr, dx4); raw4_unpack<T>(gr, dg4);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const int d = d0 + e;
-            if (d >= D) continue;
-            const float iv = mmf_to_float(i_in[r * ldi + d]), fv = mmf_to_float(f_in[r * ldf + d]);
-            const float dX = keep ? mmf_to_float(gx[r * (int64_t)D + d]) : 0.0f, dG = mmf_to_float(gg[r * (int64_t)D + d]);
+            const float iv = iv4[e], fv = fv4[e];
+            const float dX = keep ? dx4[e] : 0.0f, dG = dg4[e];
             const float s = fast_sigmoid(fv), g = lb ? lbv[e] + (1.0f - lbv[e]) * s : s;
             const float si = fast_sigmoid(iv), sw = iv * si, u = 1.0f - g;
             const float dgt = dG - dX * sw;                        // u = 1 - g
             const float ds = lb ? dgt * (1.0f - lbv[e]) : dgt;
-            acc[e] += dgt * (1.0f - s);
-            di[r * lddi + d] = mmf_from_float<T>(dX * u * si * (1.0f + iv * (1.0f - si)));
-            df[r * lddf + d] = mmf_from_float<T>(ds * s * (1.0f - s));
+            if (d0 + e < D) acc[e] += dgt * (1.0f - s);
+            di4[e] = dX * u * si * (1.0f + iv * (1.0f - si));
+            df4[e] = ds * s * (1.0f - s);
         }
+        raw4_store<T, VEC>(di + r * lddi, d0, D, di4);
+        raw4_store<T, VEC>(df + r * lddf, d0, D, df4);
     }
     if (dlb_part) {
 #pragma unroll
@@ -480,13 +513,17 @@ int mmf_hgrn_gate_bwd(const void* i_in, int64_t ldi, const void* f_in, int64_t l
     const int groups = mmf_backward_groups(rows);
     float* part = (lower_bound && dlb) ? dlb_partial : nullptr;
     dim3 grid((unsigned)mmf_ceil_div(D, 1024), (unsigned)groups);
-#define MMF_GB(T) hgrn_gate_bwd_kernel<T><<<grid, 256, 0, stream>>>(static_cast<const T*>(i_in), ldi, static_cast<const T*>(f_in), ldf, \
+    const uintptr_t al = (dtype == MMF_F32 ? 16 : 8) - 1;
+    auto ok = [&](const void* p) { return (reinterpret_cast<uintptr_t>(p) & al) == 0; };
+    const bool vec = D % 4 == 0 && ldi % 4 == 0 && ldf % 4 == 0 && lddi % 4 == 0 && lddf % 4 == 0 && ok(i_in) && ok(f_in) &&
+                     ok(grad_x) && ok(grad_g) && ok(di) && ok(df);
+#define MMF_GB(T, V) hgrn_gate_bwd_kernel<T, V><<<grid, 256, 0, stream>>>(static_cast<const T*>(i_in), ldi, static_cast<const T*>(f_in), ldf, \
         lower_bound, mask, static_cast<const T*>(grad_x), static_cast<const T*>(grad_g), static_cast<T*>(di), lddi, static_cast<T*>(df), \
         lddf, part, rows, (int)D)
     switch (dtype) {
-        case MMF_F32: MMF_GB(float); break;
-        case MMF_BF16: MMF_GB(bf16_t); break;
-        case MMF_F16: MMF_GB(f16_t); break;
+        case MMF_F32: if (vec) MMF_GB(float, true); else MMF_GB(float, false); break;
+        case MMF_BF16: if (vec) MMF_GB(bf16_t, true); else MMF_GB(bf16_t, false); break;
+        case MMF_F16: if (vec) MMF_GB(f16_t, true); else MMF_GB(f16_t, false); break;
         default: return MMF_ERR_ARG;
     }
 #undef MMF_GB

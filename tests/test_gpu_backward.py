@@ -33,7 +33,7 @@ def leaf(t, dev=None):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("mk", [(7, 64), (33, 300), (16, 2048), (5, 5632)])
+@pytest.mark.parametrize("mk", [(7, 64), (33, 300), (16, 2048), (5, 5632), (9, 301)])   # 301: the element-wise access path
 @pytest.mark.parametrize("residual", [False, True])
 def test_rmsnorm_backward(dev, dtype, mk, residual):
     import matmulfreellm_amd as mm
@@ -141,10 +141,11 @@ def test_swiglu_backward_on_column_slices(dev, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("use_lb", [False, True])
-def test_gate_math_backward(dev, dtype, use_lb):
+@pytest.mark.parametrize("d", [192, 70])                                                 # 70: the element-wise access path
+def test_gate_math_backward(dev, dtype, use_lb, d):
     from matmulfreellm_amd.autograd import HGRNGateFn
     torch.manual_seed(6)
-    b, t, d = 3, 5, 192
+    b, t = 3, 5
     i, f = (2 * torch.randn(b, t, d)).to(dtype), (2 * torch.randn(b, t, d)).to(dtype)
     lb = torch.rand(d) * 0.5 if use_lb else None
     mask = torch.ones(b, t)
