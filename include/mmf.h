@@ -110,6 +110,7 @@ int mmf_layernorm_quant(const void* x, const void* residual, const void* weight,
 
 /* mmf_rmsnorm_quant_fused: the same quantiser (tiled codes) with the elementwise op that precedes a
  * BitLinear in the model folded in, for batches that go to the matrix cores:
+ *   0 PLAIN      v = x (what mmf_rmsnorm_quant computes, in the many-rows-per-workgroup form; w1 unused)
  *   1 NORM       v = RMSNorm(x; w1, eps1)                                  modeling_hgrn_bit.py:98
  *   2 RESNORM    s = x + aux; res_out = s; v = RMSNorm(s; w1, eps1)        modeling_hgrn_bit.py:107
  *   3 STEP_GATE  x, aux, aux2 = raw i, f, g projections of ONE token per row: gate math and one recurrence

@@ -210,6 +210,7 @@ int dispatch_x(const RowArgs& a, int x_dtype, int r_dtype, int w_dtype, hipStrea
 // ---------------------------------------------------------------- fused prologue + quantiser
 // The int8 quantiser with the elementwise op that precedes each BitLinear of a decode step
 // folded in (batch sizes that go to the matrix cores, where the codes must exist in memory):
+//   QPRO_PLAIN      v = x                                                  (nothing in front: many-row form of ROW_QUANT)
 //   QPRO_NORM       v = T(RMSNorm(x; w1, eps1))                            (block norm)
 //   QPRO_RESNORM    s = x + aux; res_out = s; v = T(RMSNorm(s; w1, eps1))  (fused residual norm)
 //   QPRO_STEP_GATE  i = x, f = aux, g = aux2 (raw projections of one token): gate math, one recurrence
@@ -217,7 +218,7 @@ int dispatch_x(const RowArgs& a, int x_dtype, int r_dtype, int w_dtype, hipStrea
 //   QPRO_SWIGLU     v = T((x * aux) / (1 + exp(-x)))                       (MLP activation)
 //   QPRO_GATEDNORM  v = T(RMSNorm(x; w1, eps1) * aux * sigmoid(aux))       (g_norm in front of o_proj, any T)
 // then  y = RMSNorm(v; norm_w, eps),  q = int8 absmax codes of y  (tiled operand layout).
-enum QPro : int { QPRO_NORM = 1, QPRO_RESNORM = 2, QPRO_STEP_GATE = 3, QPRO_SWIGLU = 4, QPRO_GATEDNORM = 5 };
+enum QPro : int { QPRO_PLAIN = 0, QPRO_NORM = 1, QPRO_RESNORM = 2, QPRO_STEP_GATE = 3, QPRO_SWIGLU = 4, QPRO_GATEDNORM = 5 };
 
 struct FusedQuantArgs {
     const void* x; const void* aux; const void* aux2;
@@ -245,7 +246,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
     __shared__ double red_a[kQWaves], red_b[kQWaves];
     __shared__ float red_f[kQWaves];
     __shared__ int red_i[kQWaves];
-    constexpr bool HAS_AUX = PRO >= QPRO_RESNORM, STEP = PRO == QPRO_STEP_GATE, HAS_W1 = PRO != QPRO_SWIGLU;
+    constexpr bool HAS_AUX = PRO >= QPRO_RESNORM, STEP = PRO == QPRO_STEP_GATE, HAS_W1 = PRO != QPRO_SWIGLU && PRO != QPRO_PLAIN;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int w0 = (wave / WPR) * WPR;                          // first wave of this row
     const int tr = (int)threadIdx.x % TPR;                      // thread within the row
@@ -347,7 +348,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
                 xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(y) : 0.0f;
             }
         }
-    } else {
+    } else if constexpr (PRO == QPRO_SWIGLU) {
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int k0 = (v * TPR + tr) * 4;
@@ -464,6 +465,7 @@ int launch_fused_quant(const FusedQuantArgs& a, bool vec, hipStream_t s) {
 template <typename T, typename TW>
 int dispatch_fused_quant(const FusedQuantArgs& a, int pro, bool vec, hipStream_t s) {
     switch (pro) {
+        case QPRO_PLAIN: return launch_fused_quant<T, TW, QPRO_PLAIN>(a, vec, s);
         case QPRO_NORM: return launch_fused_quant<T, TW, QPRO_NORM>(a, vec, s);
         case QPRO_RESNORM: return launch_fused_quant<T, TW, QPRO_RESNORM>(a, vec, s);
         case QPRO_STEP_GATE: return launch_fused_quant<T, TW, QPRO_STEP_GATE>(a, vec, s);
@@ -600,10 +602,10 @@ int mmf_rmsnorm_quant_fused(int prologue, const void* x, int64_t ldx, const void
     if (M < 0 || K <= 0 || ldx < K) return MMF_ERR_ARG;
     if (M == 0) return 0;
     if (!x || !q || !deq || !qsum) return MMF_ERR_ARG;
-    if (prologue < QPRO_NORM || prologue > QPRO_GATEDNORM) return MMF_ERR_ARG;
+    if (prologue < QPRO_PLAIN || prologue > QPRO_GATEDNORM) return MMF_ERR_ARG;
     if (prologue >= QPRO_RESNORM && (!aux || ldaux < K)) return MMF_ERR_ARG;
     if (prologue == QPRO_STEP_GATE && (!aux2 || ldaux2 < K || !state)) return MMF_ERR_ARG;
-    if (prologue != QPRO_SWIGLU && !w1) return MMF_ERR_ARG;
+    if (prologue != QPRO_SWIGLU && prologue != QPRO_PLAIN && !w1) return MMF_ERR_ARG;
     FusedQuantArgs a{};
     a.x = x; a.aux = aux ? aux : x; a.aux2 = aux2 ? aux2 : x; a.ldx = ldx; a.ldaux = aux ? ldaux : ldx;
     a.ldaux2 = aux2 ? ldaux2 : ldx; a.res_out = res_out; a.w1 = w1; a.norm_w = norm_weight; a.lb = lower_bound; a.state = state;

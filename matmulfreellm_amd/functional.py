@@ -172,6 +172,18 @@ def rmsnorm_quant(x, weight, residual=None, eps=1e-8, tiled=False, prenorm=False
     if norm_bias is not None:
         raise ValueError("norm_bias needs is_rms_norm=False (the RMSNorm of the BitLinear path has no bias)")
     m, k = x2.shape
+    if (tiled and r2 is None and res_out is None and m > 256 and k % 4 == 0 and k <= 8192
+            and (w is None or w.dtype in (x2.dtype, torch.float32))):
+        # many rows: the form that puts several rows in a workgroup (one wave per 2048 elements of a row)
+        q = torch.empty(lib.mmf_codes_bytes(m, k, 1), dtype=torch.int8, device=dev)
+        deq = torch.empty(m, dtype=torch.float32, device=dev)
+        qsum = torch.empty(m, dtype=torch.int32, device=dev)
+        with torch.cuda.device(dev):
+            L.check(lib.mmf_rmsnorm_quant_fused(0, x2.data_ptr(), x2.stride(0), None, 0, None, 0, None, None, 0.0, L.ptr(w), eps,
+                                                None, None, q.data_ptr(), deq.data_ptr(), qsum.data_ptr(), m, k,
+                                                L.dtype_id(x2.dtype), L.dtype_id(w.dtype) if w is not None else 0, L.stream()),
+                    "mmf_rmsnorm_quant_fused")
+        return (q, deq, qsum, x) if prenorm else (q, deq, qsum)
     kp = -(-k // 128) * 128
     nbytes = lib.mmf_codes_bytes(m, k, 1 if tiled else 0)
     q = torch.empty(nbytes, dtype=torch.int8, device=dev)

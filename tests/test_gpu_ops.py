@@ -133,7 +133,8 @@ def test_swiglu(dev, dtype):
 
 # ------------------------------------------------------------------ activation codes
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("mk", [(1, 2048), (64, 2048), (33, 5632), (5, 300), (4096, 2048), (130, 1536)])
+@pytest.mark.parametrize("mk", [(1, 2048), (64, 2048), (33, 5632), (5, 300), (4096, 2048), (130, 1536), (300, 5632), (257, 300),
+                                (700, 8192)])   # more than 256 rows, tiled: several rows per workgroup
 @pytest.mark.parametrize("tiled", [False, True])
 def test_rmsnorm_quant_codes(dev, dtype, mk, tiled):
     torch.manual_seed(6)
