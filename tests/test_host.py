@@ -179,7 +179,7 @@ def test_rejected_shapes_and_pointers_return_their_code_before_any_launch():
     # fused quantiser
     fq = lambda pro, k: lib.mmf_rmsnorm_quant_fused(pro, P, k, P, k, None, 0, None, P, 1e-6, P, 1e-8, None, None, P, P, P, 3, k,
                                                     1, 1, None)
-    assert fq(9, 2048) == -1 and fq(0, 2048) == -1
+    assert fq(9, 2048) == -1 and fq(-1, 2048) == -1              # 0 is the plain prologue
     assert fq(1, 20000) == -2
     assert lib.mmf_rmsnorm_quant_fused(1, P + 2, 2048, None, 0, None, 0, None, P, 1e-6, P, 1e-8, None, None, P, P, P, 3, 2048,
                                        1, 1, None) == -3
