@@ -295,10 +295,10 @@ int mmf_cross_entropy_train_bwd(const void* logits, int64_t ld, const int64_t* l
  *   cumulative sum, nucleus mask, renormalisation and the multinomial draw -- one launch, no sort.
  *   All decisions are made on integer probability masses, so the result does not depend on a summation order:
  *     l_i = logit_i / temperature (NaN counts as -inf);  p_i = 1 if l_i == max l, else exp(l_i - max l) in fp32;
- *     m_i = trunc(p_i * 2^31);
- *     top_k > 0: m_i = 0 unless m_i >= the top_k-th largest mass (transformers' TopKLogitsWarper runs before the
+ *     top_k > 0: l_i = -inf unless l_i >= the top_k-th largest l (transformers' TopKLogitsWarper runs before the
  *       top-p one; the reference's call passes no top_k and so gets the default generation parameters' 50;
- *       equal masses stay together; top_k = 0 or >= V: no limit);
+ *       equal values stay together; top_k = 0 or >= V: no limit) -- applied before p_i, with max l unchanged;
+ *     m_i = trunc(p_i * 2^31);
  *     Z = sum m_i;  P = max(1, trunc(double(top_p) * double(Z)))  (top_p clamped to [0, 1]);
  *     token i is kept iff m_i > 0 and the mass of all tokens with m_j > m_i is below P;
  *     S = mass of the kept tokens;  target = trunc(double(u[r]) * double(S));

@@ -9,9 +9,9 @@
 // reproduces it exactly:
 //   l_i   = logit_i / temperature                      (fp32 division; NaN counts as -inf)
 //   p_i   = 1 if l_i == max l, else exp(l_i - max l)   (the deterministic fp32 exp of mmf_common.h)
+//   top_k > 0:  l_i = -inf unless l_i >= the top_k-th largest l        (transformers' TopKLogitsWarper, which the
+//               reference's call gets from the default generation parameters, top_k = 50; equal values stay together)
 //   m_i   = trunc(p_i * 2^31)                          (uint32 probability mass; the row maximum has 2^31)
-//   top_k > 0:  m_i = 0 unless m_i >= the top_k-th largest mass        (transformers' TopKLogitsWarper, which the
-//               reference's call gets from the default generation parameters, top_k = 50; equal masses stay together)
 //   Z     = sum m_i,  P = max(1, trunc(double(top_p) * double(Z)))
 //   keep i  iff  m_i > 0 and  sum{ m_j : m_j > m_i } < P     (the smallest set of most probable tokens whose mass
 //                                                             reaches top_p; tokens of equal mass stay together)
@@ -22,8 +22,9 @@
 // registers.  The nucleus threshold (the smallest kept mass) is found by a radix descent over the 32-bit mass, 8 bits
 // a pass: a 256-bin histogram of mass (LDS atomics on 64-bit integers, 16 interleaved copies of every bin so that
 // neighbouring lanes hit different banks; a thread merges runs of equal bins before it touches LDS), a suffix scan of
-// the bins by one wave, and the digit whose bin straddles P.  The top_k-th largest mass comes from the same descent on
-// token counts instead of masses.
+// the bins by one wave, and the digit whose bin straddles P.  The top_k-th largest scaled logit comes from the same
+// descent on token counts over an order-preserving integer image of the floats, BEFORE the exp: only the kept tokens
+// (some 50 of 32000) then pay for it.
 #include "mmf_common.h"
 
 namespace {
@@ -132,6 +133,8 @@ __global__ __launch_bounds__(kSampThreads) void sample_top_p_kernel(SampleArgs a
     __shared__ u64 sel[2];
     __shared__ float wmax[kSampWaves];
     __shared__ int wcand[kSampWaves];
+    __shared__ int few_n, few_i[64];
+    __shared__ unsigned few_m[64];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int V = a.V;
     const T* row = static_cast<const T*>(a.logits) + (int64_t)blockIdx.x * a.ld;
@@ -166,15 +169,77 @@ __global__ __launch_bounds__(kSampThreads) void sample_top_p_kernel(SampleArgs a
     for (int w = 0; w < kSampWaves; ++w) mx = fmaxf(mx, wmax[w]);
 
     unsigned m[NPT];
-#pragma unroll
-    for (int j = 0; j < NPT; ++j) {
-        const float p = l[j] == mx ? 1.0f : mmf_exp(__fsub_rn(l[j], mx));
-        m[j] = base + j < V ? (unsigned)__fmul_rn(p, 2147483648.0f) : 0u;
-    }
     if (a.top_k > 0 && a.top_k < V) {
-        const unsigned kth = samp_descent<true, NPT>(m, (u64)a.top_k, hist, hsum, sel);
+        // order-preserving image of the scaled logits: non-negative floats above the negative ones, -inf and the slots
+        // past V at 0 (which the descent ignores)
 #pragma unroll
-        for (int j = 0; j < NPT; ++j) m[j] = m[j] >= kth ? m[j] : 0u;
+        for (int j = 0; j < NPT; ++j) {
+            const unsigned b = __float_as_uint(__fadd_rn(l[j], 0.0f));       // -0 counts as +0, as the comparison of floats does
+            m[j] = l[j] == -INFINITY ? 0u : (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+        }
+        const unsigned kth = samp_descent<true, NPT>(m, (u64)a.top_k, hist, hsum, sel);
+        // the kept tokens (top_k of them, more on ties) with their masses, in any order, for one wave to finish
+        if (t == 0) few_n = 0;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < NPT; ++j) {
+            const bool keep = m[j] != 0u && m[j] >= kth;
+            float p = 0.0f;
+            if (__builtin_amdgcn_ballot_w64(keep) != 0) {         // wave-uniform: most waves skip the exp for most slots
+                p = l[j] == mx ? 1.0f : mmf_exp(__fsub_rn(l[j], mx));
+                p = keep ? p : 0.0f;
+            }
+            m[j] = (unsigned)__fmul_rn(p, 2147483648.0f);
+            if (keep) {
+                const int pos = atomicAdd(&few_n, 1);
+                if (pos < 64) { few_m[pos] = m[j]; few_i[pos] = base + j; }
+            }
+        }
+        __syncthreads();
+        const int n = few_n;
+        if (n <= 64) {
+            // Few enough for one lane each: the nucleus and the draw by direct comparison (64 x 64), same rule as below.
+            if (wave == 0) {
+                const unsigned mi = lane < n ? few_m[lane] : 0u;
+                const int ii = lane < n ? few_i[lane] : 0x7fffffff;
+                u64 Zf = mi;
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) Zf += samp_shfl_down(Zf, o);
+                Zf = ((u64)(unsigned)__builtin_amdgcn_readfirstlane((int)(Zf >> 32)) << 32) | (unsigned)__builtin_amdgcn_readfirstlane((int)Zf);
+                u64 Pf = (u64)((double)a.top_p * (double)Zf);
+                if (Pf < 1) Pf = 1;
+                u64 heavier = 0;
+#pragma unroll
+                for (int j = 0; j < 64; ++j) {
+                    const unsigned mj = (unsigned)__builtin_amdgcn_readlane((int)mi, j);
+                    heavier += mj > mi ? mj : 0u;
+                }
+                const unsigned kept = (mi != 0u && heavier < Pf) ? mi : 0u;
+                u64 Sf = kept;
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) Sf += samp_shfl_down(Sf, o);
+                Sf = ((u64)(unsigned)__builtin_amdgcn_readfirstlane((int)(Sf >> 32)) << 32) | (unsigned)__builtin_amdgcn_readfirstlane((int)Sf);
+                float uf = a.u[blockIdx.x];
+                uf = uf >= 0.0f ? uf : 0.0f;
+                u64 target = (u64)((double)uf * (double)Sf);
+                if (target >= Sf) target = Sf - 1;
+                u64 before = 0;                                   // kept mass at lower vocabulary indices
+#pragma unroll
+                for (int j = 0; j < 64; ++j) {
+                    const unsigned kj = (unsigned)__builtin_amdgcn_readlane((int)kept, j);
+                    const int ij = __builtin_amdgcn_readlane(ii, j);
+                    before += ij < ii ? kj : 0u;
+                }
+                if (kept != 0u && before <= target && target < before + kept) a.out[blockIdx.x] = ii;
+            }
+            return;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < NPT; ++j) {
+            const float p = l[j] == mx ? 1.0f : mmf_exp(__fsub_rn(l[j], mx));
+            m[j] = base + j < V ? (unsigned)__fmul_rn(p, 2147483648.0f) : 0u;
+        }
     }
     u64 zs = 0;
 #pragma unroll

@@ -22,22 +22,18 @@ from .detmath import det_exp
 MASS_ONE = 2147483648.0          # 2^31
 
 
-def masses(logits, temperature):
-    """uint64 array [V]: trunc(p_i * 2^31), p_i = exp(l_i - max l) with the deterministic fp32 exp, l = logits / T."""
+def masses(logits, temperature, top_k=0):
+    """uint64 array [V]: trunc(p_i * 2^31), p_i = exp(l_i - max l) with the deterministic fp32 exp, l = logits / T;
+    top_k > 0: every l_i below the top_k-th largest becomes -inf first (equal values stay together)."""
     l = torch.as_tensor(logits).float() / torch.tensor(temperature, dtype=torch.float32)
     l = torch.where(torch.isnan(l), torch.full_like(l, float("-inf")), l)
+    if 0 < top_k < l.shape[0]:
+        kth = torch.sort(l).values[-top_k]
+        l = torch.where(l >= kth, l, torch.full_like(l, float("-inf")))
     mx = l.max()
     p = torch.where(l == mx, torch.ones_like(l), det_exp(l - mx))
     m = (p * torch.tensor(MASS_ONE, dtype=torch.float32)).to(torch.float64).floor()
     return m.numpy().astype(np.uint64)
-
-
-def top_k_spec(m, top_k):
-    """Masses with everything below the top_k-th largest mass set to 0 (equal masses stay together); 0: no limit."""
-    if top_k <= 0 or top_k >= m.shape[0]:
-        return m
-    kth = np.sort(m)[-top_k]
-    return np.where(m >= kth, m, np.uint64(0))
 
 
 def nucleus_spec(m, top_p):
@@ -56,7 +52,7 @@ def nucleus_spec(m, top_p):
 
 def sample_top_p_spec(logits, temperature, top_p, u, top_k=0):
     """One row: (token, keep mask, masses after the top-k limit).  u is the caller's uniform number in [0, 1) (fp32)."""
-    m = top_k_spec(masses(logits, temperature), top_k)
+    m = masses(logits, temperature, top_k)
     keep = nucleus_spec(m, top_p)
     cum = np.cumsum(np.where(keep, m.astype(np.int64), 0))
     s = int(cum[-1])

@@ -67,11 +67,11 @@ def test_top_k_then_nucleus_is_what_transformers_keeps(top_k, top_p):
         scores = TopPLogitsWarper(top_p=top_p)(None, TopKLogitsWarper(top_k=top_k)(None, scores))[0]
         hf_keep = torch.isfinite(scores).numpy()
         lit = S.nucleus_literal(lg, t, top_p, top_k)
-        m = S.top_k_spec(S.masses(lg, t), top_k)
+        m = S.masses(lg, t, top_k)
         spec = S.nucleus_spec(m, top_p)
         assert (lit == hf_keep).all()
         assert (spec == hf_keep).all()
-        assert int((m > 0).sum()) == top_k
+        assert int((m > 0).sum()) <= top_k          # a kept token far below the maximum may still round to mass 0
         limited += int(hf_keep.sum() < S.nucleus_literal(lg, t, top_p).sum())
     assert limited > 0 or top_k >= 300, "no case where the top-k limit bites: the test would not see it dropped"
 
