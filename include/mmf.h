@@ -288,6 +288,30 @@ int mmf_cross_entropy_train_bwd(const void* logits, int64_t ld, const int64_t* l
                                 const float* dloss, float smoothing, float logit_scale, float lse_square_scale, void* dlogits,
                                 int64_t ldd, int64_t rows, int64_t V, int dtype, void* stream);
 
+/* ---- ShortConvolution (mmfreelm/modules/convolution.py:45-162) -------------------------------
+ * The causal depthwise convolution of kernel size W (<= mmf_short_conv_max_kernel_size() = 8, else MMF_ERR_WIDE) with an
+ * optional SiLU (activation = 1) that HGRNBitAttention(use_short_conv=True) puts in front of its projections.
+ * x, y: [B, T, D] contiguous; weight: [D, W] (nn.Conv1d's [D, 1, W]); bias: [D] or NULL; all in `dtype`.
+ *   pre[b, t, d] = T( sum_{w, t-(W-1)+w >= 0} weight[d, w] * x[b, t-(W-1)+w, d]  (+ bias[d]) ),   fp32 sum, oldest input first
+ *   y = T( pre / (1 + exp(-pre)) )  or  pre
+ * mmf_short_conv_fwd replaces ShortConvolution.forward for whole sequences (:98-131; causal_conv1d_fn or
+ *   nn.Conv1d + activation there); cache ([B, D, W], `dtype`) may be NULL, else it receives the last W inputs of every
+ *   channel, oldest first, zero filled when T < W (the state a following step continues from).
+ * mmf_short_conv_step replaces ShortConvolution.step (:133-158; causal_conv1d_update there): x, y [B, D]; the cache drops
+ *   its oldest entry, takes x, and y is the same sum over it.
+ * mmf_short_conv_bwd: gradients of the whole-sequence form.  dpre: [B, T, D] fp32 scratch; partial:
+ *   [mmf_short_conv_bwd_groups(B * T), (W + 1) * D] fp32 scratch; dweight_bias: [(W + 1) * D] fp32, entry w * D + d =
+ *   dweight[d, w], the last D entries = dbias. */
+int mmf_short_conv_max_kernel_size(void);
+int mmf_short_conv_fwd(const void* x, const void* weight, const void* bias, void* y, void* cache, int64_t B, int64_t T,
+                       int64_t D, int W, int activation, int dtype, void* stream);
+int mmf_short_conv_step(const void* x, const void* weight, const void* bias, void* cache, void* y, int64_t B, int64_t D,
+                        int W, int activation, int dtype, void* stream);
+int mmf_short_conv_bwd_groups(int64_t rows);
+int mmf_short_conv_bwd(const void* x, const void* weight, const void* bias, const void* dy, void* dx, float* dpre,
+                       float* partial, float* dweight_bias, int64_t B, int64_t T, int64_t D, int W, int activation,
+                       int dtype, void* stream);
+
 /* ---- top-p (nucleus) sampling of the next token -----------------------------------------------
  * mmf_sample_top_p replaces, per decoded token of the loop that mmfreelm's generate.py:11 runs
  *   (model.generate(do_sample=True, top_p=0.4, temperature=0.6)), what transformers' sampling path does with the

@@ -14,10 +14,12 @@ Name map (reference module -> here):
     mmfreelm.layers.hgrn_bit      HGRNBitAttention                         -> .attention
     mmfreelm.models.hgrn_bit      HGRNBitConfig, HGRNBitModel, HGRNBitForCausalLM -> .modeling_hgrn_bit
     mmfreelm.models.utils         RecurrentCache                           -> .cache
+    mmfreelm.modules.convolution  ShortConvolution                         -> .convolution
 """
 from .activations import swiglu
 from .bitlinear import (BitLinear, FusedBitLinear, activation_quant, layer_norm_linear_quant_fn, weight_quant)
 from .cache import RecurrentCache
+from .convolution import ShortConvolution
 from .fused_norm_gate import FusedRMSNormSwishGate
 from .hgrn import chunk_hgrn, fused_recurrent_hgrn
 from .layernorm import RMSNorm, rms_norm_fn
@@ -30,7 +32,7 @@ _LAZY = {"HGRNBitAttention": ".attention", "HGRNBitConfig": ".configuration_hgrn
          "save_packed": ".checkpoint", "load_packed": ".checkpoint", "load_pretrained": ".checkpoint", "pack_all": ".checkpoint"}
 
 __all__ = ["swiglu", "BitLinear", "FusedBitLinear", "activation_quant", "weight_quant", "layer_norm_linear_quant_fn",
-           "RecurrentCache", "FusedRMSNormSwishGate", "chunk_hgrn", "fused_recurrent_hgrn", "RMSNorm", "rms_norm_fn",
+           "RecurrentCache", "ShortConvolution", "FusedRMSNormSwishGate", "chunk_hgrn", "fused_recurrent_hgrn", "RMSNorm", "rms_norm_fn",
            *_LAZY]
 
 _registered = False

@@ -64,6 +64,11 @@ SIGNATURES = {
     "mmf_hgrn_recurrent_bwd": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i32, _i32, _ptr]),
     "mmf_cross_entropy_train_fwd": (_i32, [_ptr, _i64, _ptr, _i64, _f32, _f32, _f32, _ptr, _ptr, _ptr, _i64, _i64, _i32, _ptr]),
     "mmf_cross_entropy_train_bwd": (_i32, [_ptr, _i64, _ptr, _i64, _ptr, _ptr, _f32, _f32, _f32, _ptr, _i64, _i64, _i64, _i32, _ptr]),
+    "mmf_short_conv_max_kernel_size": (_i32, []),
+    "mmf_short_conv_fwd": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i32, _i32, _i32, _ptr]),
+    "mmf_short_conv_step": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i32, _i32, _i32, _ptr]),
+    "mmf_short_conv_bwd_groups": (_i32, [_i64]),
+    "mmf_short_conv_bwd": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i32, _i32, _i32, _ptr]),
     "mmf_sample_top_p_max_vocab": (_i64, []),
     "mmf_sample_top_p": (_i32, [_ptr, _i64, _i64, _i64, _f32, _f32, _i64, _ptr, _ptr, _i32, _ptr]),
 }

@@ -43,14 +43,22 @@ class HGRNBitAttention(nn.Module):
 
         assert mode in ["fused_recurrent", "chunk"], f"Not supported mode `{mode}`."
         assert self.hidden_size % num_heads == 0, f"hidden size must be divisible by num_heads of {num_heads}"
-        if use_short_conv:
-            # The reference's call site for the convolution is broken (three positionals into a
-            # two-argument forward, mmfreelm/layers/hgrn_bit.py:101) and the option defaults to off.
-            raise NotImplementedError("use_short_conv=True is not supported")
 
         self.i_proj = BitLinear(hidden_size, self.input_dim, bias=False)
         self.f_proj = BitLinear(hidden_size, self.input_dim, bias=False)
         self.g_proj = BitLinear(hidden_size, self.input_dim, bias=False)
+        if use_short_conv:
+            # mmfreelm/layers/hgrn_bit.py:60-67.  The reference's forward cannot run with this option (it hands
+            # ShortConvolution.forward(x, cache) three positionals, :101/:107-108); here the evident intent runs:
+            # conv(x, conv_state).  States of a layer: (conv_state, recurrent_state) with a shared kernel, else
+            # (conv_state_i, conv_state_f, recurrent_state) - the tuples the reference's forward writes back (:131-134).
+            from .convolution import ShortConvolution
+            if share_conv_kernel:
+                self.h_conv1d = ShortConvolution(hidden_size, conv_size, activation="silu")
+            else:
+                self.q_conv1d = ShortConvolution(self.input_dim, conv_size, activation="silu")
+                self.f_conv1d = ShortConvolution(self.input_dim, conv_size, activation="silu")
+                self.i_conv1d = ShortConvolution(self.input_dim, conv_size, activation="silu")
         self.g_norm = FusedRMSNormSwishGate(self.input_dim, layernorm_eps)
         self.o_proj = BitLinear(self.input_dim, hidden_size, bias=False)
         self.apply(self._initialize_weights)
@@ -87,6 +95,8 @@ class HGRNBitAttention(nn.Module):
         stacked i/f/g projection instead of running as a launch of its own."""
         B, T, _ = hidden_states.shape
         D = self.input_dim
+        if self.use_short_conv:
+            return self._forward_short_conv(hidden_states, attention_mask, past_key_values, use_cache, lower_bound, input_norm)
         if self.training and torch.is_grad_enabled():
             return self._forward_train(hidden_states, attention_mask, lower_bound, input_norm), None, past_key_values
         last_state = past_key_values[self.layer_idx] if use_cache else None
@@ -144,10 +154,58 @@ class HGRNBitAttention(nn.Module):
         o = self.g_norm(g, o.view(B, T, D))
         return self.o_proj(o)
 
+    def _forward_short_conv(self, hidden_states, attention_mask, past_key_values, use_cache, lower_bound, input_norm):
+        """The layer with the short convolutions in front of the projections (mmfreelm/layers/hgrn_bit.py:97-139), one
+        launch per op (no folding), differentiable; see __init__ for how it departs from the reference's call."""
+        from .autograd import HGRNGateFn, needs_grad
+        from .hgrn import fused_recurrent_hgrn
+        B, T, _ = hidden_states.shape
+        D = self.input_dim
+        if input_norm is not None:
+            hidden_states = input_norm(hidden_states)
+        last_state = past_key_values[self.layer_idx] if use_cache else None
+        if self.share_conv_kernel:
+            conv_state = last_state[0] if use_cache else None
+            hidden_states = self.h_conv1d(hidden_states, conv_state)          # the conv state is updated in place
+            i, f = self.i_proj(hidden_states), self.f_proj(hidden_states)
+        else:
+            conv_state_i = last_state[0] if use_cache else None
+            conv_state_f = last_state[1] if use_cache else None
+            i = self.i_conv1d(self.i_proj(hidden_states), conv_state_i)
+            f = self.f_conv1d(self.f_proj(hidden_states), conv_state_f)
+        lb = lower_bound if (lower_bound is not None and self.layer_idx > 0) else None
+        if needs_grad(i, f, lb):
+            x_in, gate = HGRNGateFn.apply(i, f, lb, attention_mask)
+        else:
+            x_in, gate = F_.hgrn_gate(i, f, lb, attention_mask)
+        recurrent_state = last_state[-1] if use_cache else None
+        h0 = recurrent_state.reshape(B, 1, D) if recurrent_state is not None else None
+        o, new_state = fused_recurrent_hgrn(x_in.view(B, 1, T, D), gate.view(B, 1, T, D), initial_state=h0,
+                                            output_final_state=bool(use_cache))
+        if past_key_values is not None and use_cache:
+            recurrent_state = new_state.view(B, self.num_heads, self.head_dim)
+            state = (conv_state, recurrent_state) if self.share_conv_kernel else (conv_state_i, conv_state_f, recurrent_state)
+            past_key_values.update(state, self.layer_idx, T)
+        o = self.g_norm(self.g_proj(hidden_states), o.view(B, T, D))
+        return self.o_proj(o), None, past_key_values
+
     def init_state(self, batch_size: int) -> Tuple[torch.Tensor]:
-        """Zero recurrent state [B, num_heads, head_dim], kept in fp32."""
+        """Zero states of one layer: the recurrent state [B, num_heads, head_dim] in fp32, behind the convolution
+        caches [B, channels, conv_size] (activation dtype) when use_short_conv."""
         device = self.g_norm.weight.device       # the projections' latent weights may be absent (packed checkpoints)
-        return (torch.zeros(batch_size, self.num_heads, self.head_dim, dtype=torch.float32, device=device),)
+        state = tuple()
+        if self.use_short_conv:
+            dt = self.g_norm.weight.dtype
+            if self.share_conv_kernel:
+                state += (torch.zeros(batch_size, self.hidden_size, self.conv_size, dtype=dt, device=device),)
+            else:
+                state += (torch.zeros(batch_size, self.input_dim, self.conv_size, dtype=dt, device=device),
+                          torch.zeros(batch_size, self.input_dim, self.conv_size, dtype=dt, device=device))
+        return state + (torch.zeros(batch_size, self.num_heads, self.head_dim, dtype=torch.float32, device=device),)
 
     def state_size(self, **kwargs) -> int:
-        return self.hidden_size
+        state_size = self.hidden_size
+        for module in self.children():
+            if hasattr(module, "state_size") and isinstance(module, nn.Conv1d):
+                state_size += module.state_size
+        return state_size

@@ -309,3 +309,23 @@ class FusedCrossEntropyLoss(torch.nn.Module):
         elif self.reduction == "sum":
             loss, z_loss = loss.sum(), z_loss.sum()
         return (loss, z_loss) if self.return_z_loss else loss
+
+
+class ShortConvFn(torch.autograd.Function):
+    """ShortConvolution.forward over whole sequences (mmfreelm/modules/convolution.py:98-131) as one differentiable op."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, activation):
+        with torch.no_grad():
+            y = F_.short_conv(x, weight, bias, activation)
+        ctx.save_for_backward(x, weight, bias)
+        ctx.activation = activation
+        return y
+
+    @staticmethod
+    def backward(ctx, g):
+        x, weight, bias = ctx.saved_tensors
+        dx, dw, db = F_.short_conv_bwd(x, weight, bias, g, ctx.activation)
+        dweight = dw.reshape(weight.shape).to(weight.dtype) if ctx.needs_input_grad[1] else None
+        dbias = db.to(bias.dtype) if (bias is not None and ctx.needs_input_grad[2]) else None
+        return dx, dweight, dbias, None

@@ -11,7 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBPATH = os.path.join(LIBDIR, "libmmf_hip.so")
-SOURCES = ["norm.hip", "quant_pack.hip", "bitlinear_gemv.hip", "bitlinear_mfma.hip", "hgrn.hip", "misc.hip", "decode_layers.hip", "sampling.hip", "loss.hip", "backward.hip"]
+SOURCES = ["norm.hip", "quant_pack.hip", "bitlinear_gemv.hip", "bitlinear_mfma.hip", "hgrn.hip", "misc.hip", "decode_layers.hip", "sampling.hip", "loss.hip", "backward.hip", "conv.hip"]
 
 # -ffp-contract=off: no multiply-add fusion, so results match a CPU restatement bit for bit.
 # packed-fp32-ops disabled: keep the compiler from forming v_pk_*_f32.

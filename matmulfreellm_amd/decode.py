@@ -48,6 +48,9 @@ class DecodeEngine:
 
     def __init__(self, model, batch_size: int, use_graph: bool = True, fuse: bool = True, resident: Optional[bool] = None):
         cfg = model.config
+        if getattr(cfg, "use_short_conv", False):
+            raise NotImplementedError("DecodeEngine has no convolution state: models with use_short_conv decode through "
+                                      "the module path (generate() does so by itself)")
         self.lib = L.load()
         self.model = model
         self.B = B = batch_size

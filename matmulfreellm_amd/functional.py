@@ -590,3 +590,66 @@ def cross_entropy(logits, labels, ignore_index=-100):
                                           l2.shape[0], v, L.dtype_id(l2.dtype), L.stream()), "mmf_cross_entropy_fwd")
     counted = ((lab != ignore_index) & (lab >= 0) & (lab < v)).sum()
     return rows.sum() / counted
+
+
+# ------------------------------------------------------------------------------ ShortConvolution
+def _conv_args(x, weight, bias):
+    dev = L.require_gpu(x, weight, bias)
+    if x.dim() != 3:
+        raise ValueError("x must be [batch, seq_len, hidden_size]")
+    d = x.shape[-1]
+    w2 = weight.detach().reshape(weight.shape[0], -1).to(x.dtype).contiguous()       # nn.Conv1d keeps [D, 1, W]
+    if w2.shape[0] != d:
+        raise ValueError(f"convolution has {w2.shape[0]} channels, the input {d}")
+    b1 = bias.detach().to(x.dtype).contiguous() if bias is not None else None
+    return dev, w2, b1
+
+
+def short_conv(x, weight, bias=None, activation=True, cache=None):
+    """Causal depthwise convolution (+ SiLU) of x [B, T, D] with weight [D, 1, W] / [D, W]; cache [B, D, W] (x.dtype,
+    contiguous), when given, receives the last W inputs."""
+    lib = L.load()
+    dev, w2, b1 = _conv_args(x, weight, bias)
+    b, t, d = x.shape
+    xc = x.contiguous()
+    y = torch.empty_like(xc)
+    if cache is not None and not (cache.shape == (b, d, w2.shape[1]) and cache.dtype == x.dtype and cache.is_contiguous()
+                                  and cache.device == dev):
+        raise L.MMFError(f"short_conv: the cache must be a contiguous [{b}, {d}, {w2.shape[1]}] {x.dtype} tensor on {dev}")
+    with torch.cuda.device(dev):
+        L.check(lib.mmf_short_conv_fwd(xc.data_ptr(), w2.data_ptr(), L.ptr(b1), y.data_ptr(), L.ptr(cache), b, t, d, w2.shape[1],
+                                       1 if activation else 0, L.dtype_id(x.dtype), L.stream()), "mmf_short_conv_fwd")
+    return y
+
+
+def short_conv_step(x, weight, bias, cache, activation=True):
+    """One token: x [B, D]; the cache [B, D, W] is updated in place; returns y [B, D]."""
+    lib = L.load()
+    dev, w2, b1 = _conv_args(x.unsqueeze(1), weight, bias)
+    b, d = x.shape
+    if not (cache.shape == (b, d, w2.shape[1]) and cache.dtype == x.dtype and cache.is_contiguous() and cache.device == dev):
+        raise L.MMFError(f"short_conv_step: the cache must be a contiguous [{b}, {d}, {w2.shape[1]}] {x.dtype} tensor on {dev}")
+    xc = x.contiguous()
+    y = torch.empty_like(xc)
+    with torch.cuda.device(dev):
+        L.check(lib.mmf_short_conv_step(xc.data_ptr(), w2.data_ptr(), L.ptr(b1), cache.data_ptr(), y.data_ptr(), b, d, w2.shape[1],
+                                        1 if activation else 0, L.dtype_id(x.dtype), L.stream()), "mmf_short_conv_step")
+    return y
+
+
+def short_conv_bwd(x, weight, bias, dy, activation=True):
+    """Gradients of short_conv: (dx [B, T, D] x.dtype, dweight [D, W] fp32, dbias [D] fp32)."""
+    lib = L.load()
+    dev, w2, b1 = _conv_args(x, weight, bias)
+    b, t, d = x.shape
+    w = w2.shape[1]
+    xc, dyc = x.contiguous(), dy.contiguous()
+    dx = torch.empty_like(xc)
+    dpre = torch.empty(b, t, d, dtype=torch.float32, device=dev)
+    part = torch.empty(lib.mmf_short_conv_bwd_groups(b * t), (w + 1) * d, dtype=torch.float32, device=dev)
+    dwb = torch.empty((w + 1) * d, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        L.check(lib.mmf_short_conv_bwd(xc.data_ptr(), w2.data_ptr(), L.ptr(b1), dyc.data_ptr(), dx.data_ptr(), dpre.data_ptr(),
+                                       part.data_ptr(), dwb.data_ptr(), b, t, d, w, 1 if activation else 0, L.dtype_id(x.dtype),
+                                       L.stream()), "mmf_short_conv_bwd")
+    return dx, dwb[:w * d].view(w, d).t(), dwb[w * d:]

@@ -404,7 +404,7 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
         tokens = [input_ids]
         finished = torch.zeros(B, dtype=torch.bool, device=input_ids.device)
         engine = None
-        if use_graph and max_new_tokens > 1:
+        if use_graph and max_new_tokens > 1 and not self.config.use_short_conv:   # the graph engine has no convolution state
             from .decode import DecodeEngine
             engine = DecodeEngine.for_model(self, B, resident=resident)
             engine.load_state([c[-1] for c in cache])

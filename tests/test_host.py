@@ -102,8 +102,9 @@ def test_layer_norm_linear_quant_fn_rejects_unsupported_forms():
         mm.layer_norm_linear_quant_fn(x, torch.ones(64), None, w, None, is_rms_norm=False)
     with pytest.raises(NotImplementedError):           # a norm bias exists for the LayerNorm form only
         mm.layer_norm_linear_quant_fn(x, torch.ones(64), torch.zeros(64), w, None, is_rms_norm=True)
-    with pytest.raises(NotImplementedError):
-        mm.HGRNBitAttention(hidden_size=64, num_heads=1, use_short_conv=True)
+    attn = mm.HGRNBitAttention(hidden_size=64, num_heads=1, use_short_conv=True, share_conv_kernel=False)
+    assert isinstance(attn.i_conv1d, mm.ShortConvolution) and attn.state_size() == 64 + 3 * 64 * 4
+    assert [tuple(s.shape) for s in attn.init_state(2)] == [(2, 64, 4), (2, 64, 4), (2, 1, 64)]
 
 
 def test_division_free_quotient_is_the_correctly_rounded_one():
