@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kBT) void rmsnorm_bwd_kernel(NormBwdArgs a) {
                 dv[v][i] = in ? dv[v][i] : 0.0f;
                 if constexpr (MODE == BWD_GATED) gv[v][i] = in ? gv[v][i] : 0.0f;
                 rv[v][i] = (dr && in) ? rv[v][i] : 0.0f;
-                ss += (double)xv[v][i] * (double)xv[v][i];
+                ss = mmf_add_square(ss, xv[v][i]);
             }
         }
         ss = mmf_block_sum<kBT / 64>(ss, red_d);

@@ -180,7 +180,7 @@ __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
 #pragma unroll
         for (int v = 0; v < NV; ++v)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) s1 += (double)xv[v][i] * (double)xv[v][i];
+            for (int i = 0; i < 4; ++i) s1 = mmf_add_square(s1, xv[v][i]);
         s1 = mmf_block_sum_once<kGemvWaves>(s1, red_a);
         const float rstd1 = mmf_rstd(s1, K, a.inv_K, a.eps1);
 #pragma unroll
@@ -214,7 +214,7 @@ __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
 #pragma unroll
     for (int v = 0; v < NV; ++v)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
+        for (int i = 0; i < 4; ++i) ss = mmf_add_square(ss, xv[v][i]);
     ss = mmf_block_sum_once<kGemvWaves>(ss, red_b);
     const float rstd = mmf_rstd(ss, K, a.inv_K, a.eps);
     float amax = 0.0f;

@@ -311,7 +311,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
 #pragma unroll
         for (int v = 0; v < NV; ++v)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) s1 += (double)xv[v][i] * (double)xv[v][i];
+            for (int i = 0; i < 4; ++i) s1 = mmf_add_square(s1, xv[v][i]);
         s1 = mmf_block_sum_once<kNW>(s1, sm.red_a);
         const float rstd1 = mmf_rstd(s1, K, ph.inv_K, ph.eps1);
 #pragma unroll
@@ -334,7 +334,7 @@ __device__ __forceinline__ void run_phase(const Phase& ph, const LayersArgs& a, 
 #pragma unroll
     for (int v = 0; v < NV; ++v)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
+        for (int i = 0; i < 4; ++i) ss = mmf_add_square(ss, xv[v][i]);
     ss = mmf_block_sum_once<kNW>(ss, sm.red_b);
     MMF_STAMP(3);
     const float rstd = mmf_rstd(ss, K, ph.inv_K, ph.eps);

@@ -352,6 +352,12 @@ __device__ __forceinline__ float mmf_block_max_once(float v, float* slot) {
 // inv_K = RN(1 / K) from the host, q0 = sumsq * inv_K is within two ulps, one residual step
 // makes it faithful, and a second one (r exact through the fused multiply-add) lands on the
 // correctly rounded quotient (Markstein's theorem; K is a small integer, 0 <= sumsq < 2^200).
+// s + v * v in fp64.  The square of an fp32 value is exact in fp64 (48 significant bits), so the fused multiply-add rounds
+// exactly what the separate multiply and add would: same result, one fp64 operation instead of two.
+__device__ __forceinline__ double mmf_add_square(double s, float v) {
+    const double d = (double)v;
+    return __builtin_fma(d, d, s);
+}
 __device__ __forceinline__ double mmf_quotient_by_count(double sum, int64_t K, double inv_K) {
     const double Kd = (double)K;
     double q = sum * inv_K;

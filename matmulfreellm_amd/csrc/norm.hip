@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kThreads) void row_kernel(RowArgs a) {
             }
             if (res_out) mmf_store8<TR>(res_out, k0, K, vec_ok, xv[v]);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
+            for (int i = 0; i < 8; ++i) ss = mmf_add_square(ss, xv[v][i]);
         } else {
 #pragma unroll
             for (int i = 0; i < 8; ++i) xv[v][i] = 0.0f;
@@ -98,7 +98,7 @@ __global__ __launch_bounds__(kThreads) void row_kernel(RowArgs a) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 xv[v][i] = k0 + i < K ? __fsub_rn(xv[v][i], mean) : 0.0f;
-                ss += (double)xv[v][i] * (double)xv[v][i];
+                ss = mmf_add_square(ss, xv[v][i]);
             }
         }
     }
@@ -326,7 +326,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
 #pragma unroll
         for (int v = 0; v < NV; ++v)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) s1 += (double)xv[v][i] * (double)xv[v][i];
+            for (int i = 0; i < 4; ++i) s1 = mmf_add_square(s1, xv[v][i]);
         s1 = mmf_wave_sum(s1);
         if constexpr (WPR > 1) {
             if ((threadIdx.x & 63) == 0) red_a[wave] = s1;
@@ -365,7 +365,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
 #pragma unroll
     for (int v = 0; v < NV; ++v)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ss += (double)xv[v][i] * (double)xv[v][i];
+        for (int i = 0; i < 4; ++i) ss = mmf_add_square(ss, xv[v][i]);
     ss = mmf_wave_sum(ss);
     if constexpr (WPR > 1) {
         if ((threadIdx.x & 63) == 0) red_b[wave] = ss;
