@@ -254,6 +254,8 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
     const bool live = row_raw < a.M;                            // rows past M compute on row M-1 and store nothing
     const int64_t row = live ? row_raw : a.M - 1;
     const int K = (int)a.K, Kp = (int)a.Kp;
+    // element k0 + i of the row exists; with vector accesses (K a multiple of 4) a thread's 4 elements stand or fall together
+    auto inb = [&](int k0, int i) { return VEC ? k0 < K : k0 + i < K; };
     const T* x = static_cast<const T*>(a.x) + row * a.ldx;
     const T* aux = static_cast<const T*>(a.aux) + row * a.ldaux;
     const T* aux2 = static_cast<const T*>(a.aux2) + row * a.ldaux2;
@@ -286,14 +288,14 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
         if constexpr (HAS_AUX) raw4_unpack<T>(araw[v], av[v]);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            if (k0 + i >= K) xv[v][i] = 0.0f;
+            if (!inb(k0, i)) xv[v][i] = 0.0f;
     }
     if constexpr (PRO == QPRO_RESNORM) {
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int k0 = (v * TPR + tr) * 4;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) xv[v][i] = k0 + i < K ? __fadd_rn(xv[v][i], av[v][i]) : 0.0f;
+            for (int i = 0; i < 4; ++i) xv[v][i] = inb(k0, i) ? __fadd_rn(xv[v][i], av[v][i]) : 0.0f;
             if (a.res_out && live) raw4_store<T, VEC>(static_cast<T*>(a.res_out) + row * K, k0, K, xv[v]);
         }
     }
@@ -316,7 +318,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
                 const float h = __fadd_rn(__fmul_rn(go, stv[i]), xo);
                 stv[i] = h;
                 av[v][i] = mmf_round_to<T>(h);          // o, the swish gate of the gated norm
-                xv[v][i] = k0 + i < K ? gv[i] : 0.0f;   // the gated norm normalises the g projection
+                xv[v][i] = inb(k0, i) ? gv[i] : 0.0f;   // the gated norm normalises the g projection
             }
             if (live) raw4_store<float, VEC>(st, k0, K, stv);
         }
@@ -345,7 +347,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
             for (int i = 0; i < 4; ++i) {
                 float y = __fmul_rn(__fmul_rn(xv[v][i], rstd1), w1v[i]);
                 if constexpr (STEP || PRO == QPRO_GATEDNORM) y = __fmul_rn(__fmul_rn(y, av[v][i]), mmf_sigmoid(av[v][i]));
-                xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(y) : 0.0f;
+                xv[v][i] = inb(k0, i) ? mmf_round_to<T>(y) : 0.0f;
             }
         }
     } else if constexpr (PRO == QPRO_SWIGLU) {
@@ -356,7 +358,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
             for (int i = 0; i < 4; ++i) {
                 const float g = xv[v][i];
                 const float z = __fdiv_rn(__fmul_rn(g, av[v][i]), __fadd_rn(1.0f, mmf_exp(-g)));
-                xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(z) : 0.0f;
+                xv[v][i] = inb(k0, i) ? mmf_round_to<T>(z) : 0.0f;
             }
         }
     }
@@ -405,7 +407,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
             uint32_t packed4 = 0;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int c = (k0 + i < K) ? mmf_code(xv[v][i], scale) : 0;
+                const int c = inb(k0, i) ? mmf_code(xv[v][i], scale) : 0;
                 qs += c;
                 packed4 |= (uint32_t)(c & 0xff) << (8 * i);
             }
