@@ -175,19 +175,6 @@ int mmf_bitlinear_mfma_swiglu(const int8_t* codes_tiled, const float* deq, const
                               const float* wdeq, int64_t seg_rows, void* out, int64_t ldo, int64_t M, int64_t K, int64_t N,
                               int out_dtype, void* stream);
 
-/* Measuring aids of the tiled contraction (no counterpart in the reference; bench.py's mfma leg uses them).
- * mmf_bitlinear_mfma_clock_sink: sink = [workgroups][2] int64 on the device, or NULL to switch off.  While set, thread 0
- *   of each of the first `workgroups` workgroups of every later tiled launch (mmf_bitlinear_mfma with M > 64,
- *   mmf_bitlinear_mfma_swiglu) stores the shader-clock ticks (s_memtime) and the 100 MHz ticks (s_memrealtime) it
- *   spent in the kernel: their ratio is the clock the part sustained under that kernel.  Process-wide, not
- *   thread-safe; the buffer must outlive the launches.
- * mmf_mfma_pipe_probe: `workgroups` x 8 waves each issue steps x 4 independent v_mfma_i32_32x32x32_i8 on register
- *   operands (the tiled kernel's inner step with every load, barrier and LDS read taken away) and store the same two
- *   tick counts; clocks = [workgroups][2] int64 plus one spare int64.  random_operands != 0: per-lane random int8 codes
- *   and ternary weights (the switching activity, hence the power draw, of real operands) instead of constant ones. */
-int mmf_bitlinear_mfma_clock_sink(int64_t* sink, int64_t workgroups);
-int mmf_mfma_pipe_probe(int64_t steps, int64_t workgroups, int random_operands, int64_t* clocks, void* stream);
-
 /* ---- HGRN recurrence ------------------------------------------------------------------
  * x, g, o: [BH, T, D] contiguous (BH = batch * heads); h0 / ht: [BH, D] fp32 or NULL.
  * mmf_hgrn_recurrent replaces fused_recurrent_hgrn, mmfreelm/ops/hgrn/recurrent_fuse.py:
@@ -333,7 +320,7 @@ int64_t mmf_sample_top_p_max_vocab(void);
 int mmf_sample_top_p(const void* logits, int64_t ld, int64_t rows, int64_t V, float temperature, float top_p,
                      int64_t top_k, const float* u, int64_t* out, int dtype, void* stream);
 
-/* ---- all layers of one batch-1 decode step in one persistent launch ---------------------------
+/* ---- one whole batch-1 decode step in one persistent launch ---------------------------------
  * mmf_decode_layers replaces, for one token, the loop over HGRNBitBlock.forward in HGRNBitModel.forward
  *   (mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py:236-262, the block at :97-109, the attention at
  *   mmfreelm/layers/hgrn_bit.py:83-162): embedding row of *tok -> n_layers x [block norm, i/f/g BitLinear, gate math +
@@ -341,30 +328,28 @@ int mmf_sample_top_p(const void* logits, int64_t ld, int64_t rows, int64_t V, fl
  *   residual] -> h_out [H] (the input of the final norm + lm_head).  Same arithmetic, operation for operation, as the
  *   chain of mmf_bitlinear_gemv_fused launches it stands for.
  *   256 workgroups stay resident and hand activations to each other as 32-bit words (16-bit value | 16-bit tag of the
- *   producing link), so the device must have at least 256 CUs free for the launch (fewer CUs: MMF_ERR_ARG).
+ *   producing link), each row kept in mmf_decode_layers_copies() copies (one per XCD), so the device must have at least
+ *   256 CUs free for the launch (fewer CUs: MMF_ERR_ARG).
  *   phases: device array of 4 * n_layers records of mmf_decode_layers_phase_bytes() bytes each, in the order i/f/g, o,
  *     gate, down: { const void* w1; const void* norm_w; const void* packed; const float* wdeq; const float* lower_bound;
  *     float* state; double inv_K; float eps; float eps1; int K; int N; int seg_rows; int pad; } (w1: weight of the norm
- *     in front of the BitLinear, null for down; norm weights in the activation dtype; inv_K = 1.0 / K).
- *   h0, h1 [H], o, g [D], attn, res [H], z [I]: uint32 scratch words, zero-initialised once, owned by the caller and
- *     reused by every call; epoch: one uint32, zero-initialised once, advanced by the kernel; err: one int, set to 1
- *     if a wait ran out of its `spin` polling rounds (results are then invalid; the launch still terminates).
+ *     in front of the BitLinear, null for down; norm weights in the activation dtype; inv_K = 1.0 / K; seg_rows = N for
+ *     one matrix, the rows of a segment for stacked ones).  The table must not change while the launch runs.
+ *   words: mmf_decode_layers_words(H, D, I) uint32 scratch words (16-byte aligned), zero-initialised once, owned by the
+ *     caller and reused by every call; epoch: one uint32, zero-initialised once, advanced by the kernel; err: one int,
+ *     set to 1 if a wait ran out of its `spin` polling rounds (results are then invalid; the launch still terminates).
  *   head: null, or a device record like the ones of `phases` for the final norm + lm_head (w1 = final norm weight,
  *     K = H, N = vocabulary size); the launch then also writes the logits [N] (activation dtype), and the greedy token
  *     (lowest index of the largest logit; NaNs never win) to *tok_out, which may be the buffer `tok` points to.
  *     am_words: 256 uint64 scratch words, zero-initialised once.  With head == null the three pointers are ignored.
- *   trace: null, or mmf_decode_layers_trace_words() int64 words (zeroed by the caller): thread 0 of workgroups 0, 37 and
- *     200 stores the shader clock at ten points of each of the first 128 links, [workgroup][link][12]: 0 link entered,
- *     1 input row arrived, 2 block norm applied, 3 sum of squares reduced, 4 rstd, 5 absmax reduced, 6 codes in LDS,
- *     7 dot products done, 8 partial sums met, 9 epilogue stored (a measuring aid; costs a few scalar branches).
- *   Requires D == H, H, I multiples of 128, H <= 4096, I <= 8192 (else MMF_ERR_WIDE), 16-bit activations (dtype 1 or 2), batch 1.
- *   Calls on one device must not overlap (they share the scratch words). */
+ *   Requires D == H, H, I multiples of 128, H <= 4096, I <= 8192 (else MMF_ERR_WIDE), 16-bit activations (dtype 1 or 2),
+ *   batch 1, norm weights of magnitude below 2^40.  Calls on one device must not overlap (they share the scratch words). */
 int mmf_decode_layers_phase_bytes(void);
-int mmf_decode_layers_trace_words(void);
-int mmf_decode_layers(const void* phases, int n_layers, const void* table, const int64_t* tok, int64_t vocab,
-                      uint32_t* h0, uint32_t* h1, uint32_t* o, uint32_t* g, uint32_t* attn, uint32_t* res, uint32_t* z,
+int mmf_decode_layers_copies(void);
+int64_t mmf_decode_layers_words(int H, int D, int I);
+int mmf_decode_layers(const void* phases, int n_layers, const void* table, const int64_t* tok, int64_t vocab, uint32_t* words,
                       void* h_out, const void* head, void* logits, uint64_t* am_words, int64_t* tok_out, uint32_t* epoch, int* err,
-                      int64_t* trace, int H, int D, int I, int spin, int dtype, void* stream);
+                      int H, int D, int I, int spin, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

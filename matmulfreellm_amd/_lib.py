@@ -19,7 +19,7 @@ _ERRORS = {-1: "MMF_ERR_ARG (bad shape, null pointer or unsupported dtype combin
 
 _i64, _i32, _f32, _ptr = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_void_p
 
-# name -> (restype, argtypes); must list every symbol include/mmf.h declares.
+# name -> (restype, argtypes); must list every symbol include/mmf.h and include/mmf_diag.h declare.
 SIGNATURES = {
     "mmf_packed_bytes": (_i64, [_i64, _i64]),
     "mmf_ternarize_workspace_bytes": (_i64, []),
@@ -36,9 +36,13 @@ SIGNATURES = {
     "mmf_rmsnorm_quant_fused": (_i32, [_i32, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _f32, _ptr, _f32, _ptr, _ptr, _ptr, _ptr,
                                        _ptr, _i64, _i64, _i32, _i32, _ptr]),
     "mmf_decode_layers_phase_bytes": (_i32, []),
+    "mmf_decode_layers_copies": (_i32, []),
+    "mmf_decode_layers_words": (_i64, [_i32, _i32, _i32]),
+    "mmf_decode_layers": (_i32, [_ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
+                                 _i32, _i32, _i32, _i32, _i32, _ptr]),
     "mmf_decode_layers_trace_words": (_i32, []),
-    "mmf_decode_layers": (_i32, [_ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
-                                 _ptr, _ptr, _ptr, _ptr, _i32, _i32, _i32, _i32, _i32, _ptr]),
+    "mmf_decode_layers_traced": (_i32, [_ptr, _i32, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
+                                        _i32, _i32, _i32, _i32, _i32, _i32, _ptr]),
     "mmf_bitlinear_gemv_max_k": (_i64, []),
     "mmf_bitlinear_gemv": (_i32, [_ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _i64, _i64, _i64, _f32, _i32, _i32, _ptr]),
     "mmf_bitlinear_gemv_fused": (_i32, [_i32, _i32, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _f32, _ptr, _f32, _ptr, _ptr, _i64, _ptr,

@@ -17,7 +17,8 @@
 // whatever -ffp-contract the translation unit is built with.
 #pragma clang fp contract(off)
 
-#include "../../include/mmf.h"   // dtype ids, error codes, entry-point declarations
+#include "../../include/mmf.h"        // dtype ids, error codes, entry-point declarations
+#include "../../include/mmf_diag.h"   // measuring aids
 
 #define MMF_CHECK_LAUNCH()                          \
     do {                                            \

@@ -192,31 +192,37 @@ class DecodeEngine:
         fill(table[4 * self.L], self.final_norm, self.eps, self.head, H, self.V)
         raw = torch.frombuffer(bytearray(bytes(table)), dtype=torch.uint8)
         self.phases = raw.to(self.dev)
-        sizes = [H, H, D, D, H, H, I]                       # h0, h1, o, g, attn, res, z
-        words = torch.zeros(sum(sizes), dtype=torch.int32, device=self.dev)
+        # tagged hand-off words: every row in `copies` copies (one per XCD), [copies, n] each, in the kernel's order
+        R = self.lib.mmf_decode_layers_copies()
+        sizes = [H, H, D, D, H, I]                          # h0, h1, o, g, attn, z
+        words = torch.zeros(self.lib.mmf_decode_layers_words(H, D, I), dtype=torch.int32, device=self.dev)
         self.words, off = [], 0
         for n in sizes:
-            self.words.append(words[off:off + n])
-            off += n
+            self.words.append(words[off:off + R * n].view(R, n))
+            off += R * n
+        assert off == words.numel()
         self._words = words
         self.am_words = torch.zeros(256, dtype=torch.int64, device=self.dev)
         self.epoch = torch.zeros(1, dtype=torch.int32, device=self.dev)
         self.err = torch.zeros(1, dtype=torch.int32, device=self.dev)
 
-    def _launch_layers(self, with_head: bool, trace: Optional[torch.Tensor] = None):
-        w = [t.data_ptr() for t in self.words]
+    def _launch_layers(self, with_head: bool, trace: Optional[torch.Tensor] = None, delay: int = 6):
         head = self.phases.data_ptr() + 4 * self.L * ctypes.sizeof(_Phase) if with_head else None
-        L.check(self.lib.mmf_decode_layers(self.phases.data_ptr(), self.L, self.table.data_ptr(), self.tok.data_ptr(), self.V,
-                                           *w, self.h.data_ptr(), head, self.logits.data_ptr(), self.am_words.data_ptr(),
-                                           self.tok.data_ptr(), self.epoch.data_ptr(), self.err.data_ptr(), L.ptr(trace),
-                                           self.H, self.D, self.I, self.SPIN, self.dt_id, L.stream()), "mmf_decode_layers")
+        args = (self.phases.data_ptr(), self.L, self.table.data_ptr(), self.tok.data_ptr(), self.V, self._words.data_ptr(),
+                self.h.data_ptr(), head, self.logits.data_ptr(), self.am_words.data_ptr(), self.tok.data_ptr(),
+                self.epoch.data_ptr(), self.err.data_ptr())
+        if trace is None:
+            L.check(self.lib.mmf_decode_layers(*args, self.H, self.D, self.I, self.SPIN, self.dt_id, L.stream()), "mmf_decode_layers")
+        else:
+            L.check(self.lib.mmf_decode_layers_traced(*args, trace.data_ptr(), self.H, self.D, self.I, self.SPIN, delay, self.dt_id,
+                                                      L.stream()), "mmf_decode_layers_traced")
 
-    def link_trace(self) -> torch.Tensor:
+    def link_trace(self, delay: int = 6) -> torch.Tensor:
         """One resident step with the kernel's cycle trace on: int64 [3 workgroups, 128 links, 12 stamps] (see
-        mmf_decode_layers in include/mmf.h), on the host."""
+        mmf_decode_layers_traced in include/mmf_diag.h), on the host."""
         assert self.resident
         t = torch.zeros(self.lib.mmf_decode_layers_trace_words(), dtype=torch.int64, device=self.dev)
-        self._launch_layers(True, trace=t)
+        self._launch_layers(True, trace=t, delay=delay)
         torch.cuda.synchronize(self.dev)
         return t.view(3, 128, 12).cpu()
 

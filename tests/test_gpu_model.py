@@ -440,9 +440,9 @@ def test_resident_engine_is_clean_after_a_timed_out_launch(dev, tiny_bf16):
     torch.cuda.synchronize()
     assert not eng.resident_ok()
     e = int(eng.epoch.item())
-    h0, h1, ob, gb, ab, rb, zb = eng.words
+    h0, h1, ob, gb, ab, zb = eng.words                           # [copies, n] each
     wrong = 0x3F80 << 16                                         # bf16 1.0 in the value half
-    for buf, link in ((ob, 0), (gb, 0), (ab, 1), (rb, 2), (zb, 2), (h0, 3)):
+    for buf, link in ((ob, 0), (gb, 0), (ab, 1), (zb, 2), (h0, 3)):
         buf.fill_(wrong | ((e + link + 1) & 0xFFFF))
     with pytest.raises(L_.MMFError):
         eng.check()

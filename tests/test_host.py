@@ -11,9 +11,13 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def header_symbols():
-    text = open(os.path.join(ROOT, "include", "mmf.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(mmf_[a-z0-9_]+)\s*\(", text)))
+    """Every function the two public headers declare: the drop-in boundary (mmf.h) and the measuring aids (mmf_diag.h)."""
+    syms = set()
+    for name in ("mmf.h", "mmf_diag.h"):
+        text = open(os.path.join(ROOT, "include", name)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        syms |= set(re.findall(r"\b(mmf_[a-z0-9_]+)\s*\(", text))
+    return sorted(syms)
 
 
 def test_library_exports_every_declared_symbol():
@@ -23,7 +27,7 @@ def test_library_exports_every_declared_symbol():
     syms = header_symbols()
     assert len(syms) >= 18
     for s in syms:
-        assert hasattr(lib, s), f"{s} declared in include/mmf.h but not exported"
+        assert hasattr(lib, s), f"{s} declared in include/ but not exported"
     assert sorted(_lib.SIGNATURES) == syms, "ctypes signature table and header disagree"
 
 
@@ -193,16 +197,20 @@ def test_rejected_shapes_and_pointers_return_their_code_before_any_launch():
     # gate math: row stride shorter than the row
     assert lib.mmf_hgrn_gate(P, 32, P, 64, None, None, P, P, 2, 64, 1, None) == -1
     # resident layer chain: D must equal H, rows are whole k-blocks, 16-bit activations only, bounded widths, aligned rows
-    layers = lambda h, d, i, dtype=1, h0=P, spin=100: lib.mmf_decode_layers(P, 2, P, P, 1000, h0, P, P, P, P, P, P, P, None, None, None,
-                                                                          None, P, P, None, h, d, i, spin, dtype, None)
+    # arguments: phases, n_layers, table, tok, vocab, words, h_out, head, logits, am_words, tok_out, epoch, err, H, D, I, spin, dtype
+    layers = lambda h, d, i, dtype=1, words=P, spin=100: lib.mmf_decode_layers(P, 2, P, P, 1000, words, P, None, None, None, None, P, P,
+                                                                             h, d, i, spin, dtype, None)
     assert layers(512, 256, 1536) == -1 and layers(500, 500, 1536) == -1 and layers(512, 512, 1500) == -1
     assert layers(512, 512, 1536, dtype=0) == -1 and layers(512, 512, 1536, spin=0) == -1
     assert layers(4224, 4224, 4096) == -2 and layers(2048, 2048, 8320) == -2
-    assert layers(512, 512, 1536, h0=P + 4) == -3
-    assert lib.mmf_decode_layers(None, 2, P, P, 1000, P, P, P, P, P, P, P, P, None, None, None, None, P, P, None, 512, 512, 1536,
-                                 100, 1, None) == -1
-    assert lib.mmf_decode_layers(P, 2, P, P, 1000, P, P, P, P, P, P, P, P, P, None, P, P, P, P, None, 512, 512, 1536, 100, 1,
+    assert layers(512, 512, 1536, words=P + 4) == -3
+    assert lib.mmf_decode_layers(None, 2, P, P, 1000, P, P, None, None, None, None, P, P, 512, 512, 1536, 100, 1, None) == -1
+    assert lib.mmf_decode_layers(P, 2, P, P, 1000, P, P, P, None, P, P, P, P, 512, 512, 1536, 100, 1,
                                  None) == -1                      # a head record without its logits buffer
+    assert lib.mmf_decode_layers_traced(P, 2, P, P, 1000, P, P, None, None, None, None, P, P, None, 512, 512, 1536, 100, 6, 1,
+                                        None) == -1               # the traced form needs its trace buffer
+    assert lib.mmf_decode_layers_copies() == 8
+    assert lib.mmf_decode_layers_words(512, 512, 1536) == 8 * (5 * 512 + 1536)
     assert lib.mmf_decode_layers_trace_words() == 3 * 128 * 12
     assert lib.mmf_decode_layers_phase_bytes() == 80
 
