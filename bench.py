@@ -156,9 +156,10 @@ def gemv_roofline(eng, iters=20):
             "avg_launch_us": round(us_per_launch, 3)}
 
 
-def link_trace_bench(model, dev):
+def link_trace_bench(model, dev, delay=6):
     """Where a link of the resident batch-1 launch spends its cycles: the kernel's own cycle stamps (thread 0 of three
-    workgroups, ten points per link), averaged per kind of link over the layers of one decode step."""
+    workgroups, nine points per link; the traced build of the kernel), averaged per kind of link over the layers of one
+    decode step."""
     import numpy as np
     from matmulfreellm_amd.decode import DecodeEngine
     eng = DecodeEngine.for_model(model, 1, use_graph=True)
@@ -166,19 +167,23 @@ def link_trace_bench(model, dev):
         return None
     for _ in range(4):
         eng._launch_layers(True)
-    t = eng.link_trace().numpy().astype(np.float64)
+    t = eng.link_trace(delay=delay).numpy().astype(np.float64)
     assert eng.resident_ok()
     names = ["i/f/g", "o_proj", "gate/up", "down"]
-    stages = ["row arrives", "block norm", "sum of squares", "rstd", "absmax", "codes -> LDS", "dot", "partials meet", "epilogue"]
-    out = {"unit": "shader clock cycles (s_memtime), mean over layers 2.. of one step", "stages": stages, "workgroups": {}}
+    stages = ["row arrives", "block norm", "sum of squares", "absmax", "codes -> LDS", "dot", "partials meet", "epilogue"]
+    out = {"unit": "shader clock cycles (s_memtime), mean over layers 2.. of one step", "stages": stages, "poll_delay": delay,
+           "workgroups": {}}
     nl = 4 * eng.L
     for slot, wg in enumerate((0, 37, 200)):
         per = {}
         for kind in range(4):
-            rows = t[slot, kind:nl:4, :10][2:]
+            rows = t[slot, kind:nl:4, :9][2:]
+            nxt = t[slot, kind + 1:nl + 1:4, 0][2:]                     # entry of the following link
+            n = min(len(rows), len(nxt))
             per[names[kind]] = {"stages": [round(float(v)) for v in np.diff(rows, axis=1).mean(axis=0)],
-                                "link_total": round(float((rows[:, 9] - rows[:, 0]).mean()))}
-        per["whole_chain_cycles"] = int(t[slot, nl - 1, 9] - t[slot, 0, 0])
+                                "link_total": round(float((rows[:, 8] - rows[:, 0]).mean())),
+                                "entry_to_next_entry": round(float((nxt[:n] - rows[:n, 0]).mean()))}
+        per["whole_chain_cycles"] = int(t[slot, nl - 1, 8] - t[slot, 0, 0])
         out["workgroups"][str(wg)] = per
     return out
 

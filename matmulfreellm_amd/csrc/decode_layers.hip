@@ -3,15 +3,16 @@
 // A decode step is a chain of 4 dependent fused BitLinears per layer (mmfreelm/models/hgrn_bit/
 // modeling_hgrn_bit.py:97-109 around mmfreelm/layers/hgrn_bit.py:83-162): block norm -> i/f/g -> gate math +
 // recurrence step; gated norm -> o_proj; residual + norm -> gate_proj -> swiglu; down_proj + residual.
-// 256 workgroups of 4 waves stay resident (one per CU, one wave per SIMD) and walk the 4L links themselves.
+// 256 workgroups of 4 waves stay resident (one per CU, one wave per SIMD) and walk the 4L links themselves, all
+// through ONE loop body (a single wave per SIMD has nobody to hide instruction fetch behind: the code stays small).
 //
 // Hand-off.  Activations travel between workgroups as self-validating 32-bit words: a 16-bit value in the high half,
-// a 16-bit tag naming the producing link in the low half.  A producer stores its words to 8 replicas of the row (one
+// a 16-bit tag naming the producing link in the low half.  A producer stores its words to 8 copies of the row (one
 // per XCD: a row polled by 256 workgroups at once is a hot spot in the memory-side cache, 32 pollers per copy are
-// not); a consumer polls the copy of its XCD with 16-byte device-coherent loads until every word carries the tag.
-// The poll is both the synchronisation and the transfer: no fence, no grid barrier.  The first poll of a link is
-// held back a little so that it reaches memory after the producers' stores rather than just before them (a poll that
-// comes back stale costs a whole round trip).
+// not); a consumer polls the copy of its XCD with device-coherent loads until every word carries the tag.  The poll
+// is both the synchronisation and the transfer: no fence, no grid barrier.  The first poll of a link is held back a
+// little so that it reaches memory after the producers' stores rather than just before them (a poll that comes back
+// stale costs a whole round trip).
 //
 // Body of a link.  A wave owns a contiguous slice of the row's k-blocks from the poll to the dot products: it polls
 // that slice, takes part in the row statistics (per-wave partial -> LDS -> barrier: sum of squares of the block norm,
@@ -19,9 +20,14 @@
 // of the packed weights -- the codes never cross waves, so no barrier sits between quantiser and dot.  The per-wave
 // partial dot products meet in LDS for the epilogue (one more barrier).  A workgroup owns row-groups of 8 output rows
 // (row-group g of a segment belongs to workgroup g mod 256); 16 lanes = (2 halves x 8 rows) read the 2-bit weights of
-// one k-block, so a wave load covers 4 k-blocks.  The packed weights, norm weights and epilogue operands of link n+1
-// are requested as soon as link n's row has arrived, so they stream from HBM under link n's arithmetic and the
-// hand-off (loads return in order: requested before the poll they would delay it).
+// one k-block, so a wave load covers 4 k-blocks.
+//
+// Nothing a link needs besides its input row is waited for inside the link: the phase table is copied to LDS when the
+// launch starts; the packed weights and the norm weights of link n+1 are brought into LDS by the DMA path
+// (global_load_lds, no registers) while link n computes, each wave fetching exactly the slices it will read itself;
+// the few epilogue operands (recurrent state, lower bound, scales, residual operands) are loaded into registers one
+// link ahead.  All of these are requested after link n's row has arrived: loads return in order, requested before
+// the poll they would delay it.
 //
 // The arithmetic of every link is that of bitlinear_gemv_kernel with the same prologue / epilogue, operation for
 // operation (sums of squares in fp64 are order-insensitive to rounding, integer sums exact).
@@ -41,15 +47,17 @@
 // error word.
 #include "mmf_common.h"
 #include <stdlib.h>
+#include <type_traits>
 
 namespace {
 
 constexpr int kNW = 4, kNT = 64 * kNW;
 constexpr int kWGs = 256, kRep = 8;
-constexpr int kHeadChunk = 16;                 // row-groups of the lm_head a workgroup takes per pass
+constexpr int kMaxLayers = 96;
+constexpr int kItems = 8;                      // (row-group, segment) items of a pass over a link's outputs
 
 #define MMF_AS_GLOBAL __attribute__((address_space(1)))
-#define MMF_AS_CONST __attribute__((address_space(4)))
+#define MMF_AS_LDS __attribute__((address_space(3)))
 
 struct Phase {                // one fused BitLinear; four per layer: i/f/g, o, gate, down
     const void* w1;           // weight of the norm in front of the BitLinear (null for down)
@@ -62,6 +70,7 @@ struct Phase {                // one fused BitLinear; four per layer: i/f/g, o, 
     float eps, eps1;
     int K, N, seg_rows, pad_;
 };
+static_assert(sizeof(Phase) == 80, "five 16-byte pieces per record");
 
 struct LayersArgs {
     const Phase* phases;      // [4 * n_layers], device memory, not written during the launch
@@ -78,6 +87,9 @@ struct LayersArgs {
     int* err;                 // set to 1 when a poll ran out of rounds
     long long* trace;         // TRACE builds: kTraceWGs * kTraceLinks * kTraceStamps cycle stamps
     int n_layers, H, D, I, spin, delay;
+    int nqmax;                // k-quads of the widest wave slice: a wave's norm-weight region in LDS is nqmax KiB
+    int itemsA, itemsB;       // 1 KiB weight loads per wave the two weight buffers hold
+    uint32_t off_q, off_nrm, off_w;   // dynamic LDS: codes, norm weights (w1 regions, then the BitLinear's), weight buffers
 };
 
 constexpr int kTraceWGs = 3, kTraceLinks = 128, kTraceStamps = 12;
@@ -87,10 +99,6 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 // Loads through the global address space (pointers read from the phase table are generic to the compiler; these keep
 // the accesses off the flat path).  Builtin vector types only: they can be read from any address space.
-__device__ __forceinline__ uint4 gload16(const void* base, uint32_t byte_off) {
-    const u32x4 v = *reinterpret_cast<const MMF_AS_GLOBAL u32x4*>((const MMF_AS_GLOBAL char*)(base) + byte_off);
-    return make_uint4(v.x, v.y, v.z, v.w);
-}
 __device__ __forceinline__ uint2 gload8(const void* base, uint32_t byte_off) {
     const u32x2 v = *reinterpret_cast<const MMF_AS_GLOBAL u32x2*>((const MMF_AS_GLOBAL char*)(base) + byte_off);
     return make_uint2(v.x, v.y);
@@ -98,8 +106,22 @@ __device__ __forceinline__ uint2 gload8(const void* base, uint32_t byte_off) {
 __device__ __forceinline__ float gloadf(const void* base, int i) { return ((const MMF_AS_GLOBAL float*)base)[i]; }
 __device__ __forceinline__ uint16_t gload2(const void* base, int i) { return ((const MMF_AS_GLOBAL uint16_t*)base)[i]; }
 
-enum Pro : int { PRO_PLAIN = 0, PRO_NORM = 1, PRO_RESNORM = 2, PRO_GATEDNORM = 3 };
-enum Epi : int { EPI_PLAIN = 0, EPI_STEP = 1, EPI_SWIGLU = 2, EPI_HEAD = 3 };
+// 64 lanes x 16 bytes from global memory straight into 1 KiB of LDS at `lds` (wave-uniform), lane order.
+// Issued by hand: told about a transfer into LDS, the compiler makes every later LDS read (the statistics exchanged a
+// few hundred cycles on, the partial sums) wait for it -- a trip to HBM in the middle of every link.  The data is
+// only read after the next link's input row has arrived, and that wait covers it (loads return in order).
+__device__ __forceinline__ void dma16(const void* gbase, uint32_t byte_off, unsigned char* lds) {
+    const uint32_t l = (uint32_t)(uintptr_t)(MMF_AS_LDS unsigned char*)lds;
+    const uint64_t b = (uint64_t)gbase;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(l), "v"(byte_off), "s"(b) : "memory");
+}
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding vector-memory
+// operation -- here that would be the DMA of the NEXT link's weights, requested a moment ago, i.e. a trip to HBM in
+// the middle of every link.  Those requests are waited for where their data is needed (the next link's poll).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+enum Kind : int { K_IFG = 0, K_O = 1, K_GATE = 2, K_DOWN = 3, K_HEAD = 4 };
 
 // Running greedy choice of one epilogue lane: lowest index of the largest value seen; NaNs never win.
 struct Best {
@@ -111,17 +133,17 @@ __device__ __forceinline__ void best_take(Best& b, float v, uint32_t i) {
     if (i != kNone && (b.i == kNone || v > b.v || (v == b.v && i < b.i))) { b.v = v; b.i = i; }
 }
 
-struct Smem {
-    int8_t q[8192];                          // int8 codes of the row; a wave reads and writes its own slice only
+struct Small {
     double sum1[kNW], sum2[kNW];             // per-wave partial sums of squares
     float amax[kNW];
     int qs[kNW];                             // per-wave sums of codes
-    int part[kHeadChunk][8][2 * kNW];        // [row-group x segment][row][wave x lane half] partial dot products
+    int part[kItems][8][2 * kNW];            // [row-group x segment][row][wave x lane half] partial dot products
     float best_v[kNW];
     uint32_t best_i[kNW];
 };
 
 __device__ __forceinline__ uint64_t ll_ld8(const uint64_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ uint32_t ll_ld4(const uint32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void ll_st8(uint64_t* p, uint64_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 // Four tagged words as two 8-byte device-coherent loads (relaxed atomics: the compiler keeps track of them, so a whole
@@ -150,547 +172,566 @@ struct RowSrc {
     uint32_t tag;
 };
 
-// Geometry of a link for this wave and workgroup (all wave-uniform).
-struct Geo {
-    int K, KB, kb0, nkb, nq;                 // row width, its k-blocks, this wave's slice [kb0, kb0 + nkb), k-quads per item
-    int Nseg, NBseg, RG, NG;                 // rows / n-blocks / row-groups per segment, row-groups of this workgroup
+// Wave-uniform values read from the LDS copy of the phase table, as scalars.
+__device__ __forceinline__ uint32_t uni32(const void* lds) { return (uint32_t)__builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(lds)); }
+__device__ __forceinline__ uint64_t uni64(const void* lds) {
+    const int* p = reinterpret_cast<const int*>(lds);
+    return (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane(p[0]) | ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane(p[1]) << 32);
+}
+// Shape of the model a kernel instantiation serves.  Static: hidden and intermediate width are compile-time constants,
+// so every link's geometry (k-blocks per wave, passes, loads, masks) folds into the code -- with one wave per SIMD a
+// wave issues one instruction every four cycles, scalar or vector, so bookkeeping instructions cost as much as
+// arithmetic and are worth compiling away.  Dynamic: the same source with the widths read from the arguments.
+template <int H_, int I_>
+struct StaticShape {
+    static constexpr bool kStatic = true;
+    static constexpr int H = H_, I = I_;
 };
-template <int R>
-__device__ __forceinline__ Geo make_geo(int K, int N, int wave) {
+struct DynShape {
+    static constexpr bool kStatic = false;
+    static constexpr int H = 0, I = 0;
+};
+constexpr int ceil_div_c(int a, int b) { return (a + b - 1) / b; }
+// passes of 256 elements over a wave's slice of a K-wide row, k-quads of that slice
+constexpr int passes_of(int K) { return ceil_div_c(ceil_div_c(K / 128, kNW), 2); }
+constexpr int quads_of(int K) { return ceil_div_c(ceil_div_c(K / 128, kNW), 4); }
+
+// Geometry of a link for this wave and workgroup (all wave-uniform; constants when the shape is static).
+struct Geo {
+    int K, KB, kb0, nkb, nq, np;             // row width, its k-blocks, this wave's slice [kb0, kb0 + nkb), k-quads and 256-element passes of a slice
+    int R, Nseg, NBseg, NG;                  // segments, rows / n-blocks per segment, row-groups of this workgroup
+    bool even;                               // every wave's slice is nq whole k-quads: no clamps, no masks
+};
+__device__ __forceinline__ Geo make_geo(int K, int N, int kind, int wave) {
     Geo g;
     g.K = K;
     g.KB = K >> 7;
     const int kbw = (g.KB + kNW - 1) / kNW;
     g.kb0 = wave * kbw;
     g.nkb = g.KB - g.kb0 < 0 ? 0 : (g.KB - g.kb0 < kbw ? g.KB - g.kb0 : kbw);
+    if (g.KB % kNW == 0) g.nkb = kbw;        // (folds when K is a constant)
     if (g.nkb == 0) g.kb0 = 0;
     g.nq = (kbw + 3) >> 2;
-    g.Nseg = N / R;
+    g.np = (kbw + 1) >> 1;
+    g.even = g.KB % (4 * kNW) == 0;
+    g.R = kind == K_IFG ? 3 : kind == K_GATE ? 2 : 1;
+    g.Nseg = kind == K_IFG ? N / 3 : kind == K_GATE ? N >> 1 : N;
     g.NBseg = (g.Nseg + 31) >> 5;
-    g.RG = (g.Nseg + 7) >> 3;
-    g.NG = g.RG > (int)blockIdx.x ? (g.RG - (int)blockIdx.x + kWGs - 1) / kWGs : 0;
+    const int RG = (g.Nseg + 7) >> 3;
+    g.NG = RG > (int)blockIdx.x ? (RG - (int)blockIdx.x + kWGs - 1) / kWGs : 0;
     return g;
 }
 
-// Everything a link needs that does not depend on the link before it: requested one link ahead.
-template <typename T, int NP, int MAXLD, int R, int NGE = 1>
-struct Pre {
-    uint4 w[MAXLD];                          // packed weights: load j = (row-group, segment, k-quad), 4 k-blocks x 16 lanes
-    Raw4<T> w1raw[NP], nwraw[NP];            // norm weights of this wave's slice
-    float wdeq[R];
-    float lb[NGE], state[NGE];               // i/f/g epilogue: lower bound and recurrent state of this lane's channel, per row-group
-                                             // (read here, before any wave's epilogue writes the new state)
-    uint32_t add0, add1;                     // down epilogue: the two operands of the residual (tagged words or plain)
-};
+template <typename T, class S, bool TRACE>
+__global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
+    extern __shared__ __align__(16) unsigned char dyn[];
+    __shared__ Small sm;
+    const uint32_t e = *a.epoch;
+    int64_t id = *a.tok;
+    if (id < 0 || id >= a.vocab) id = 0;
+    const int L = a.n_layers;
+    const T* emb_row = static_cast<const T*>(a.table) + id * (S::kStatic ? S::H : a.H);
 
-// The weights of row-groups [g0, g0 + ng) of this workgroup (at most MAXLD loads; the rest is left alone).
-template <int R, int MAXLD>
-__device__ __forceinline__ void load_weights(const Phase& ph, const Geo& g, int g0, int ng, int lane, uint4 (&w)[MAXLD]) {
-    if (g.nkb == 0) return;
-    const int slot = lane >> 4;
-    const uint32_t lane_off = (uint32_t)(((lane >> 3) & 1) * 512 + (lane & 7) * 16);
-    int gi = 0, r = 0, q = 0;
-#pragma unroll
-    for (int j = 0; j < MAXLD; ++j) {
-        if (gi < ng) {
-            const int rg = (int)blockIdx.x + kWGs * (g0 + gi);
-            const int nb = (rg >> 2) + r * g.NBseg;
-            const uint32_t s_off = (uint32_t)(nb * g.KB + g.kb0) * 1024u + (uint32_t)(rg & 3) * 128u;
-            int kbl = 4 * q + slot;
-            kbl = kbl < g.nkb ? kbl : g.nkb - 1;
-            w[j] = gload16(ph.packed, s_off + (uint32_t)kbl * 1024u + lane_off);
-        }
-        if (++q == g.nq) { q = 0; if (++r == R) { r = 0; ++gi; } }
+    // ---- the phase table into LDS: a record is then an LDS read away, not a cold trip to memory in front of every link
+    {
+        const int n16 = 4 * L * 5;
+        for (int i = threadIdx.x; i < n16; i += kNT) reinterpret_cast<uint4*>(dyn)[i] = reinterpret_cast<const uint4*>(a.phases)[i];
+        if (a.head && threadIdx.x < 5) reinterpret_cast<uint4*>(dyn)[n16 + threadIdx.x] = reinterpret_cast<const uint4*>(a.head)[threadIdx.x];
     }
-}
+    __syncthreads();
 
-// Element index (within the row) of the first of the four elements lane `lane` holds in pass v of this wave's slice.
-__device__ __forceinline__ int slice_elem(const Geo& g, int v, int lane) { return g.kb0 * 128 + 4 * (64 * v + lane); }
-__device__ __forceinline__ bool slice_has(const Geo& g, int v, int lane) { return 4 * (64 * v + lane) < g.nkb * 128; }
-
-template <typename T, int NP>
-__device__ __forceinline__ void load_norm_weights(const void* wp, const Geo& g, int lane, Raw4<T> (&raw)[NP]) {
-    static_assert(sizeof(T) == 2, "16-bit activations");
-#pragma unroll
-    for (int v = 0; v < NP; ++v) {
-        const int k0 = slice_has(g, v, lane) ? slice_elem(g, v, lane) : 0;
-        raw[v].v = gload8(wp, (uint32_t)k0 * 2u);
-    }
-}
-
-template <typename T, int NPH, int NPI, int NQH, int NQI, int NGH, int NGI, bool TRACE>
-struct Chain {
-    // loads per wave and link kind
-    static constexpr int LD_IFG = NGH * 3 * NQH, LD_O = NGH * NQH, LD_GATE = NGI * 2 * NQH, LD_DOWN = NGH * NQI,
-                         LD_HEAD = kHeadChunk * NQH;
-    using PreIfg = Pre<T, NPH, LD_IFG, 3, NGH>;
-    using PreO = Pre<T, NPH, LD_O, 1>;
-    using PreGate = Pre<T, NPH, LD_GATE, 2>;
-    using PreDown = Pre<T, NPI, LD_DOWN, 1>;
-    using PreHead = Pre<T, NPH, LD_HEAD, 1>;
-
-    const LayersArgs& a;
-    Smem& sm;
-    const int lane, wave;
-    const uint32_t e;
-    uint32_t* const hb0;                      // bases of the word buffers (copy 0)
-    uint32_t* const hb1;
-    uint32_t* const ob;
-    uint32_t* const gb;
-    uint32_t* const ab;
-    uint32_t* const zb;
-    const int rep;                            // the copy this workgroup polls
-
-    __device__ Chain(const LayersArgs& a_, Smem& sm_, uint32_t e_)
-        : a(a_), sm(sm_), lane(threadIdx.x & 63), wave(__builtin_amdgcn_readfirstlane(threadIdx.x >> 6)), e(e_),
-          hb0(a_.words), hb1(a_.words + kRep * a_.H), ob(a_.words + 2 * kRep * a_.H), gb(a_.words + 2 * kRep * a_.H + kRep * a_.D),
-          ab(a_.words + 2 * kRep * a_.H + 2 * kRep * a_.D), zb(a_.words + 3 * kRep * a_.H + 2 * kRep * a_.D), rep((int)blockIdx.x & (kRep - 1)) {}
-
-    __device__ __forceinline__ uint32_t tag_of(int link) const { return (e + (uint32_t)link + 1u) & 0xffffu; }
-
-    __device__ __forceinline__ void stamp(int link, int i) const {
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int slot = lane >> 4, half = (lane >> 3) & 1;
+    const uint32_t lane_off = (uint32_t)(half * 512 + (lane & 7) * 16);       // this lane's 16 bytes within a 1 KiB weight block, less the k-block
+    const int rep = (int)blockIdx.x & (kRep - 1);                             // the copy this workgroup polls
+    constexpr int NP = S::kStatic ? (passes_of(S::H) > passes_of(S::I) ? passes_of(S::H) : passes_of(S::I)) : 8;   // passes of the widest row
+    constexpr int NPH = S::kStatic ? passes_of(S::H) : 4;                                                           // passes of a hidden-wide row
+    using KIfg = std::integral_constant<int, K_IFG>;
+    using KO = std::integral_constant<int, K_O>;
+    using KGate = std::integral_constant<int, K_GATE>;
+    using KDown = std::integral_constant<int, K_DOWN>;
+    using KHead = std::integral_constant<int, K_HEAD>;
+    Best best{0.0f, kNone};
+    // epilogue operands of this lane, loaded one link ahead; a set per kind of link, so that the request for the next
+    // link does not replace what the current link's epilogue is about to use
+    float wdk[5][3] = {};
+    float lb[2] = {0.0f, 0.0f}, st[2] = {0.0f, 0.0f};     // i/f/g: lower bound and recurrent state of this lane's channel, per row-group
+    uint32_t a0 = 0u, a1 = 0u;                             // down: the two operands of the residual
+    const int Hh = S::kStatic ? S::H : a.H, Ii = S::kStatic ? S::I : a.I;
+    int8_t* const qbuf = reinterpret_cast<int8_t*>(dyn + a.off_q);
+    unsigned char* const nrm_w1 = dyn + a.off_nrm;                                   // kNW regions of nqmax KiB
+    unsigned char* const nrm_nw = dyn + a.off_nrm + kNW * a.nqmax * 1024;
+    unsigned char* const wbufA = dyn + a.off_w;                                      // weights of i/f/g and gate/up (and the lm_head's even passes)
+    unsigned char* const wbufB = dyn + a.off_w + kNW * a.itemsA * 1024;              // weights of o_proj and down_proj (and the lm_head's odd passes)
+    uint32_t* const hb0 = a.words;
+    uint32_t* const hb1 = a.words + kRep * Hh;
+    uint32_t* const ob = a.words + 2 * kRep * Hh;
+    uint32_t* const gb = a.words + 3 * kRep * Hh;
+    uint32_t* const ab = a.words + 4 * kRep * Hh;
+    uint32_t* const zb = a.words + 5 * kRep * Hh;
+    auto tag_of = [&](int link) -> uint32_t { return (e + (uint32_t)link + 1u) & 0xffffu; };
+    auto stamp = [&](int link, int i) {
         if constexpr (TRACE) {
             if (threadIdx.x == 0 && link < kTraceLinks) {
-                const int slot = blockIdx.x == 0 ? 0 : blockIdx.x == 37 ? 1 : blockIdx.x == 200 ? 2 : -1;
-                if (slot >= 0) a.trace[(slot * kTraceLinks + link) * kTraceStamps + i] = __builtin_amdgcn_s_memtime();
+                const int s = blockIdx.x == 0 ? 0 : blockIdx.x == 37 ? 1 : blockIdx.x == 200 ? 2 : -1;
+                if (s >= 0) a.trace[(s * kTraceLinks + link) * kTraceStamps + i] = __builtin_amdgcn_s_memtime();
             }
         }
-    }
-
-    // ---- what a link requests one link ahead
-    template <int NP, int MAXLD, int R, int PRO, int EPI, int NGE>
-    __device__ __forceinline__ void prefetch(const Phase& ph, const Geo& g, Pre<T, NP, MAXLD, R, NGE>& pre, const RowSrc& add0, const RowSrc& add1) {
-        if (g.NG == 0) return;
-        load_weights<R, MAXLD>(ph, g, 0, g.NG < kHeadChunk ? g.NG : kHeadChunk, lane, pre.w);
-        if constexpr (PRO >= PRO_NORM) load_norm_weights<T, NP>(ph.w1, g, lane, pre.w1raw);
-        load_norm_weights<T, NP>(ph.norm_w, g, lane, pre.nwraw);
-#pragma unroll
-        for (int r = 0; r < R; ++r) pre.wdeq[r] = gloadf(ph.wdeq, ph.seg_rows == g.Nseg ? r : 0);
-        if constexpr (EPI == EPI_STEP) {
-            // lanes of a 32-lane half: 0-7 the i rows, 8-15 the f rows, 16-23 the g rows of one row-group
-#pragma unroll
-            for (int gi = 0; gi < NGE; ++gi) {
-                const int ch = ((int)blockIdx.x + kWGs * gi) * 8 + (lane & 7);
-                pre.lb[gi] = 0.0f;
-                pre.state[gi] = 0.0f;
-                if (gi < g.NG && ch < g.Nseg) {
-                    if (ph.lb) pre.lb[gi] = gloadf(ph.lb, ch);
-                    pre.state[gi] = gloadf(ph.state, ch);
-                }
-            }
+    };
+    // the record of link ln in the LDS copy of the phase table
+    auto rec = [&](int ln) -> const unsigned char* { return dyn + ln * (int)sizeof(Phase); };
+    auto geo = [&](auto kc, int ln) -> Geo {
+        constexpr int KIND = decltype(kc)::value;
+        if constexpr (S::kStatic) {
+            constexpr int K = KIND == K_DOWN ? S::I : S::H;
+            const int N = KIND == K_IFG ? 3 * S::H : KIND == K_O ? S::H : KIND == K_GATE ? 2 * S::I : KIND == K_DOWN ? S::H : (int)uni32(rec(ln) + 68);
+            return make_geo(K, N, KIND, wave);
+        } else {
+            return make_geo((int)uni32(rec(ln) + 64), (int)uni32(rec(ln) + 68), KIND, wave);
         }
-        if constexpr (EPI == EPI_PLAIN && PRO == PRO_PLAIN) {
-            // down: the residual operands of this lane's channel (lane = copy x row; wave = row-group)
-            const int ch = ((int)blockIdx.x + kWGs * wave) * 8 + (lane & 7);
-            pre.add0 = pre.add1 = 0u;
-            if (wave < g.NG && ch < g.Nseg) {
-                pre.add0 = fetch_word(add0, ch);
-                pre.add1 = fetch_word(add1, ch);
-            }
-        }
-    }
-
+    };
+    auto h_src = [&](int l) -> RowSrc {        // the residual stream that enters layer l (this XCD's copy)
+        return l == 0 ? RowSrc{emb_row, nullptr, tag_of(-1)} : RowSrc{nullptr, ((l - 1) & 1 ? hb1 : hb0) + rep * Hh, tag_of(4 * (l - 1) + 3)};
+    };
     // One element of a row as a tagged word (a plain element gets the tag it is expected to carry).
-    __device__ __forceinline__ uint32_t fetch_word(const RowSrc& s, int ch) const {
+    auto fetch_word = [&](const RowSrc& s, int ch) -> uint32_t {
         if (s.plain) return ((uint32_t)gload2(s.plain, ch) << 16) | s.tag;
-        return __hip_atomic_load(s.words + ch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __device__ __forceinline__ float finish_word(uint32_t w, const RowSrc& s, int ch) const {
-        int n = 0;
-        while ((w & 0xffffu) != s.tag && n++ < a.spin) w = __hip_atomic_load(s.words + ch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((w & 0xffffu) != s.tag) *a.err = 1;
-        return word_value<T>(w);
-    }
-
-    // ---- the row (and the prologue's second operand) of this wave's slice: poll until every word carries the tag
-    template <int NP, bool HAS_AUX>
-    __device__ __forceinline__ void poll(const Geo& g, const RowSrc& xs, const RowSrc& as, u32x4 (&X)[NP], u32x4 (&A)[HAS_AUX ? NP : 1]) {
-        auto plain4 = [&](const RowSrc& s, int k0) {
-            const uint2 r = gload8(s.plain, (uint32_t)k0 * 2u);
-            u32x4 w;
-            w.x = (r.x << 16) | s.tag; w.y = (r.x & 0xffff0000u) | s.tag; w.z = (r.y << 16) | s.tag; w.w = (r.y & 0xffff0000u) | s.tag;
-            return w;
-        };
-        const bool x_tagged = xs.plain == nullptr, a_tagged = HAS_AUX && as.plain == nullptr;
-        int k0[NP];
-#pragma unroll
-        for (int v = 0; v < NP; ++v) k0[v] = slice_has(g, v, lane) ? slice_elem(g, v, lane) : g.kb0 * 128;
-        if (x_tagged || a_tagged)
-            for (int d = 0; d < a.delay; ++d) __builtin_amdgcn_s_sleep(1);
-#pragma unroll
-        for (int v = 0; v < NP; ++v) {
-            if (x_tagged) X[v] = poll_issue(xs.words + k0[v]);
-            else X[v] = plain4(xs, k0[v]);
-            if constexpr (HAS_AUX) {
-                if (a_tagged) A[v] = poll_issue(as.words + k0[v]);
-                else A[v] = plain4(as, k0[v]);
-            }
+        return ll_ld4(s.words + ch);
+    };
+    auto finish_word = [&](uint32_t w, const RowSrc& s, int ch) -> float {
+        if (!s.plain) {
+            int n = 0;
+            while ((w & 0xffffu) != s.tag && n++ < a.spin) w = ll_ld4(s.words + ch);
+            if ((w & 0xffffu) != s.tag) *a.err = 1;
         }
-        if (!(x_tagged || a_tagged)) return;
-        for (int n = 0;; ++n) {
-            bool all = true;
+        return word_value<T>(w);
+    };
+    auto wbuf_of = [&](auto kc, int pass) -> unsigned char* {
+        constexpr int KIND = decltype(kc)::value;
+        const bool useA = KIND == K_HEAD ? !(pass & 1) : (KIND == K_IFG || KIND == K_GATE);
+        return (useA ? wbufA + wave * a.itemsA * 1024 : wbufB + wave * a.itemsB * 1024);
+    };
+
+    // ---- requests made one link ahead
+    // packed weights of row-groups [g0, g0 + ng) of this workgroup, this wave's k-slice, into dst
+    auto dma_weights = [&](const void* packed, const Geo& g, int g0, int ng, unsigned char* dst) {
+        if (g.nkb == 0) return;
+        int j = 0;
+        for (int gi = 0; gi < ng; ++gi) {
+            const int rg = (int)blockIdx.x + kWGs * (g0 + gi);
 #pragma unroll
-            for (int v = 0; v < NP; ++v) {
-                if (x_tagged && __builtin_amdgcn_ballot_w64(!words_valid(X[v], xs.tag)) != 0) { all = false; X[v] = poll_issue(xs.words + k0[v]); }
-                if constexpr (HAS_AUX) {
-                    if (a_tagged && __builtin_amdgcn_ballot_w64(!words_valid(A[v], as.tag)) != 0) { all = false; A[v] = poll_issue(as.words + k0[v]); }
+            for (int r = 0; r < 3; ++r) {
+                if (r < g.R) {
+                    const int nb = (rg >> 2) + r * g.NBseg;
+                    const uint32_t s_off = (uint32_t)(nb * g.KB + g.kb0) * 1024u + (uint32_t)(rg & 3) * 128u + lane_off;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        if (q < g.nq) {
+                            int kbl = 4 * q + slot;
+                            if (!g.even) kbl = kbl < g.nkb ? kbl : g.nkb - 1;
+                            dma16(packed, s_off + (uint32_t)kbl * 1024u, dst + j * 1024);
+                            ++j;
+                        }
+                    }
                 }
             }
-            if (all) break;
-            if (n >= a.spin) {
-                if (lane == 0) *a.err = 1;
-                break;
+        }
+    };
+    // norm weights of this wave's slice (the region of a wave is written and read by that wave only)
+    auto dma_norm = [&](auto kc, const unsigned char* rc, const Geo& g) {
+        constexpr int KIND = decltype(kc)::value;
+        if (g.nkb == 0 || g.NG == 0) return;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (q < g.nq) {
+                const int el = q * 512 + lane * 8;
+                const uint32_t off = (uint32_t)(g.kb0 * 128 + (g.even || el < g.nkb * 128 ? el : 0)) * 2u;
+                if constexpr (KIND != K_DOWN) dma16(reinterpret_cast<const void*>(uni64(rc)), off, nrm_w1 + (wave * a.nqmax + q) * 1024);
+                dma16(reinterpret_cast<const void*>(uni64(rc + 8)), off, nrm_nw + (wave * a.nqmax + q) * 1024);
             }
         }
-    }
+    };
+    // epilogue operands of this lane for the link that comes next
+    auto load_ep = [&](auto kc, const unsigned char* rc, const Geo& g, const RowSrc& add0, const RowSrc& add1) {
+        constexpr int KIND = decltype(kc)::value;
+        const void* wdeq = reinterpret_cast<const void*>(uni64(rc + 24));
+        const bool per_seg = (int)uni32(rc + 72) == g.Nseg;
+#pragma unroll
+        for (int r = 0; r < 3; ++r)
+            if (r < g.R) wdk[KIND][r] = gloadf(wdeq, per_seg ? r : 0);
+        if constexpr (KIND == K_IFG) {
+            const void* lbp = reinterpret_cast<const void*>(uni64(rc + 32));
+            const void* stp = reinterpret_cast<const void*>(uni64(rc + 40));
+#pragma unroll
+            for (int gi = 0; gi < 2; ++gi) {
+                // read here, one link ahead, so that no wave reads a state another wave's epilogue has already replaced
+                const int ch = ((int)blockIdx.x + kWGs * gi) * 8 + (lane & 7);
+                lb[gi] = 0.0f;
+                st[gi] = 0.0f;
+                if (gi < g.NG && ch < g.Nseg) {
+                    if (lbp) lb[gi] = gloadf(lbp, ch);
+                    st[gi] = gloadf(stp, ch);
+                }
+            }
+        }
+        if constexpr (KIND == K_DOWN) {
+            const int ch = ((int)blockIdx.x + kWGs * wave) * 8 + (lane & 7);
+            a0 = a1 = 0u;
+            if (wave < g.NG && ch < g.Nseg) { a0 = fetch_word(add0, ch); a1 = fetch_word(add1, ch); }
+        }
+    };
+    // everything link ln (of kind KIND) needs besides its row; called while the link before it computes
+    auto request = [&](auto kc, int ln) {
+        constexpr int KIND = decltype(kc)::value;
+        const Geo g = geo(kc, ln);
+        if (g.NG == 0) return;
+        const unsigned char* rc = rec(ln);
+        const int cap = (KIND == K_IFG || KIND == K_GATE || KIND == K_HEAD ? a.itemsA : a.itemsB) / (g.R * g.nq);   // row-groups a buffer holds
+        dma_weights(reinterpret_cast<const void*>(uni64(rc + 16)), g, 0, g.NG < cap ? g.NG : cap, wbuf_of(kc, 0));
+        const int l = ln >> 2;
+        const RowSrc none{nullptr, nullptr, 0u};
+        if constexpr (KIND == K_DOWN) load_ep(kc, rc, g, RowSrc{nullptr, ab + rep * Hh, tag_of(4 * l + 1)}, h_src(l));
+        else load_ep(kc, rc, g, none, none);
+    };
 
-    // ---- prologue: norms, absmax int8 codes of this wave's slice into LDS.  Returns deq (1 / scale).
-    template <int NP, int PRO>
-    __device__ __forceinline__ float prologue(const Phase& ph, const Geo& g, const u32x4 (&X)[NP], const u32x4 (&A)[PRO >= PRO_RESNORM ? NP : 1],
-                                              const Raw4<T> (&w1raw)[NP], const Raw4<T> (&nwraw)[NP], int link) {
-        constexpr bool HAS_AUX = PRO >= PRO_RESNORM, HAS_W1 = PRO >= PRO_NORM;
-        float xv[NP][4], av[HAS_AUX ? NP : 1][4];
-        bool has[NP];
+    // the integer result of item `it`, row `row`: the waves' partial sums less the row's code sum (weights are stored as t + 1)
+    auto total = [&](int it, int row) -> int {
+        const int4 p0 = *reinterpret_cast<const int4*>(&sm.part[it][row][0]);
+        const int4 p1 = *reinterpret_cast<const int4*>(&sm.part[it][row][4]);
+        const int4 qv = *reinterpret_cast<const int4*>(&sm.qs[0]);
+        return ((p0.x + p0.y) + (p0.z + p0.w)) + ((p1.x + p1.y) + (p1.z + p1.w)) - ((qv.x + qv.y) + (qv.z + qv.w));
+    };
+    // Two neighbouring rows' words become one 8-byte store by the even row (fewer, wider stores travel faster).
+    auto store_pair = [&](uint32_t* base, int ch, uint32_t word, bool active) {
+        const uint32_t next = (uint32_t)mmf_dpp<kDppXor1>((int)word);
+        if (active && !(lane & 1)) ll_st8(reinterpret_cast<uint64_t*>(base + ch), (uint64_t)word | ((uint64_t)next << 32));
+    };
+
+    // ---- one link.  NEXT: the kind of the link that follows (its requests are made here, once this link's row is in).
+    auto link = [&](auto kc, auto nc, int ln, bool more) {
+        constexpr int KIND = decltype(kc)::value, NEXT = decltype(nc)::value;
+        constexpr bool HAS_AUX = KIND == K_O || KIND == K_GATE, HAS_W1 = KIND != K_DOWN;
+        constexpr int NPK = KIND == K_DOWN ? NP : NPH;                       // passes this link's row can take
+        const int l = ln >> 2;
+        const Geo g = geo(kc, ln);
+        stamp(ln, 0);
+        if (g.NG == 0) {
+            // nothing of this link falls to this workgroup; it still requests what its next link needs
+            if (more) { request(nc, ln + 1); dma_norm(nc, rec(ln + 1), geo(nc, ln + 1)); }
+            return;
+        }
+        const unsigned char* rc = rec(ln);
+        const RowSrc none{nullptr, nullptr, 0u};
+        RowSrc xs = none, as = none, add0 = none, add1 = none;
+        if constexpr (KIND == K_IFG) xs = h_src(l);
+        if constexpr (KIND == K_O) { xs = RowSrc{nullptr, gb + rep * Hh, tag_of(4 * l)}; as = RowSrc{nullptr, ob + rep * Hh, tag_of(4 * l)}; }
+        if constexpr (KIND == K_GATE) { xs = RowSrc{nullptr, ab + rep * Hh, tag_of(4 * l + 1)}; as = h_src(l); }
+        if constexpr (KIND == K_DOWN) { xs = RowSrc{nullptr, zb + rep * Ii, tag_of(4 * l + 2)}; add0 = RowSrc{nullptr, ab + rep * Hh, tag_of(4 * l + 1)}; add1 = h_src(l); }
+        if constexpr (KIND == K_HEAD) xs = h_src(L);
+
+        // ---- the row (and the prologue's second operand) of this wave's slice: poll until every word carries the tag
+        u32x4 X[NPK], A[HAS_AUX ? NPK : 1];
+        bool has[NPK];
+        int k0[NPK];
 #pragma unroll
-        for (int v = 0; v < NP; ++v) {
-            has[v] = slice_has(g, v, lane);
-            xv[v][0] = has[v] ? word_value<T>(X[v].x) : 0.0f; xv[v][1] = has[v] ? word_value<T>(X[v].y) : 0.0f;
-            xv[v][2] = has[v] ? word_value<T>(X[v].z) : 0.0f; xv[v][3] = has[v] ? word_value<T>(X[v].w) : 0.0f;
-            if constexpr (HAS_AUX) {
-                av[v][0] = has[v] ? word_value<T>(A[v].x) : 0.0f; av[v][1] = has[v] ? word_value<T>(A[v].y) : 0.0f;
-                av[v][2] = has[v] ? word_value<T>(A[v].z) : 0.0f; av[v][3] = has[v] ? word_value<T>(A[v].w) : 0.0f;
+        for (int v = 0; v < NPK; ++v) {
+            has[v] = g.even || 4 * (64 * v + lane) < g.nkb * 128;
+            k0[v] = g.kb0 * 128 + (has[v] ? 4 * (64 * v + lane) : 0);
+        }
+        {
+            auto plain4 = [&](const RowSrc& s, int k) {
+                const uint2 r = gload8(s.plain, (uint32_t)k * 2u);
+                u32x4 w;
+                w.x = (r.x << 16) | s.tag; w.y = (r.x & 0xffff0000u) | s.tag; w.z = (r.y << 16) | s.tag; w.w = (r.y & 0xffff0000u) | s.tag;
+                return w;
+            };
+            const bool x_tagged = xs.plain == nullptr, a_tagged = HAS_AUX && as.plain == nullptr;
+            if (x_tagged || a_tagged)
+                for (int d = 0; d < a.delay; ++d) __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+            for (int v = 0; v < NPK; ++v) {
+                if (v < g.np) {
+                    X[v] = x_tagged ? poll_issue(xs.words + k0[v]) : plain4(xs, k0[v]);
+                    if constexpr (HAS_AUX) A[v] = a_tagged ? poll_issue(as.words + k0[v]) : plain4(as, k0[v]);
+                }
+            }
+            if (x_tagged || a_tagged) {
+                for (int n = 0;; ++n) {
+                    bool ok = true;
+#pragma unroll
+                    for (int v = 0; v < NPK; ++v) {
+                        if (v < g.np) {
+                            if (x_tagged) ok = ok & words_valid(X[v], xs.tag);
+                            if constexpr (HAS_AUX) {
+                                if (a_tagged) ok = ok & words_valid(A[v], as.tag);
+                            }
+                        }
+                    }
+                    if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+                    if (n >= a.spin) {
+                        if (lane == 0) *a.err = 1;
+                        break;
+                    }
+#pragma unroll
+                    for (int v = 0; v < NPK; ++v) {
+                        if (v < g.np) {
+                            if (x_tagged) X[v] = poll_issue(xs.words + k0[v]);
+                            if constexpr (HAS_AUX) {
+                                if (a_tagged) A[v] = poll_issue(as.words + k0[v]);
+                            }
+                        }
+                    }
+                }
             }
         }
-        if constexpr (PRO == PRO_RESNORM) {
+        // every load made so far has been waited for (said explicitly: the requests below are not to be waited for here)
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        stamp(ln, 1);
+        // ---- the row is here: now request what the next link needs
+        if (more) request(nc, ln + 1);
+
+        // ---- prologue: norms, absmax int8 codes of this wave's slice into LDS
+        float xv[NPK][4], av[HAS_AUX ? NPK : 1][4];
 #pragma unroll
-            for (int v = 0; v < NP; ++v)
+        for (int v = 0; v < NPK; ++v) {
+            const bool on = v < g.np && has[v];
+            xv[v][0] = on ? word_value<T>(X[v].x) : 0.0f; xv[v][1] = on ? word_value<T>(X[v].y) : 0.0f;
+            xv[v][2] = on ? word_value<T>(X[v].z) : 0.0f; xv[v][3] = on ? word_value<T>(X[v].w) : 0.0f;
+            if constexpr (HAS_AUX) {
+                av[v][0] = on ? word_value<T>(A[v].x) : 0.0f; av[v][1] = on ? word_value<T>(A[v].y) : 0.0f;
+                av[v][2] = on ? word_value<T>(A[v].z) : 0.0f; av[v][3] = on ? word_value<T>(A[v].w) : 0.0f;
+            }
+        }
+        const unsigned char* my_w1 = nrm_w1 + wave * a.nqmax * 1024 + lane * 8;
+        const unsigned char* my_nw = nrm_nw + wave * a.nqmax * 1024 + lane * 8;
+        const double inv_K = __longlong_as_double((long long)uni64(rc + 48));
+        if constexpr (KIND == K_GATE) {
+#pragma unroll
+            for (int v = 0; v < NPK; ++v)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) xv[v][i] = __fadd_rn(xv[v][i], av[v][i]);
         }
         if constexpr (HAS_W1) {
             double s1 = 0.0;
 #pragma unroll
-            for (int v = 0; v < NP; ++v)
+            for (int v = 0; v < NPK; ++v)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) s1 = mmf_add_square(s1, xv[v][i]);
             s1 = mmf_wave_sum(s1);
             if (lane == 0) sm.sum1[wave] = s1;
-            float sg[PRO == PRO_GATEDNORM ? NP : 1][4];
-            if constexpr (PRO == PRO_GATEDNORM) {             // the swish gate does not wait for the statistics
+            float sg[KIND == K_O ? NPK : 1][4];
+            if constexpr (KIND == K_O) {                          // the swish gate does not wait for the statistics
 #pragma unroll
-                for (int v = 0; v < NP; ++v)
+                for (int v = 0; v < NPK; ++v)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) sg[v][i] = mmf_sigmoid(av[v][i]);
+                    for (int i = 0; i < 4; ++i) sg[v][i] = v < g.np ? mmf_sigmoid(av[v][i]) : 0.0f;
             }
-            __syncthreads();
+            lds_barrier();
             const double tot = (sm.sum1[0] + sm.sum1[1]) + (sm.sum1[2] + sm.sum1[3]);
-            const float rstd1 = mmf_rstd(tot, g.K, ph.inv_K, ph.eps1);
+            const float rstd1 = mmf_rstd(tot, g.K, inv_K, __uint_as_float(uni32(rc + 60)));
 #pragma unroll
-            for (int v = 0; v < NP; ++v) {
-                float w1v[4];
-                raw4_unpack<T>(w1raw[v], w1v);
+            for (int v = 0; v < NPK; ++v) {
+                if (v < g.np) {
+                    Raw4<T> raw;
+                    raw.v = *reinterpret_cast<const uint2*>(my_w1 + v * 512);
+                    float w1v[4];
+                    raw4_unpack<T>(raw, w1v);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float y = __fmul_rn(__fmul_rn(xv[v][i], rstd1), w1v[i]);
-                    if constexpr (PRO == PRO_GATEDNORM) y = __fmul_rn(__fmul_rn(y, av[v][i]), sg[v][i]);
-                    xv[v][i] = has[v] ? mmf_round_to<T>(y) : 0.0f;
+                    for (int i = 0; i < 4; ++i) {
+                        float y = __fmul_rn(__fmul_rn(xv[v][i], rstd1), w1v[i]);
+                        if constexpr (KIND == K_O) y = __fmul_rn(__fmul_rn(y, av[v][i]), sg[v][i]);
+                        xv[v][i] = has[v] ? mmf_round_to<T>(y) : 0.0f;
+                    }
                 }
             }
         }
-        stamp(link, 2);
+        stamp(ln, 2);
         // the BitLinear's own norm
         double ss = 0.0;
 #pragma unroll
-        for (int v = 0; v < NP; ++v)
+        for (int v = 0; v < NPK; ++v)
 #pragma unroll
             for (int i = 0; i < 4; ++i) ss = mmf_add_square(ss, xv[v][i]);
         ss = mmf_wave_sum(ss);
         if (lane == 0) sm.sum2[wave] = ss;
-        __syncthreads();
+        lds_barrier();
         const double tot2 = (sm.sum2[0] + sm.sum2[1]) + (sm.sum2[2] + sm.sum2[3]);
-        const float rstd = mmf_rstd(tot2, g.K, ph.inv_K, ph.eps);
-        stamp(link, 3);
+        const float rstd = mmf_rstd(tot2, g.K, inv_K, __uint_as_float(uni32(rc + 56)));
+        stamp(ln, 3);
         float amax = 0.0f;
 #pragma unroll
-        for (int v = 0; v < NP; ++v) {
-            float wv[4];
-            raw4_unpack<T>(nwraw[v], wv);
+        for (int v = 0; v < NPK; ++v) {
+            if (v < g.np) {
+                Raw4<T> raw;
+                raw.v = *reinterpret_cast<const uint2*>(my_nw + v * 512);
+                float wv[4];
+                raw4_unpack<T>(raw, wv);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float y = has[v] ? __fmul_rn(__fmul_rn(xv[v][i], rstd), wv[i]) : 0.0f;
-                xv[v][i] = y;
-                amax = fmaxf(amax, fabsf(y));
+                for (int i = 0; i < 4; ++i) {
+                    const float y = has[v] ? __fmul_rn(__fmul_rn(xv[v][i], rstd), wv[i]) : 0.0f;
+                    xv[v][i] = y;
+                    amax = fmaxf(amax, fabsf(y));
+                }
             }
         }
+        // this wave is done with its norm-weight regions: the next link's may come in
+        if (more) dma_norm(nc, rec(ln + 1), geo(nc, ln + 1));
         amax = mmf_wave_max(amax);
         if (lane == 0) sm.amax[wave] = amax;
-        __syncthreads();
+        lds_barrier();
         amax = fmaxf(fmaxf(sm.amax[0], sm.amax[1]), fmaxf(sm.amax[2], sm.amax[3]));
-        stamp(link, 4);
+        stamp(ln, 4);
         const float scale = __fdiv_rn(127.0f, fmaxf(amax, 1e-5f));
         int qs = 0;
 #pragma unroll
-        for (int v = 0; v < NP; ++v) {
-            uint32_t packed4 = 0;
+        for (int v = 0; v < NPK; ++v) {
+            if (v < g.np) {
+                uint32_t packed4 = 0;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int c = mmf_code(xv[v][i], scale);
-                qs += c;
-                packed4 |= (uint32_t)(c & 0xff) << (8 * i);
+                for (int i = 0; i < 4; ++i) packed4 |= (uint32_t)(mmf_code(xv[v][i], scale) & 0xff) << (8 * i);
+                qs = __builtin_amdgcn_sdot4((int)packed4, 0x01010101, qs, false);      // the sum of the four codes
+                if (has[v]) *reinterpret_cast<uint32_t*>(qbuf + k0[v]) = packed4;
             }
-            if (has[v]) *reinterpret_cast<uint32_t*>(sm.q + slice_elem(g, v, lane)) = packed4;
         }
         qs = mmf_wave_sum(qs);
         if (lane == 0) sm.qs[wave] = qs;
-        // the codes are read back by this wave only: LDS operations of a wave execute in order, no barrier needed
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        stamp(link, 5);
-        return __fdiv_rn(1.0f, scale);       // needed by the epilogue only
-    }
+        const float deq = __fdiv_rn(1.0f, scale);       // needed by the epilogue only
+        stamp(ln, 5);
 
-    // ---- dot products of this wave's slice with the weights of row-groups [0, ng) x R segments; partial sums to LDS
-    template <int R, int MAXLD>
-    __device__ __forceinline__ void dot(const Geo& g, int ng, const uint4 (&w)[MAXLD]) {
-        if (g.nkb == 0) {
-            // nothing of this row belongs to the wave: its partial sums are zero
-            for (int it = lane >> 4; it < ng * R; it += 4)
-                if ((lane & 15) < 8) { sm.part[it][lane & 7][2 * wave] = 0; sm.part[it][lane & 7][2 * wave + 1] = 0; }
-            return;
-        }
-        const int slot = lane >> 4, half = (lane >> 3) & 1;
-        int gi = 0, r = 0, q = 0, acc = 0;
+        const uint32_t tag = tag_of(ln);
+        const int rq = g.R * g.nq;
+        const int capA = a.itemsA / rq, capB = a.itemsB / rq;
+        const int cap0 = (KIND == K_IFG || KIND == K_GATE || KIND == K_HEAD) ? capA : capB;       // row-groups of the first pass
+        int g0 = 0;
+        for (int pass = 0; g0 < g.NG; ++pass) {
+            const int cap = KIND == K_HEAD ? ((pass & 1) ? capB : capA) : cap0;
+            const int ng = g.NG - g0 < cap ? g.NG - g0 : cap;
+            if (pass > 0) {
+                __builtin_amdgcn_s_waitcnt(0x0F70);                   // vmcnt(0): this pass's weights, requested a pass ago, have landed
+                lds_barrier();                                        // part[] of the pass before has been read
+            }
+            if (KIND == K_HEAD || !S::kStatic) {
+                // more row-groups than a buffer holds (the lm_head): the next pass's weights travel under this one
+                const int gn = g0 + ng;
+                if (gn < g.NG) {
+                    const int capn = KIND == K_HEAD ? ((pass & 1) ? capA : capB) : cap0;
+                    dma_weights(reinterpret_cast<const void*>(uni64(rc + 16)), g, gn, g.NG - gn < capn ? g.NG - gn : capn, wbuf_of(kc, pass + 1));
+                }
+            }
+            // ---- dot products of this wave's slice with the weights of this pass; partial sums to LDS.  The weights were
+            // requested a link (or a pass) ago; the wait for the row (or the one above) has seen them land (loads return in
+            // order).  The codes are read back by this wave only: LDS operations of a wave execute in order.
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            if (g.nkb == 0) {
+                for (int it = lane >> 4; it < ng * g.R; it += 4)
+                    if ((lane & 15) < 8) { sm.part[it][lane & 7][2 * wave] = 0; sm.part[it][lane & 7][2 * wave + 1] = 0; }
+            } else {
+                const unsigned char* src = wbuf_of(kc, pass) + lane * 16;
+                const int nit = ng * g.R;
+                for (int it = 0; it < nit; ++it) {
+                    int acc = 0;
 #pragma unroll
-        for (int j = 0; j < MAXLD; ++j) {
-            if (gi < ng) {
-                const int kraw = 4 * q + slot;
-                const bool live = kraw < g.nkb;
-                const int kb = g.kb0 + (live ? kraw : g.nkb - 1);
-                uint4 wq = w[j];
-                if (!live) wq = make_uint4(0u, 0u, 0u, 0u);
-                acc = mmf_dot_block(sm.q, wq, kb, half, acc);
-                if (q == g.nq - 1) {
+                    for (int q = 0; q < 4; ++q) {
+                        if (q < g.nq) {
+                            const int kraw = 4 * q + slot;
+                            const bool live = g.even || kraw < g.nkb;
+                            const int kb = g.kb0 + (live ? kraw : g.nkb - 1);
+                            uint4 wq = *reinterpret_cast<const uint4*>(src + (it * g.nq + q) * 1024);
+                            if (!live) wq = make_uint4(0u, 0u, 0u, 0u);
+                            acc = mmf_dot_block(qbuf, wq, kb, half, acc);
+                        }
+                    }
                     acc += mmf_dpp<0x128>(acc);                              // the other half of the 16 lanes (rotate by 8)
                     acc += __builtin_amdgcn_ds_swizzle(acc, 0x401F);         // lane ^ 16: the neighbouring k-block
-                    if ((lane & 31) < 8) sm.part[gi * R + r][lane & 7][2 * wave + (lane >> 5)] = acc;
-                    acc = 0;
+                    if ((lane & 31) < 8) sm.part[it][lane & 7][2 * wave + (lane >> 5)] = acc;
                 }
             }
-            if (++q == g.nq) { q = 0; if (++r == R) { r = 0; ++gi; } }
-        }
-    }
-
-    // the integer result of item `it`, row `row`: the waves' partial sums less the row's code sum (weights are stored as t + 1)
-    __device__ __forceinline__ int total(int it, int row) const {
-        const int4 p0 = *reinterpret_cast<const int4*>(&sm.part[it][row][0]);
-        const int4 p1 = *reinterpret_cast<const int4*>(&sm.part[it][row][4]);
-        const int4 qv = *reinterpret_cast<const int4*>(&sm.qs[0]);
-        return ((p0.x + p0.y) + (p0.z + p0.w)) + ((p1.x + p1.y) + (p1.z + p1.w)) - ((qv.x + qv.y) + (qv.z + qv.w));
-    }
-
-    // Two neighbouring rows' words become one 8-byte store by the even row (fewer, wider stores travel faster).
-    __device__ __forceinline__ void store_pair(uint32_t* base, int ch, uint32_t word, bool active) const {
-        const uint32_t next = (uint32_t)mmf_dpp<kDppXor1>((int)word);
-        if (active && !(lane & 1)) ll_st8(reinterpret_cast<uint64_t*>(base + ch), (uint64_t)word | ((uint64_t)next << 32));
-    }
-
-    // ================================================================ the four links of a layer
-    // i/f/g: block norm -> stacked projection -> gate math + recurrence step
-    template <class PreNext, class FNext>
-    __device__ __forceinline__ void link_ifg(const Phase& ph, const Geo& g, PreIfg& pre, const RowSrc& h_in, int link, FNext&& next) {
-        stamp(link, 0);
-        if (g.NG == 0) { next(); return; }
-        u32x4 X[NPH], A[1];
-        poll<NPH, false>(g, h_in, h_in, X, A);
-        stamp(link, 1);
-        next();
-        const float deq = prologue<NPH, PRO_NORM>(ph, g, X, A, pre.w1raw, pre.nwraw, link);
-        dot<3, LD_IFG>(g, g.NG, pre.w);
-        stamp(link, 6);
-        __syncthreads();
-        stamp(link, 7);
-        const uint32_t tag = tag_of(link);
-        // a wave serves two copies: lanes 0-23 of each 32-lane half run the i, f and g rows of the 8 channels side by
-        // side, so the two exp / divide chains of the gate math run in parallel; the f lanes' gate reaches the i lanes by
-        // a rotate within the 16-lane row.  Operation for operation the arithmetic of the single-lane form.
-        const int r3 = (lane & 31) >> 3, row = lane & 7, copy = 2 * wave + (lane >> 5);
+            stamp(ln, 6);
+            lds_barrier();
+            stamp(ln, 7);
+            // ---- epilogue
+            if constexpr (KIND == K_IFG) {
+                // a wave serves two copies: lanes 0-23 of each 32-lane half run the i, f and g rows of the 8 channels side
+                // by side, so the two exp / divide chains of the gate math run in parallel; the f lanes' gate reaches the i
+                // lanes by a rotate within the 16-lane row.  Operation for operation the arithmetic of the single-lane form.
+                const int r3 = (lane & 31) >> 3, row = lane & 7, copy = 2 * wave + (lane >> 5);
+                const void* lbp = reinterpret_cast<const void*>(uni64(rc + 32));
+                float* stp = reinterpret_cast<float*>(uni64(rc + 40));
 #pragma unroll
-        for (int gi = 0; gi < NGH; ++gi) {
-            if (gi >= g.NG) break;
-            const int ch = ((int)blockIdx.x + kWGs * gi) * 8 + row;
-            const float lb = pre.lb[gi], st = pre.state[gi];
-            const int tot = total(gi * 3 + (r3 < 3 ? r3 : 0), row);
-            const float wd = r3 == 0 ? pre.wdeq[0] : r3 == 1 ? pre.wdeq[1] : pre.wdeq[2];
-            const float res = __fmul_rn(__fmul_rn((float)tot, deq), wd);
-            const float v16 = mmf_round_to<T>(res);                       // iv on the i lanes, fv on the f lanes
-            const float ex = __fadd_rn(1.0f, mmf_exp(-v16));
-            float sg = __fdiv_rn(1.0f, ex);                               // sigmoid(fv) on the f lanes
-            if (ph.lb) sg = __fadd_rn(lb, __fmul_rn(__fsub_rn(1.0f, lb), sg));
-            const float go = mmf_dpp<0x128>(mmf_round_to<T>(sg));         // lanes 0-7 read lanes 8-15
-            const float xo = mmf_round_to<T>(__fdiv_rn(__fmul_rn(v16, __fsub_rn(1.0f, go)), ex));
-            const float h = __fadd_rn(__fmul_rn(go, st), xo);
-            const bool live = ch < g.Nseg;
-            if (live && r3 == 0 && copy == 0) ((MMF_AS_GLOBAL float*)ph.state)[ch] = h;
-            store_pair(ob + copy * a.D, ch, make_word<T>(h, tag), live && r3 == 0);
-            store_pair(gb + copy * a.D, ch, make_word<T>(res, tag), live && r3 == 2);
-        }
-        stamp(link, 8);
-    }
-
-    // a link whose 8 x 8 epilogue lanes are copy x row, one row-group per wave: o_proj, gate/up, down
-    template <int NP, int MAXLD, int R, int PRO, int EPI, class FNext>
-    __device__ __forceinline__ void link_plain(const Phase& ph, const Geo& g, Pre<T, NP, MAXLD, R, 1>& pre, const RowSrc& xs, const RowSrc& as,
-                                               const RowSrc& add0, const RowSrc& add1, uint32_t* out, int out_n, T* plain_out, int link,
-                                               FNext&& next) {
-        stamp(link, 0);
-        if (g.NG == 0) { next(); return; }
-        constexpr bool HAS_AUX = PRO >= PRO_RESNORM;
-        u32x4 X[NP], A[HAS_AUX ? NP : 1];
-        poll<NP, HAS_AUX>(g, xs, as, X, A);
-        stamp(link, 1);
-        next();
-        const float deq = prologue<NP, PRO>(ph, g, X, A, pre.w1raw, pre.nwraw, link);
-        dot<R, MAXLD>(g, g.NG, pre.w);
-        stamp(link, 6);
-        __syncthreads();
-        stamp(link, 7);
-        const uint32_t tag = tag_of(link);
-        const int row = lane & 7, copy = lane >> 3;
-        for (int gi = wave; gi < g.NG; gi += kNW) {
-            const int ch = ((int)blockIdx.x + kWGs * gi) * 8 + row;
-            const bool live = ch < g.Nseg;
-            float res[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r) res[r] = __fmul_rn(__fmul_rn((float)total(gi * R + r, row), deq), pre.wdeq[r]);
-            float o;
-            if constexpr (EPI == EPI_SWIGLU) {
-                const float gt = mmf_round_to<T>(res[0]), u = mmf_round_to<T>(res[1]);
-                o = __fdiv_rn(__fmul_rn(gt, u), __fadd_rn(1.0f, mmf_exp(-gt)));
-            } else {
-                o = res[0];
-                if constexpr (PRO == PRO_PLAIN) {
-                    // down: the residual it adds is T(attn + h), formed here from its two operands
-                    uint32_t w0 = pre.add0, w1 = pre.add1;
-                    if (gi != wave && live) { w0 = fetch_word(add0, ch); w1 = fetch_word(add1, ch); }
-                    float r0 = 0.0f, r1 = 0.0f;
-                    if (live) {
-                        r0 = add0.plain ? word_value<T>(w0) : finish_word(w0, add0, ch);
-                        r1 = add1.plain ? word_value<T>(w1) : finish_word(w1, add1, ch);
+                for (int gl = 0; gl < 2; ++gl) {
+                    if (gl >= ng) break;
+                    const int ch = ((int)blockIdx.x + kWGs * (g0 + gl)) * 8 + row;
+                    const float lbv = g0 + gl == 0 ? lb[0] : lb[1], stv = g0 + gl == 0 ? st[0] : st[1];
+                    const int tot = total(gl * 3 + (r3 < 3 ? r3 : 0), row);
+                    const float wdv = r3 == 0 ? wdk[KIND][0] : r3 == 1 ? wdk[KIND][1] : wdk[KIND][2];
+                    const float res = __fmul_rn(__fmul_rn((float)tot, deq), wdv);
+                    const float v16 = mmf_round_to<T>(res);                       // iv on the i lanes, fv on the f lanes
+                    const float ex = __fadd_rn(1.0f, mmf_exp(-v16));
+                    float sgm = __fdiv_rn(1.0f, ex);                              // sigmoid(fv) on the f lanes
+                    if (lbp) sgm = __fadd_rn(lbv, __fmul_rn(__fsub_rn(1.0f, lbv), sgm));
+                    const float go = mmf_dpp<0x128>(mmf_round_to<T>(sgm));        // lanes 0-7 read lanes 8-15
+                    const float xo = mmf_round_to<T>(__fdiv_rn(__fmul_rn(v16, __fsub_rn(1.0f, go)), ex));
+                    const float h = __fadd_rn(__fmul_rn(go, stv), xo);
+                    const bool live = ch < g.Nseg;
+                    if (live && r3 == 0 && copy == 0) ((MMF_AS_GLOBAL float*)stp)[ch] = h;
+                    store_pair(ob + copy * Hh, ch, make_word<T>(h, tag), live && r3 == 0);
+                    store_pair(gb + copy * Hh, ch, make_word<T>(res, tag), live && r3 == 2);
+                }
+            } else if constexpr (KIND == K_HEAD) {
+                const int row = lane & 7;                                 // a wave takes 8 row-groups of a pass
+                for (int gl = wave * 8 + (lane >> 3); gl < ng; gl += 8 * kNW) {
+                    const int ch = ((int)blockIdx.x + kWGs * (g0 + gl)) * 8 + row;
+                    if (ch < g.Nseg) {
+                        const float o = __fmul_rn(__fmul_rn((float)total(gl, row), deq), wdk[KIND][0]);
+                        static_cast<T*>(a.logits)[ch] = mmf_from_float<T>(o);
+                        const float ov = mmf_round_to<T>(o);
+                        if (ov == ov) best_take(best, ov, (uint32_t)ch);
                     }
-                    o = __fadd_rn(mmf_round_to<T>(o), mmf_round_to<T>(__fadd_rn(r0, r1)));
+                }
+            } else {
+                // 8 x 8 lanes are copy x row, one row-group per wave: o_proj, gate/up, down
+                const int row = lane & 7, copy = lane >> 3;
+                uint32_t* out = KIND == K_O ? ab : KIND == K_GATE ? zb : ((l & 1) ? hb1 : hb0);
+                const int out_n = KIND == K_GATE ? Ii : Hh;
+                for (int gl = wave; gl < ng; gl += kNW) {
+                    const int ch = ((int)blockIdx.x + kWGs * (g0 + gl)) * 8 + row;
+                    const bool live = ch < g.Nseg;
+                    float o = __fmul_rn(__fmul_rn((float)total(gl * g.R, row), deq), wdk[KIND][0]);
+                    if constexpr (KIND == K_GATE) {
+                        const float u = mmf_round_to<T>(__fmul_rn(__fmul_rn((float)total(gl * 2 + 1, row), deq), wdk[KIND][1]));
+                        const float gt = mmf_round_to<T>(o);
+                        o = __fdiv_rn(__fmul_rn(gt, u), __fadd_rn(1.0f, mmf_exp(-gt)));
+                    }
+                    if constexpr (KIND == K_DOWN) {
+                        // the residual it adds is T(attn + h), formed here from its two operands
+                        uint32_t w0 = a0, w1 = a1;
+                        if (g0 + gl != wave && live) { w0 = fetch_word(add0, ch); w1 = fetch_word(add1, ch); }
+                        float r0 = 0.0f, r1 = 0.0f;
+                        if (live) { r0 = finish_word(w0, add0, ch); r1 = finish_word(w1, add1, ch); }
+                        o = __fadd_rn(mmf_round_to<T>(o), mmf_round_to<T>(__fadd_rn(r0, r1)));
+                    }
+                    store_pair(out + copy * out_n, ch, make_word<T>(o, tag), live);
+                    if (KIND == K_DOWN && l == L - 1 && live && copy == 0) static_cast<T*>(a.h_out)[ch] = mmf_from_float<T>(o);
                 }
             }
-            store_pair(out + copy * out_n, ch, make_word<T>(o, tag), live);
-            if (plain_out && live && copy == 0) plain_out[ch] = mmf_from_float<T>(o);
+            stamp(ln, 8);
+            g0 += ng;
         }
-        stamp(link, 8);
-    }
-
-    // final norm -> lm_head: plain logits, and this lane's running candidate for the greedy token
-    template <class FNext>
-    __device__ __forceinline__ void link_head(const Phase& ph, const Geo& g, PreHead& pre, const RowSrc& h_last, int link, Best& best, FNext&& next) {
-        stamp(link, 0);
-        if (g.NG == 0) { next(); return; }
-        u32x4 X[NPH], A[1];
-        poll<NPH, false>(g, h_last, h_last, X, A);
-        stamp(link, 1);
-        next();
-        const float deq = prologue<NPH, PRO_NORM>(ph, g, X, A, pre.w1raw, pre.nwraw, link);
-        T* logits = static_cast<T*>(a.logits);
-        for (int c0 = 0; c0 < g.NG; c0 += kHeadChunk) {
-            const int ng = g.NG - c0 < kHeadChunk ? g.NG - c0 : kHeadChunk;
-            if (c0 > 0) load_weights<1, LD_HEAD>(ph, g, c0, ng, lane, pre.w);
-            dot<1, LD_HEAD>(g, ng, pre.w);
-            __syncthreads();
-            const int gl = wave * 8 + (lane >> 3), row = lane & 7;        // a wave takes 8 row-groups of the chunk
-            if (gl < ng) {
-                const int ch = ((int)blockIdx.x + kWGs * (c0 + gl)) * 8 + row;
-                if (ch < g.Nseg) {
-                    const float o = __fmul_rn(__fmul_rn((float)total(gl, row), deq), pre.wdeq[0]);
-                    logits[ch] = mmf_from_float<T>(o);
-                    const float ov = mmf_round_to<T>(o);
-                    if (ov == ov) best_take(best, ov, (uint32_t)ch);
-                }
-            }
-            if (c0 + kHeadChunk < g.NG) __syncthreads();                  // part[] is reused by the next chunk
-        }
-        stamp(link, 8);
-    }
-};
-
-// A record of the phase table, read with scalar loads (the table is not written during the launch).
-__device__ __forceinline__ Phase load_phase(const Phase* table, int i) {
-    const MMF_AS_CONST Phase* p = (const MMF_AS_CONST Phase*)table + i;
-    Phase r;
-    r.w1 = p->w1; r.norm_w = p->norm_w; r.packed = p->packed; r.wdeq = p->wdeq; r.lb = p->lb; r.state = p->state;
-    r.inv_K = p->inv_K; r.eps = p->eps; r.eps1 = p->eps1; r.K = p->K; r.N = p->N; r.seg_rows = p->seg_rows; r.pad_ = 0;
-    return r;
-}
-
-template <typename T, int NPH, int NPI, int NQH, int NQI, int NGH, int NGI, bool TRACE>
-__global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
-    using C = Chain<T, NPH, NPI, NQH, NQI, NGH, NGI, TRACE>;
-    __shared__ Smem sm;
-    const uint32_t e = *a.epoch;
-    int64_t id = *a.tok;
-    if (id < 0 || id >= a.vocab) id = 0;
-    const T* emb_row = static_cast<const T*>(a.table) + id * a.H;
-    C c(a, sm, e);
-    const int L = a.n_layers;
-    const RowSrc none{nullptr, nullptr, 0u};
-
-    typename C::PreIfg pa;
-    typename C::PreO pb;
-    typename C::PreGate pc;
-    typename C::PreDown pd;
-    typename C::PreHead phd;
-
-    auto h_src = [&](int l) {        // the residual stream that enters layer l (this XCD's copy)
-        return l == 0 ? RowSrc{emb_row, nullptr, c.tag_of(-1)} : RowSrc{nullptr, ((l - 1) & 1 ? c.hb1 : c.hb0) + c.rep * a.H, c.tag_of(4 * (l - 1) + 3)};
     };
-
-    Phase p0 = load_phase(a.phases, 0);
-    Geo g0 = make_geo<3>(p0.K, p0.N, c.wave);
-    c.template prefetch<NPH, C::LD_IFG, 3, PRO_NORM, EPI_STEP, NGH>(p0, g0, pa, none, none);
+    request(KIfg{}, 0);
+    dma_norm(KIfg{}, rec(0), geo(KIfg{}, 0));
     for (int l = 0; l < L; ++l) {
         const bool last = l == L - 1;
-        const RowSrc h_in = h_src(l);
-        const Phase p1 = load_phase(a.phases, 4 * l + 1), p2 = load_phase(a.phases, 4 * l + 2), p3 = load_phase(a.phases, 4 * l + 3);
-        const Geo g1 = make_geo<1>(p1.K, p1.N, c.wave), g2 = make_geo<2>(p2.K, p2.N, c.wave), g3 = make_geo<1>(p3.K, p3.N, c.wave);
-        const RowSrc g_in{nullptr, c.gb + c.rep * a.D, c.tag_of(4 * l)}, o_in{nullptr, c.ob + c.rep * a.D, c.tag_of(4 * l)};
-        const RowSrc a_in{nullptr, c.ab + c.rep * a.H, c.tag_of(4 * l + 1)};
-        const RowSrc z_in{nullptr, c.zb + c.rep * a.I, c.tag_of(4 * l + 2)};
-        c.template link_ifg<typename C::PreO>(p0, g0, pa, h_in, 4 * l,
-                                              [&] { c.template prefetch<NPH, C::LD_O, 1, PRO_GATEDNORM, EPI_PLAIN, 1>(p1, g1, pb, none, none); });
-        c.template link_plain<NPH, C::LD_O, 1, PRO_GATEDNORM, EPI_PLAIN>(p1, g1, pb, g_in, o_in, none, none, c.ab, a.H, nullptr, 4 * l + 1,
-                                              [&] { c.template prefetch<NPH, C::LD_GATE, 2, PRO_RESNORM, EPI_SWIGLU, 1>(p2, g2, pc, none, none); });
-        c.template link_plain<NPH, C::LD_GATE, 2, PRO_RESNORM, EPI_SWIGLU>(p2, g2, pc, a_in, h_in, none, none, c.zb, a.I, nullptr, 4 * l + 2,
-                                              [&] { c.template prefetch<NPI, C::LD_DOWN, 1, PRO_PLAIN, EPI_PLAIN, 1>(p3, g3, pd, a_in, h_in); });
-        T* plain = last ? static_cast<T*>(a.h_out) : nullptr;
-        Phase pn = p0;
-        Geo gn = g0;
-        if (!last) {
-            pn = load_phase(a.phases, 4 * l + 4);
-            gn = make_geo<3>(pn.K, pn.N, c.wave);
-        } else if (a.head) {
-            pn = load_phase(a.head, 0);
-            gn = make_geo<1>(pn.K, pn.N, c.wave);
-        }
-        c.template link_plain<NPI, C::LD_DOWN, 1, PRO_PLAIN, EPI_PLAIN>(p3, g3, pd, z_in, none, a_in, h_in, (l & 1) ? c.hb1 : c.hb0, a.H, plain, 4 * l + 3,
-                                              [&] {
-                                                  if (!last) c.template prefetch<NPH, C::LD_IFG, 3, PRO_NORM, EPI_STEP, NGH>(pn, gn, pa, none, none);
-                                                  else if (a.head) c.template prefetch<NPH, C::LD_HEAD, 1, PRO_NORM, EPI_HEAD, 1>(pn, gn, phd, none, none);
-                                              });
-        p0 = pn;
-        g0 = gn;
+        link(KIfg{}, KO{}, 4 * l, true);
+        link(KO{}, KGate{}, 4 * l + 1, true);
+        link(KGate{}, KDown{}, 4 * l + 2, true);
+        if (!last) link(KDown{}, KIfg{}, 4 * l + 3, true);
+        else link(KDown{}, KHead{}, 4 * l + 3, a.head != nullptr);
     }
     if (a.head) {
-        // final norm -> lm_head: plain logits, and this workgroup's candidate for the greedy token
-        const RowSrc h_last{nullptr, ((L - 1) & 1 ? c.hb1 : c.hb0) + c.rep * a.H, c.tag_of(4 * (L - 1) + 3)};
-        const uint32_t tag_h = c.tag_of(4 * L);
-        Best best{0.0f, kNone};
-        c.link_head(p0, g0, phd, h_last, 4 * L, best, [] {});
-        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        link(KHead{}, KHead{}, 4 * L, false);
+        // this workgroup's candidate for the greedy token, then workgroup 0 combines the candidates
+        const uint32_t tag_h = tag_of(4 * L);
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) {
             const float ov = __shfl_xor(best.v, o, 64);
@@ -736,13 +777,40 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
     if (blockIdx.x == 0 && threadIdx.x == 0) *a.epoch = e + 4u * (uint32_t)a.n_layers + 2u;
 }
 
-template <typename T, bool TRACE>
-int launch_layers(const LayersArgs& a, hipStream_t s) {
-    if (a.H <= 2048 && a.I <= 6144) decode_layers_kernel<T, 2, 6, 1, 3, 1, 3, TRACE><<<kWGs, kNT, 0, s>>>(a);
-    else if (a.H <= 4096 && a.I <= 8192) decode_layers_kernel<T, 4, 8, 2, 4, 2, 4, TRACE><<<kWGs, kNT, 0, s>>>(a);
-    else return MMF_ERR_WIDE;
+template <typename T, class S, bool TRACE>
+int launch_one(const LayersArgs& a, size_t lds, hipStream_t s) {
+    auto kern = decode_layers_kernel<T, S, TRACE>;
+    static size_t allowed = 0;                                   // per instantiation; the attribute only ever grows
+    if (lds > allowed) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        allowed = lds;
+    }
+    kern<<<kWGs, kNT, lds, s>>>(a);
     MMF_CHECK_LAUNCH();
     return 0;
+}
+
+template <typename T, bool TRACE>
+int launch_layers(LayersArgs a, hipStream_t s) {
+    const int kmax = a.H > a.I ? a.H : a.I;
+    a.nqmax = quads_of(kmax);
+    // weight loads (1 KiB each) per wave a link kind needs when all its row-groups are resident: buffer A serves i/f/g
+    // and gate/up, buffer B o_proj and down_proj; the lm_head takes what they hold, pass by pass
+    const int nqh = quads_of(a.H), nqi = quads_of(a.I);
+    const int ngh = ceil_div_c(a.D / 8, kWGs), ngi = ceil_div_c(a.I / 8, kWGs);
+    const int ifg = ngh * 3 * nqh, gate = ngi * 2 * nqh, o = ngh * nqh, down = ngh * nqi;
+    a.itemsA = ifg > gate ? ifg : gate;
+    a.itemsB = o > down ? o : down;
+    if (a.itemsA > 16 || a.itemsB > 16 || ngh > 2 || ngi * 2 > kItems) return MMF_ERR_WIDE;
+    const uint32_t tab = (uint32_t)mmf_round_up((4 * a.n_layers + 1) * (int64_t)sizeof(Phase), 16);
+    a.off_q = tab;
+    a.off_nrm = a.off_q + (uint32_t)mmf_round_up(kmax, 16);
+    a.off_w = a.off_nrm + 2u * kNW * (uint32_t)a.nqmax * 1024u;
+    const size_t lds = a.off_w + (size_t)kNW * (a.itemsA + a.itemsB) * 1024u;
+    if (a.H == 2048 && a.I == 5632) return launch_one<T, StaticShape<2048, 5632>, TRACE>(a, lds, s);
+    if (a.H == 2560 && a.I == 6912) return launch_one<T, StaticShape<2560, 6912>, TRACE>(a, lds, s);
+    return launch_one<T, DynShape, TRACE>(a, lds, s);
 }
 
 int decode_layers_entry(const void* phases, int n_layers, const void* table, const int64_t* tok, int64_t vocab, uint32_t* words,
@@ -755,8 +823,8 @@ int decode_layers_entry(const void* phases, int n_layers, const void* table, con
     if (head && (!logits || !am_words || !tok_out)) return MMF_ERR_ARG;
     if (H % 128 != 0 || D != H || I % 128 != 0) return MMF_ERR_ARG;      // rows are whole k-blocks: no ragged tail in a link
     if (dtype != MMF_BF16 && dtype != MMF_F16) return MMF_ERR_ARG;        // a tagged word carries a 16-bit value
-    if (H > 4096 || I > 8192) return MMF_ERR_WIDE;
-    for (const void* p : {(const void*)words, (const void*)table, (const void*)h_out})
+    if (H > 4096 || I > 8192 || n_layers > kMaxLayers) return MMF_ERR_WIDE;
+    for (const void* p : {(const void*)words, (const void*)table, (const void*)h_out, phases, head})
         if (reinterpret_cast<uintptr_t>(p) & 15u) return MMF_ERR_ALIGN;
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
