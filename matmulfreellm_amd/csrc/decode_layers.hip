@@ -86,7 +86,8 @@ struct LayersArgs {
     uint32_t* epoch;          // tag base; advanced by 4 * n_layers + 2 at the end of the launch
     int* err;                 // set to 1 when a poll ran out of rounds
     long long* trace;         // TRACE builds: kTraceWGs * kTraceLinks * kTraceStamps cycle stamps
-    int n_layers, H, D, I, spin, delay;
+    int n_layers, H, D, I, spin;
+    int delay[5];             // hold-back of a link's first poll, per kind of link, in units of about 64 cycles
     int nqmax;                // k-quads of the widest wave slice: a wave's norm-weight region in LDS is nqmax KiB
     int itemsA, itemsB;       // 1 KiB weight loads per wave the two weight buffers hold
     uint32_t off_q, off_nrm, off_w;   // dynamic LDS: codes, norm weights (w1 regions, then the BitLinear's), weight buffers
@@ -257,6 +258,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
     float wdk[5][3] = {};
     float lb[2] = {0.0f, 0.0f}, st[2] = {0.0f, 0.0f};     // i/f/g: lower bound and recurrent state of this lane's channel, per row-group
     uint32_t a0 = 0u, a1 = 0u;                             // down: the two operands of the residual
+    u32x4 auxH[NPH] = {};                                  // gate/up: the residual stream of this wave's slice (stored links ago: fetched a link ahead)
     const int Hh = S::kStatic ? S::H : a.H, Ii = S::kStatic ? S::I : a.I;
     int8_t* const qbuf = reinterpret_cast<int8_t*>(dyn + a.off_q);
     unsigned char* const nrm_w1 = dyn + a.off_nrm;                                   // kNW regions of nqmax KiB
@@ -293,7 +295,14 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
     auto h_src = [&](int l) -> RowSrc {        // the residual stream that enters layer l (this XCD's copy)
         return l == 0 ? RowSrc{emb_row, nullptr, tag_of(-1)} : RowSrc{nullptr, ((l - 1) & 1 ? hb1 : hb0) + rep * Hh, tag_of(4 * (l - 1) + 3)};
     };
-    // One element of a row as a tagged word (a plain element gets the tag it is expected to carry).
+    // Four plain elements of a row as tagged words / one element as a tagged word (a plain element gets the tag it is
+    // expected to carry).
+    auto plain_words = [&](const RowSrc& s, int k) -> u32x4 {
+        const uint2 r = gload8(s.plain, (uint32_t)k * 2u);
+        u32x4 w;
+        w.x = (r.x << 16) | s.tag; w.y = (r.x & 0xffff0000u) | s.tag; w.z = (r.y << 16) | s.tag; w.w = (r.y & 0xffff0000u) | s.tag;
+        return w;
+    };
     auto fetch_word = [&](const RowSrc& s, int ch) -> uint32_t {
         if (s.plain) return ((uint32_t)gload2(s.plain, ch) << 16) | s.tag;
         return ll_ld4(s.words + ch);
@@ -392,6 +401,18 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
         const RowSrc none{nullptr, nullptr, 0u};
         if constexpr (KIND == K_DOWN) load_ep(kc, rc, g, RowSrc{nullptr, ab + rep * Hh, tag_of(4 * l + 1)}, h_src(l));
         else load_ep(kc, rc, g, none, none);
+        if constexpr (KIND == K_GATE) {
+            // its second operand, the residual stream, was stored three links ago: read it now, off the link's poll
+            const RowSrc hs = h_src(l);
+#pragma unroll
+            for (int v = 0; v < NPH; ++v) {
+                if (v < g.np) {
+                    const bool in = g.even || 4 * (64 * v + lane) < g.nkb * 128;
+                    const int k = g.kb0 * 128 + (in ? 4 * (64 * v + lane) : 0);
+                    auxH[v] = hs.plain ? plain_words(hs, k) : poll_issue(hs.words + k);
+                }
+            }
+        }
     };
 
     // the integer result of item `it`, row `row`: the waves' partial sums less the row's code sum (weights are stored as t + 1)
@@ -439,20 +460,15 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
             k0[v] = g.kb0 * 128 + (has[v] ? 4 * (64 * v + lane) : 0);
         }
         {
-            auto plain4 = [&](const RowSrc& s, int k) {
-                const uint2 r = gload8(s.plain, (uint32_t)k * 2u);
-                u32x4 w;
-                w.x = (r.x << 16) | s.tag; w.y = (r.x & 0xffff0000u) | s.tag; w.z = (r.y << 16) | s.tag; w.w = (r.y & 0xffff0000u) | s.tag;
-                return w;
-            };
             const bool x_tagged = xs.plain == nullptr, a_tagged = HAS_AUX && as.plain == nullptr;
             if (x_tagged || a_tagged)
-                for (int d = 0; d < a.delay; ++d) __builtin_amdgcn_s_sleep(1);
+                for (int d = 0; d < a.delay[KIND]; ++d) __builtin_amdgcn_s_sleep(1);
 #pragma unroll
             for (int v = 0; v < NPK; ++v) {
                 if (v < g.np) {
-                    X[v] = x_tagged ? poll_issue(xs.words + k0[v]) : plain4(xs, k0[v]);
-                    if constexpr (HAS_AUX) A[v] = a_tagged ? poll_issue(as.words + k0[v]) : plain4(as, k0[v]);
+                    X[v] = x_tagged ? poll_issue(xs.words + k0[v]) : plain_words(xs, k0[v]);
+                    if constexpr (KIND == K_GATE) A[v] = auxH[v];
+                    else if constexpr (HAS_AUX) A[v] = a_tagged ? poll_issue(as.words + k0[v]) : plain_words(as, k0[v]);
                 }
             }
             if (x_tagged || a_tagged) {
@@ -512,12 +528,13 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
                 for (int i = 0; i < 4; ++i) xv[v][i] = __fadd_rn(xv[v][i], av[v][i]);
         }
         if constexpr (HAS_W1) {
-            double s1 = 0.0;
+            double s1 = 0.0, s1b = 0.0;                         // two chains: half the dependent fp64 operations
 #pragma unroll
-            for (int v = 0; v < NPK; ++v)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) s1 = mmf_add_square(s1, xv[v][i]);
-            s1 = mmf_wave_sum(s1);
+            for (int v = 0; v < NPK; ++v) {
+                s1 = mmf_add_square(mmf_add_square(s1, xv[v][0]), xv[v][1]);
+                s1b = mmf_add_square(mmf_add_square(s1b, xv[v][2]), xv[v][3]);
+            }
+            s1 = mmf_wave_sum(s1 + s1b);
             if (lane == 0) sm.sum1[wave] = s1;
             float sg[KIND == K_O ? NPK : 1][4];
             if constexpr (KIND == K_O) {                          // the swish gate does not wait for the statistics
@@ -547,12 +564,13 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
         }
         stamp(ln, 2);
         // the BitLinear's own norm
-        double ss = 0.0;
+        double ss = 0.0, ssb = 0.0;
 #pragma unroll
-        for (int v = 0; v < NPK; ++v)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) ss = mmf_add_square(ss, xv[v][i]);
-        ss = mmf_wave_sum(ss);
+        for (int v = 0; v < NPK; ++v) {
+            ss = mmf_add_square(mmf_add_square(ss, xv[v][0]), xv[v][1]);
+            ssb = mmf_add_square(mmf_add_square(ssb, xv[v][2]), xv[v][3]);
+        }
+        ss = mmf_wave_sum(ss + ssb);
         if (lane == 0) sm.sum2[wave] = ss;
         lds_barrier();
         const double tot2 = (sm.sum2[0] + sm.sum2[1]) + (sm.sum2[2] + sm.sum2[3]);
@@ -625,6 +643,42 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
             if (g.nkb == 0) {
                 for (int it = lane >> 4; it < ng * g.R; it += 4)
                     if ((lane & 15) < 8) { sm.part[it][lane & 7][2 * wave] = 0; sm.part[it][lane & 7][2 * wave + 1] = 0; }
+            } else if constexpr (S::kStatic && KIND != K_HEAD) {
+                // the shape is known: every LDS read of the pass (weights, codes) is issued before the first product
+                constexpr int KK = KIND == K_DOWN ? S::I : S::H;
+                constexpr int NQ = quads_of(KK);
+                constexpr int MAXIT = ceil_div_c((KIND == K_GATE ? S::I : S::H) / 8, kWGs) * (KIND == K_IFG ? 3 : KIND == K_GATE ? 2 : 1);
+                const unsigned char* src = wbuf_of(kc, pass) + lane * 16;
+                const int nit = ng * g.R;
+                uint4 wq[MAXIT][NQ];
+                int4 qv[NQ][4];
+#pragma unroll
+                for (int q = 0; q < NQ; ++q) {
+                    const int kraw = 4 * q + slot;
+                    const int kb = g.kb0 + (g.even || kraw < g.nkb ? kraw : g.nkb - 1);
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; ++s4) qv[q][s4] = *reinterpret_cast<const int4*>(qbuf + kb * 128 + s4 * 32 + half * 16);
+                }
+#pragma unroll
+                for (int it = 0; it < MAXIT; ++it)
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) {
+                        wq[it][q] = make_uint4(0u, 0u, 0u, 0u);
+                        if (it < nit && (g.even || 4 * q + slot < g.nkb)) wq[it][q] = *reinterpret_cast<const uint4*>(src + (it * NQ + q) * 1024);
+                    }
+                int acc[MAXIT];
+#pragma unroll
+                for (int it = 0; it < MAXIT; ++it) {
+                    acc[it] = 0;
+#pragma unroll
+                    for (int q = 0; q < NQ; ++q) acc[it] = mmf_dot_block_regs(qv[q], wq[it][q], acc[it]);
+                    acc[it] += mmf_dpp<0x128>(acc[it]);                      // the other half of the 16 lanes (rotate by 8)
+                }
+#pragma unroll
+                for (int it = 0; it < MAXIT; ++it) acc[it] += __builtin_amdgcn_ds_swizzle(acc[it], 0x401F);   // lane ^ 16: the neighbouring k-block
+#pragma unroll
+                for (int it = 0; it < MAXIT; ++it)
+                    if (it < nit && (lane & 31) < 8) sm.part[it][lane & 7][2 * wave + (lane >> 5)] = acc[it];
             } else {
                 const unsigned char* src = wbuf_of(kc, pass) + lane * 16;
                 const int nit = ng * g.R;
@@ -815,11 +869,13 @@ int launch_layers(LayersArgs a, hipStream_t s) {
 
 int decode_layers_entry(const void* phases, int n_layers, const void* table, const int64_t* tok, int64_t vocab, uint32_t* words,
                         void* h_out, const void* head, void* logits, uint64_t* am_words, int64_t* tok_out, uint32_t* epoch, int* err,
-                        int64_t* trace, int H, int D, int I, int spin, int delay, int dtype, void* stream_) {
+                        int64_t* trace, int H, int D, int I, int spin, const int* delay, int dtype, void* stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (!phases || n_layers <= 0 || !table || !tok || vocab <= 0 || !words || !h_out || !epoch || !err || H <= 0 || D <= 0 || I <= 0 ||
-        spin <= 0 || delay < 0 || delay > 64)
+        spin <= 0 || !delay)
         return MMF_ERR_ARG;
+    for (int k = 0; k < 5; ++k)
+        if (delay[k] < 0 || delay[k] > 64) return MMF_ERR_ARG;
     if (head && (!logits || !am_words || !tok_out)) return MMF_ERR_ARG;
     if (H % 128 != 0 || D != H || I % 128 != 0) return MMF_ERR_ARG;      // rows are whole k-blocks: no ragged tail in a link
     if (dtype != MMF_BF16 && dtype != MMF_F16) return MMF_ERR_ARG;        // a tagged word carries a 16-bit value
@@ -834,7 +890,8 @@ int decode_layers_entry(const void* phases, int n_layers, const void* table, con
     a.phases = static_cast<const Phase*>(phases); a.n_layers = n_layers; a.table = table; a.tok = tok; a.vocab = vocab;
     a.words = words; a.h_out = h_out; a.head = static_cast<const Phase*>(head); a.logits = logits; a.am_words = am_words;
     a.tok_out = tok_out; a.epoch = epoch; a.err = err; a.trace = reinterpret_cast<long long*>(trace);
-    a.H = H; a.D = D; a.I = I; a.spin = spin; a.delay = delay;
+    a.H = H; a.D = D; a.I = I; a.spin = spin;
+    for (int k = 0; k < 5; ++k) a.delay[k] = delay[k];
     if (trace) {
         switch (dtype) {
             case MMF_BF16: return launch_layers<bf16_t, true>(a, stream);
@@ -862,10 +919,24 @@ int mmf_decode_layers_copies(void) { return kRep; }
 int mmf_decode_layers(const void* phases, int n_layers, const void* table, const int64_t* tok, int64_t vocab, uint32_t* words,
                       void* h_out, const void* head, void* logits, uint64_t* am_words, int64_t* tok_out, uint32_t* epoch, int* err,
                       int H, int D, int I, int spin, int dtype, void* stream) {
-    static const int delay = [] {
-        const char* v = getenv("MMF_DECODE_POLL_DELAY");
-        return v ? atoi(v) : 6;
-    }();
+    // hold-back of the first poll per kind of link (i/f/g, o_proj, gate/up, down_proj, lm_head); MMF_DECODE_POLL_DELAY
+    // ("a" or "a,b,c,d,e") overrides the tuned values
+    static const struct Delays {
+        int d[5] = {6, 6, 6, 6, 6};
+        Delays() {
+            const char* v = getenv("MMF_DECODE_POLL_DELAY");
+            if (!v) return;
+            int k = 0, last = 6;
+            while (*v && k < 5) {
+                last = atoi(v);
+                d[k++] = last < 0 ? 0 : last > 64 ? 64 : last;
+                while (*v && *v != ',') ++v;
+                if (*v == ',') ++v;
+            }
+            for (; k < 5; ++k) d[k] = last < 0 ? 0 : last > 64 ? 64 : last;
+        }
+    } delays;
+    const int* delay = delays.d;
     return decode_layers_entry(phases, n_layers, table, tok, vocab, words, h_out, head, logits, am_words, tok_out, epoch, err, nullptr,
                                H, D, I, spin, delay, dtype, stream);
 }
@@ -876,8 +947,9 @@ int mmf_decode_layers_traced(const void* phases, int n_layers, const void* table
                              void* h_out, const void* head, void* logits, uint64_t* am_words, int64_t* tok_out, uint32_t* epoch, int* err,
                              int64_t* trace, int H, int D, int I, int spin, int delay, int dtype, void* stream) {
     if (!trace) return MMF_ERR_ARG;
+    const int d[5] = {delay, delay, delay, delay, delay};
     return decode_layers_entry(phases, n_layers, table, tok, vocab, words, h_out, head, logits, am_words, tok_out, epoch, err, trace, H, D,
-                               I, spin, delay, dtype, stream);
+                               I, spin, d, dtype, stream);
 }
 
 }  // extern "C"

@@ -190,8 +190,7 @@ __device__ __forceinline__ void mmf_store8(T* __restrict__ p, int64_t k0, int64_
 // Cody-Waite reduction by ln2, degree-5 Horner polynomial, two-step 2^n scaling.
 // Every operation is a separately rounded fp32 add or multiply.
 __device__ __forceinline__ float mmf_exp(float x) {
-    if (x != x) return x;
-    float xc = fminf(fmaxf(x, -104.0f), 89.0f);
+    float xc = fminf(fmaxf(x, -104.0f), 89.0f);                 // a NaN argument is clamped like any other and put back at the end
     float n = rintf(__fmul_rn(xc, 1.44269504088896341f));
     float r = __fsub_rn(xc, __fmul_rn(n, 0.693359375f));
     r = __fsub_rn(r, __fmul_rn(n, -2.12194440e-4f));
@@ -210,7 +209,7 @@ __device__ __forceinline__ float mmf_exp(float x) {
     int n2 = ni - n1;
     y = __fmul_rn(y, __int_as_float((n1 + 127) << 23));
     y = __fmul_rn(y, __int_as_float((n2 + 127) << 23));
-    return y;
+    return x != x ? x : y;                                       // a select, not a branch
 }
 
 // 1 / (1 + exp(-x))
@@ -315,6 +314,19 @@ __device__ __forceinline__ int mmf_dot_block(const int8_t* q_lds, const uint4& w
         acc = __builtin_amdgcn_sdot4((int)((w >> 2) & 0x03030303u), qv.y, acc, false);
         acc = __builtin_amdgcn_sdot4((int)((w >> 4) & 0x03030303u), qv.z, acc, false);
         acc = __builtin_amdgcn_sdot4((int)((w >> 6) & 0x03030303u), qv.w, acc, false);
+    }
+    return acc;
+}
+
+// The same with the 128 codes of the k-block already in registers (qv[s] = the lane's 16 codes of k-step s).
+__device__ __forceinline__ int mmf_dot_block_regs(const int4 (&qv)[4], const uint4& wq, int acc) {
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) {
+        const uint32_t w = s4 == 0 ? wq.x : s4 == 1 ? wq.y : s4 == 2 ? wq.z : wq.w;
+        acc = __builtin_amdgcn_sdot4((int)(w & 0x03030303u), qv[s4].x, acc, false);
+        acc = __builtin_amdgcn_sdot4((int)((w >> 2) & 0x03030303u), qv[s4].y, acc, false);
+        acc = __builtin_amdgcn_sdot4((int)((w >> 4) & 0x03030303u), qv[s4].z, acc, false);
+        acc = __builtin_amdgcn_sdot4((int)((w >> 6) & 0x03030303u), qv[s4].w, acc, false);
     }
     return acc;
 }
