@@ -174,7 +174,8 @@ def link_trace_bench(model, dev, delay=6):
     out = {"unit": "shader clock cycles (s_memtime), mean over layers 2.. of one step", "stages": stages, "poll_delay": delay,
            "workgroups": {}}
     nl = 4 * eng.L
-    for slot, wg in enumerate((0, 37, 200)):
+    for wg in (0, 37, 200):
+        slot = wg
         per = {}
         for kind in range(4):
             rows = t[slot, kind:nl:4, :9][2:]

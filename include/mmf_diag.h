@@ -27,8 +27,8 @@ int mmf_mfma_pipe_probe(int64_t steps, int64_t workgroups, int random_operands, 
 
 /* mmf_decode_layers_traced: mmf_decode_layers (see mmf.h) built with its cycle trace, and with the hold-back of a link's
  *   first poll as an argument (`delay`, in units of about 64 cycles, 0..64).
- *   trace: mmf_decode_layers_trace_words() int64 words (zeroed by the caller): thread 0 of workgroups 0, 37 and 200 stores
- *   the shader clock at points of each of the first 128 links, [workgroup][link][12]: 0 link entered, 1 input row arrived,
+ *   trace: mmf_decode_layers_trace_words() int64 words (zeroed by the caller): thread 0 of every workgroup stores the
+ *   shader clock at points of each of the first 128 links, [256 workgroups][link][12]: 0 link entered, 1 input row arrived,
  *   2 block norm applied, 3 second sum of squares reduced, 4 absmax reduced, 5 codes in LDS, 6 dot products done,
  *   7 partial sums met, 8 epilogue stored.  The product launch carries none of this. */
 int mmf_decode_layers_trace_words(void);

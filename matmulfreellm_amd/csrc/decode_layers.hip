@@ -93,7 +93,7 @@ struct LayersArgs {
     uint32_t off_q, off_nrm, off_w;   // dynamic LDS: codes, norm weights (w1 regions, then the BitLinear's), weight buffers
 };
 
-constexpr int kTraceWGs = 3, kTraceLinks = 128, kTraceStamps = 12;
+constexpr int kTraceWGs = 256, kTraceLinks = 128, kTraceStamps = 12;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -275,8 +275,10 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
     auto stamp = [&](int link, int i) {
         if constexpr (TRACE) {
             if (threadIdx.x == 0 && link < kTraceLinks) {
-                const int s = blockIdx.x == 0 ? 0 : blockIdx.x == 37 ? 1 : blockIdx.x == 200 ? 2 : -1;
-                if (s >= 0) a.trace[(s * kTraceLinks + link) * kTraceStamps + i] = __builtin_amdgcn_s_memtime();
+                long long* t = a.trace + ((int)blockIdx.x * kTraceLinks + link) * kTraceStamps;
+                t[i] = __builtin_amdgcn_s_memtime();
+                // entry, arrival and end of the link also on the 100 MHz clock all XCDs share (slots 9-11)
+                if (i == 0 || i == 1 || i == 8) t[i == 0 ? 9 : i == 1 ? 10 : 11] = __builtin_amdgcn_s_memrealtime();
             }
         }
     };
@@ -429,8 +431,22 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
     };
 
     // ---- one link.  NEXT: the kind of the link that follows (its requests are made here, once this link's row is in).
-    auto link = [&](auto kc, auto nc, int ln, bool more) {
-        constexpr int KIND = decltype(kc)::value, NEXT = decltype(nc)::value;
+    // kc: the kind of this link; nc: the kind of the link that follows (its requests are made here, once this link's row
+    // is in); nc2: the kind that follows instead when `alt` is set (the lm_head after the last down_proj)
+    auto link = [&](auto kc, auto nc, auto nc2, bool alt, int ln, bool more) {
+        constexpr int KIND = decltype(kc)::value;
+        auto request_next = [&] {
+            if constexpr (decltype(nc)::value != decltype(nc2)::value) {
+                if (alt) { request(nc2, ln + 1); return; }
+            }
+            request(nc, ln + 1);
+        };
+        auto dma_norm_next = [&] {
+            if constexpr (decltype(nc)::value != decltype(nc2)::value) {
+                if (alt) { dma_norm(nc2, rec(ln + 1), geo(nc2, ln + 1)); return; }
+            }
+            dma_norm(nc, rec(ln + 1), geo(nc, ln + 1));
+        };
         constexpr bool HAS_AUX = KIND == K_O || KIND == K_GATE, HAS_W1 = KIND != K_DOWN;
         constexpr int NPK = KIND == K_DOWN ? NP : NPH;                       // passes this link's row can take
         const int l = ln >> 2;
@@ -438,7 +454,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
         stamp(ln, 0);
         if (g.NG == 0) {
             // nothing of this link falls to this workgroup; it still requests what its next link needs
-            if (more) { request(nc, ln + 1); dma_norm(nc, rec(ln + 1), geo(nc, ln + 1)); }
+            if (more) { request_next(); dma_norm_next(); }
             return;
         }
         const unsigned char* rc = rec(ln);
@@ -503,8 +519,8 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
         // every load made so far has been waited for (said explicitly: the requests below are not to be waited for here)
         __builtin_amdgcn_s_waitcnt(0x0F70);
         stamp(ln, 1);
-        // ---- the row is here: now request what the next link needs
-        if (more) request(nc, ln + 1);
+        // ---- the row is here: from now on what the next link needs may be requested (it is, below, in the shadow of the
+        // first exchange of partial sums)
 
         // ---- prologue: norms, absmax int8 codes of this wave's slice into LDS
         float xv[NPK][4], av[HAS_AUX ? NPK : 1][4];
@@ -543,6 +559,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) sg[v][i] = v < g.np ? mmf_sigmoid(av[v][i]) : 0.0f;
             }
+            if (more) request_next();                             // while the partial sums settle in LDS
             lds_barrier();
             const double tot = (sm.sum1[0] + sm.sum1[1]) + (sm.sum1[2] + sm.sum1[3]);
             const float rstd1 = mmf_rstd(tot, g.K, inv_K, __uint_as_float(uni32(rc + 60)));
@@ -572,6 +589,9 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
         }
         ss = mmf_wave_sum(ss + ssb);
         if (lane == 0) sm.sum2[wave] = ss;
+        if constexpr (!HAS_W1) {
+            if (more) request_next();
+        }
         lds_barrier();
         const double tot2 = (sm.sum2[0] + sm.sum2[1]) + (sm.sum2[2] + sm.sum2[3]);
         const float rstd = mmf_rstd(tot2, g.K, inv_K, __uint_as_float(uni32(rc + 56)));
@@ -593,7 +613,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
             }
         }
         // this wave is done with its norm-weight regions: the next link's may come in
-        if (more) dma_norm(nc, rec(ln + 1), geo(nc, ln + 1));
+        if (more) dma_norm_next();
         amax = mmf_wave_max(amax);
         if (lane == 0) sm.amax[wave] = amax;
         lds_barrier();
@@ -776,14 +796,13 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
     dma_norm(KIfg{}, rec(0), geo(KIfg{}, 0));
     for (int l = 0; l < L; ++l) {
         const bool last = l == L - 1;
-        link(KIfg{}, KO{}, 4 * l, true);
-        link(KO{}, KGate{}, 4 * l + 1, true);
-        link(KGate{}, KDown{}, 4 * l + 2, true);
-        if (!last) link(KDown{}, KIfg{}, 4 * l + 3, true);
-        else link(KDown{}, KHead{}, 4 * l + 3, a.head != nullptr);
+        link(KIfg{}, KO{}, KO{}, false, 4 * l, true);
+        link(KO{}, KGate{}, KGate{}, false, 4 * l + 1, true);
+        link(KGate{}, KDown{}, KDown{}, false, 4 * l + 2, true);
+        link(KDown{}, KIfg{}, KHead{}, last, 4 * l + 3, !last || a.head != nullptr);
     }
     if (a.head) {
-        link(KHead{}, KHead{}, 4 * L, false);
+        link(KHead{}, KHead{}, KHead{}, false, 4 * L, false);
         // this workgroup's candidate for the greedy token, then workgroup 0 combines the candidates
         const uint32_t tag_h = tag_of(4 * L);
 #pragma unroll
@@ -922,7 +941,7 @@ int mmf_decode_layers(const void* phases, int n_layers, const void* table, const
     // hold-back of the first poll per kind of link (i/f/g, o_proj, gate/up, down_proj, lm_head); MMF_DECODE_POLL_DELAY
     // ("a" or "a,b,c,d,e") overrides the tuned values
     static const struct Delays {
-        int d[5] = {6, 6, 6, 6, 6};
+        int d[5] = {8, 14, 14, 22, 8};
         Delays() {
             const char* v = getenv("MMF_DECODE_POLL_DELAY");
             if (!v) return;

@@ -218,13 +218,13 @@ class DecodeEngine:
                                                       L.stream()), "mmf_decode_layers_traced")
 
     def link_trace(self, delay: int = 6) -> torch.Tensor:
-        """One resident step with the kernel's cycle trace on: int64 [3 workgroups, 128 links, 12 stamps] (see
+        """One resident step with the kernel's cycle trace on: int64 [256 workgroups, 128 links, 12 stamps] (see
         mmf_decode_layers_traced in include/mmf_diag.h), on the host."""
         assert self.resident
         t = torch.zeros(self.lib.mmf_decode_layers_trace_words(), dtype=torch.int64, device=self.dev)
         self._launch_layers(True, trace=t, delay=delay)
         torch.cuda.synchronize(self.dev)
-        return t.view(3, 128, 12).cpu()
+        return t.view(256, 128, 12).cpu()
 
     def _launch_step_resident(self):
         self._launch_layers(True)       # the whole step: final norm, lm_head and argmax are the launch's last two links

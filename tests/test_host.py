@@ -211,7 +211,7 @@ def test_rejected_shapes_and_pointers_return_their_code_before_any_launch():
                                         None) == -1               # the traced form needs its trace buffer
     assert lib.mmf_decode_layers_copies() == 8
     assert lib.mmf_decode_layers_words(512, 512, 1536) == 8 * (5 * 512 + 1536)
-    assert lib.mmf_decode_layers_trace_words() == 3 * 128 * 12
+    assert lib.mmf_decode_layers_trace_words() == 256 * 128 * 12
     assert lib.mmf_decode_layers_phase_bytes() == 80
 
 
