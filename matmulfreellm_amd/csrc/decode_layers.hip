@@ -424,10 +424,11 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
         const int4 qv = *reinterpret_cast<const int4*>(&sm.qs[0]);
         return ((p0.x + p0.y) + (p0.z + p0.w)) + ((p1.x + p1.y) + (p1.z + p1.w)) - ((qv.x + qv.y) + (qv.z + qv.w));
     };
-    // Two neighbouring rows' words become one 8-byte store by the even row (fewer, wider stores travel faster).
-    auto store_pair = [&](uint32_t* base, int ch, uint32_t word, bool active) {
+    // Two neighbouring rows' words become one 8-byte store by the even row (fewer, wider stores travel faster); `even_active`:
+    // this lane holds an even row that is to be stored.
+    auto store_pair = [&](uint32_t* base, int ch, uint32_t word, bool even_active) {
         const uint32_t next = (uint32_t)mmf_dpp<kDppXor1>((int)word);
-        if (active && !(lane & 1)) ll_st8(reinterpret_cast<uint64_t*>(base + ch), (uint64_t)word | ((uint64_t)next << 32));
+        if (even_active) ll_st8(reinterpret_cast<uint64_t*>(base + ch), (uint64_t)word | ((uint64_t)next << 32));
     };
 
     // ---- one link.  NEXT: the kind of the link that follows (its requests are made here, once this link's row is in).
@@ -435,6 +436,11 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
     // is in); nc2: the kind that follows instead when `alt` is set (the lm_head after the last down_proj)
     auto link = [&](auto kc, auto nc, auto nc2, bool alt, int ln, bool more) {
         constexpr int KIND = decltype(kc)::value;
+        // The lane index as this link sees it.  Made opaque per link: tests on it (lane 0, the epilogue lanes, the even rows)
+        // are then a compare where they are used, not masks kept in scalar registers across the whole layer loop, where
+        // there are too many of them and they end up spilled and reloaded lane by lane.
+        int pl = lane;
+        asm volatile("" : "+v"(pl));
         auto request_next = [&] {
             if constexpr (decltype(nc)::value != decltype(nc2)::value) {
                 if (alt) { request(nc2, ln + 1); return; }
@@ -501,7 +507,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
                     }
                     if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
                     if (n >= a.spin) {
-                        if (lane == 0) *a.err = 1;
+                        if (pl == 0) *a.err = 1;
                         break;
                     }
 #pragma unroll
@@ -551,7 +557,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
                 s1b = mmf_add_square(mmf_add_square(s1b, xv[v][2]), xv[v][3]);
             }
             s1 = mmf_wave_sum(s1 + s1b);
-            if (lane == 0) sm.sum1[wave] = s1;
+            if (pl == 0) sm.sum1[wave] = s1;
             float sg[KIND == K_O ? NPK : 1][4];
             if constexpr (KIND == K_O) {                          // the swish gate does not wait for the statistics
 #pragma unroll
@@ -588,7 +594,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
             ssb = mmf_add_square(mmf_add_square(ssb, xv[v][2]), xv[v][3]);
         }
         ss = mmf_wave_sum(ss + ssb);
-        if (lane == 0) sm.sum2[wave] = ss;
+        if (pl == 0) sm.sum2[wave] = ss;
         if constexpr (!HAS_W1) {
             if (more) request_next();
         }
@@ -615,7 +621,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
         // this wave is done with its norm-weight regions: the next link's may come in
         if (more) dma_norm_next();
         amax = mmf_wave_max(amax);
-        if (lane == 0) sm.amax[wave] = amax;
+        if (pl == 0) sm.amax[wave] = amax;
         lds_barrier();
         amax = fmaxf(fmaxf(sm.amax[0], sm.amax[1]), fmaxf(sm.amax[2], sm.amax[3]));
         stamp(ln, 4);
@@ -632,7 +638,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
             }
         }
         qs = mmf_wave_sum(qs);
-        if (lane == 0) sm.qs[wave] = qs;
+        if (pl == 0) sm.qs[wave] = qs;
         const float deq = __fdiv_rn(1.0f, scale);       // needed by the epilogue only
         stamp(ln, 5);
 
@@ -662,7 +668,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
             __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
             if (g.nkb == 0) {
                 for (int it = lane >> 4; it < ng * g.R; it += 4)
-                    if ((lane & 15) < 8) { sm.part[it][lane & 7][2 * wave] = 0; sm.part[it][lane & 7][2 * wave + 1] = 0; }
+                    if ((pl & 15) < 8) { sm.part[it][pl & 7][2 * wave] = 0; sm.part[it][pl & 7][2 * wave + 1] = 0; }
             } else if constexpr (S::kStatic && KIND != K_HEAD) {
                 // the shape is known: every LDS read of the pass (weights, codes) is issued before the first product
                 constexpr int KK = KIND == K_DOWN ? S::I : S::H;
@@ -698,7 +704,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
                 for (int it = 0; it < MAXIT; ++it) acc[it] += __builtin_amdgcn_ds_swizzle(acc[it], 0x401F);   // lane ^ 16: the neighbouring k-block
 #pragma unroll
                 for (int it = 0; it < MAXIT; ++it)
-                    if (it < nit && (lane & 31) < 8) sm.part[it][lane & 7][2 * wave + (lane >> 5)] = acc[it];
+                    if (it < nit && (pl & 31) < 8) sm.part[it][pl & 7][2 * wave + (pl >> 5)] = acc[it];
             } else {
                 const unsigned char* src = wbuf_of(kc, pass) + lane * 16;
                 const int nit = ng * g.R;
@@ -717,7 +723,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
                     }
                     acc += mmf_dpp<0x128>(acc);                              // the other half of the 16 lanes (rotate by 8)
                     acc += __builtin_amdgcn_ds_swizzle(acc, 0x401F);         // lane ^ 16: the neighbouring k-block
-                    if ((lane & 31) < 8) sm.part[it][lane & 7][2 * wave + (lane >> 5)] = acc;
+                    if ((pl & 31) < 8) sm.part[it][pl & 7][2 * wave + (pl >> 5)] = acc;
                 }
             }
             stamp(ln, 6);
@@ -728,7 +734,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
                 // a wave serves two copies: lanes 0-23 of each 32-lane half run the i, f and g rows of the 8 channels side
                 // by side, so the two exp / divide chains of the gate math run in parallel; the f lanes' gate reaches the i
                 // lanes by a rotate within the 16-lane row.  Operation for operation the arithmetic of the single-lane form.
-                const int r3 = (lane & 31) >> 3, row = lane & 7, copy = 2 * wave + (lane >> 5);
+                const int r3 = (pl & 31) >> 3, row = pl & 7, copy = 2 * wave + (pl >> 5);
                 const void* lbp = reinterpret_cast<const void*>(uni64(rc + 32));
                 float* stp = reinterpret_cast<float*>(uni64(rc + 40));
 #pragma unroll
@@ -748,12 +754,12 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
                     const float h = __fadd_rn(__fmul_rn(go, stv), xo);
                     const bool live = ch < g.Nseg;
                     if (live && r3 == 0 && copy == 0) ((MMF_AS_GLOBAL float*)stp)[ch] = h;
-                    store_pair(ob + copy * Hh, ch, make_word<T>(h, tag), live && r3 == 0);
-                    store_pair(gb + copy * Hh, ch, make_word<T>(res, tag), live && r3 == 2);
+                    store_pair(ob + copy * Hh, ch, make_word<T>(h, tag), live && r3 == 0 && !(pl & 1));
+                    store_pair(gb + copy * Hh, ch, make_word<T>(res, tag), live && r3 == 2 && !(pl & 1));
                 }
             } else if constexpr (KIND == K_HEAD) {
-                const int row = lane & 7;                                 // a wave takes 8 row-groups of a pass
-                for (int gl = wave * 8 + (lane >> 3); gl < ng; gl += 8 * kNW) {
+                const int row = pl & 7;                                   // a wave takes 8 row-groups of a pass
+                for (int gl = wave * 8 + (pl >> 3); gl < ng; gl += 8 * kNW) {
                     const int ch = ((int)blockIdx.x + kWGs * (g0 + gl)) * 8 + row;
                     if (ch < g.Nseg) {
                         const float o = __fmul_rn(__fmul_rn((float)total(gl, row), deq), wdk[KIND][0]);
@@ -764,7 +770,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
                 }
             } else {
                 // 8 x 8 lanes are copy x row, one row-group per wave: o_proj, gate/up, down
-                const int row = lane & 7, copy = lane >> 3;
+                const int row = pl & 7, copy = pl >> 3;
                 uint32_t* out = KIND == K_O ? ab : KIND == K_GATE ? zb : ((l & 1) ? hb1 : hb0);
                 const int out_n = KIND == K_GATE ? Ii : Hh;
                 for (int gl = wave; gl < ng; gl += kNW) {
@@ -784,7 +790,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
                         if (live) { r0 = finish_word(w0, add0, ch); r1 = finish_word(w1, add1, ch); }
                         o = __fadd_rn(mmf_round_to<T>(o), mmf_round_to<T>(__fadd_rn(r0, r1)));
                     }
-                    store_pair(out + copy * out_n, ch, make_word<T>(o, tag), live);
+                    store_pair(out + copy * out_n, ch, make_word<T>(o, tag), live && !(pl & 1));
                     if (KIND == K_DOWN && l == L - 1 && live && copy == 0) static_cast<T*>(a.h_out)[ch] = mmf_from_float<T>(o);
                 }
             }
