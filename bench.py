@@ -23,7 +23,7 @@ inputs resident in HBM.  Prints ONE JSON line:
                HGRN scan, norm and loss bandwidths (cache-cold: the legs rotate through buffer sets
                of more than 512 MB in total; counted HBM traffic from rocprofv3 beside each),
                and one training step (forward + loss + backward) of the same model at 8 x 1024 tokens.
---only runs the named legs only (decode, bs64, prefill, mfma, scan, norms, sampling, loss, train, cpu, link_trace): the
+--only runs the named legs only (decode, bs64, prefill, mfma, gemv_stream, scan, norms, sampling, loss, train, cpu, link_trace): the
 profiles under profiles/ are made that way.
 Synthetic data: random-init N(0, 0.02) weights, uniform random token ids.
 """
@@ -86,7 +86,8 @@ def decode_bench(model, batch, steps, warmup, dev, prompt_len=128, resident=None
     import matmulfreellm_amd.functional as F_
     g = torch.Generator(device=dev).manual_seed(1)
     ids = torch.randint(0, model.config.vocab_size, (batch, prompt_len), generator=g, device=dev)
-    out = model(input_ids=ids, use_cache=True, logits_to_keep=1)
+    with torch.no_grad():
+        out = model(input_ids=ids, use_cache=True, logits_to_keep=1)
     first = F_.argmax(out.logits[:, -1])
     eng = DecodeEngine.for_model(model, batch, use_graph=True, resident=resident)
     eng.load_state([c[-1] for c in out.past_key_values])
@@ -154,6 +155,34 @@ def gemv_roofline(eng, iters=20):
             "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH if counted else None,
             "launches_per_step": n, "algorithmic_bytes_per_launch": total_bytes // n,
             "avg_launch_us": round(us_per_launch, 3)}
+
+
+def gemv_stream_bench(dev, n=600000, k=2048, iters=12):
+    """The batch-1 fused BitLinear kernel with nothing but HBM in its way: one launch over n x k packed ternary
+    weights (n * k / 4 bytes, past 300 MB), two such operands alternating so that no launch finds its weights in the
+    256 MB last-level cache, every launch independent of the others (same input row, outputs never read).  This is
+    the rate the kernel's load path and dot reach when no hand-off waits on it."""
+    import matmulfreellm_amd.functional as F_
+    g = torch.Generator(device=dev).manual_seed(12)
+    pws = []
+    for _ in range(2):
+        w = torch.empty(n, k, device=dev, dtype=torch.bfloat16).normal_(0.0, 0.02, generator=g)
+        pws.append(F_.ternarize_pack(w))
+        del w
+    x = torch.randn(1, k, generator=g, device=dev).bfloat16()
+    nw = torch.ones(k, device=dev, dtype=torch.bfloat16)
+    turn = [0]
+
+    def launch():
+        turn[0] ^= 1
+        return F_.bitlinear_gemv(x, nw, pws[turn[0]], 1e-8)
+    ms = timed(launch, iters, warmup=4)
+    packed = pws[0].packed.numel()
+    nbytes = packed + 2 * k * 2 + n * 2            # packed weights, input row and norm weight, output row
+    gbs = nbytes / ms / 1e6
+    return {"kernel": "bitlinear_gemv_kernel", "M": 1, "N": n, "K": k, "packed_weight_bytes": packed, "operands_alternating": 2,
+            "algorithmic_bytes_per_launch": nbytes, "avg_launch_us": round(ms * 1e3, 2), "GBs": round(gbs, 1),
+            "frac_of_hbm": round(gbs / HBM_PEAK_GBS, 4), "counted_fetch_bytes_per_launch": COUNTED_TRAFFIC.get("gemv_stream")}
 
 
 def link_trace_bench(model, dev, delay=6):
@@ -504,7 +533,7 @@ def main():
     ap.add_argument("--launch-chain", action="store_true",
                     help="batch 1: one launch per fused BitLinear instead of the resident layer chain")
     ap.add_argument("--no-extra", action="store_true", help="skip the batch-64 / matrix-core / scan / norm / CPU legs")
-    ap.add_argument("--only", default="", help="comma-separated legs to run instead of everything: decode, bs64, prefill, mfma, "
+    ap.add_argument("--only", default="", help="comma-separated legs to run instead of everything: decode, bs64, prefill, mfma, gemv_stream, "
                                                "scan, norms, sampling, loss, train, cpu, link_trace (profiling runs)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by)")
@@ -533,6 +562,8 @@ def main():
             res["bitlinear_mfma_down_proj"] = mfma_bench(dev, 4096, 5632, 2048)
             res["matrix_pipe_alone_random_operands"] = mfma_pipe_bench(dev, True)
             res["matrix_pipe_alone_constant_operands"] = mfma_pipe_bench(dev, False)
+        if "gemv_stream" in only:
+            res["gemv_stream"] = gemv_stream_bench(dev)
         if "scan" in only:
             res["hgrn_scan"] = scan_bench(dev)
         if "norms" in only:
@@ -587,6 +618,8 @@ def main():
         extra["bitlinear_mfma_down_proj"] = mfma_bench(dev, 4096, 5632, 2048)
         extra["matrix_pipe_alone_random_operands"] = mfma_pipe_bench(dev, True)
         extra["matrix_pipe_alone_constant_operands"] = mfma_pipe_bench(dev, False)
+    if want("gemv_stream"):
+        extra["gemv_stream"] = gemv_stream_bench(dev)
     if want("scan"):
         extra["hgrn_scan"] = scan_bench(dev)
     if want("norms"):

@@ -16,6 +16,7 @@ import torch
 import torch.nn as nn
 
 from . import functional as F_
+from .autograd import module_needs_grad
 from .bitlinear import FusedBitLinear as BitLinear
 from .fused_norm_gate import FusedRMSNormSwishGate
 
@@ -25,7 +26,7 @@ class HGRNBitAttention(nn.Module):
     def __init__(self, mode: str = "fused_recurrent", hidden_size: int = 1024, num_heads: Optional[int] = None,
                  expand_ratio: Optional[int] = 1, use_short_conv: bool = False, conv_size: int = 4,
                  conv_bias: bool = False, share_conv_kernel: bool = True, layernorm_eps: float = 1e-5,
-                 layer_idx: int = None):
+                 layer_idx: int = None, bitlinear_eps: Optional[float] = 1e-6):
         super().__init__()
         if num_heads is None:
             num_heads = 1
@@ -44,9 +45,9 @@ class HGRNBitAttention(nn.Module):
         assert mode in ["fused_recurrent", "chunk"], f"Not supported mode `{mode}`."
         assert self.hidden_size % num_heads == 0, f"hidden size must be divisible by num_heads of {num_heads}"
 
-        self.i_proj = BitLinear(hidden_size, self.input_dim, bias=False)
-        self.f_proj = BitLinear(hidden_size, self.input_dim, bias=False)
-        self.g_proj = BitLinear(hidden_size, self.input_dim, bias=False)
+        self.i_proj = BitLinear(hidden_size, self.input_dim, bias=False, fused_eps=bitlinear_eps)
+        self.f_proj = BitLinear(hidden_size, self.input_dim, bias=False, fused_eps=bitlinear_eps)
+        self.g_proj = BitLinear(hidden_size, self.input_dim, bias=False, fused_eps=bitlinear_eps)
         if use_short_conv:
             # mmfreelm/layers/hgrn_bit.py:60-67.  The reference's forward cannot run with this option (it hands
             # ShortConvolution.forward(x, cache) three positionals, :101/:107-108); here the evident intent runs:
@@ -60,7 +61,7 @@ class HGRNBitAttention(nn.Module):
                 self.f_conv1d = ShortConvolution(self.input_dim, conv_size, activation="silu")
                 self.i_conv1d = ShortConvolution(self.input_dim, conv_size, activation="silu")
         self.g_norm = FusedRMSNormSwishGate(self.input_dim, layernorm_eps)
-        self.o_proj = BitLinear(self.input_dim, hidden_size, bias=False)
+        self.o_proj = BitLinear(self.input_dim, hidden_size, bias=False, fused_eps=bitlinear_eps)
         self.apply(self._initialize_weights)
         self._ifg_key, self._ifg = None, None
 
@@ -97,7 +98,7 @@ class HGRNBitAttention(nn.Module):
         D = self.input_dim
         if self.use_short_conv:
             return self._forward_short_conv(hidden_states, attention_mask, past_key_values, use_cache, lower_bound, input_norm)
-        if self.training and torch.is_grad_enabled():
+        if module_needs_grad(self, hidden_states, lower_bound):
             return self._forward_train(hidden_states, attention_mask, lower_bound, input_norm), None, past_key_values
         last_state = past_key_values[self.layer_idx] if use_cache else None
 
@@ -124,8 +125,7 @@ class HGRNBitAttention(nn.Module):
             x_in, gate = F_.hgrn_gate(i, f, lb, attention_mask)
             x4, g4 = x_in.view(B, 1, T, D), gate.view(B, 1, T, D)      # heads are independent channels
             h0 = recurrent_state.reshape(B, 1, D) if recurrent_state is not None else None
-            if self.mode == "chunk" and T > 1:
-                raise NotImplementedError("chunk mode takes log-domain gates; the model path uses fused_recurrent")
+            self._check_mode(T)
             o, new_state = F_.hgrn_recurrent(x4, g4, initial_state=h0, output_final_state=bool(use_cache))
             o = o.view(B, T, D)
             if use_cache:
@@ -137,6 +137,12 @@ class HGRNBitAttention(nn.Module):
         # g_norm (layers/hgrn_bit.py:138) folded into o_proj
         o = self.o_proj.forward_fused(g, ("gatednorm", o.reshape(g.shape), self.g_norm.weight, self.g_norm.eps))
         return o, None, past_key_values
+
+    def _check_mode(self, T):
+        """mmfreelm/layers/hgrn_bit.py:130-134 runs fused_recurrent only and raises for any other mode; the same here, in every
+        path (inference, training, short convolutions): chunk_hgrn takes log-domain gates, which this layer does not form."""
+        if self.mode != "fused_recurrent" and T > 1:
+            raise NotImplementedError(f"Not supported mode `{self.mode}`: the model path uses fused_recurrent")
 
     def _forward_train(self, hidden_states, attention_mask, lower_bound, input_norm):
         """The layer as the reference composes it (mmfreelm/layers/hgrn_bit.py:110-140), one autograd Function per op;
@@ -150,6 +156,7 @@ class HGRNBitAttention(nn.Module):
         i, f, g = self.i_proj(hidden_states), self.f_proj(hidden_states), self.g_proj(hidden_states)
         lb = lower_bound if (lower_bound is not None and self.layer_idx > 0) else None
         x_in, gate = HGRNGateFn.apply(i, f, lb, attention_mask)
+        self._check_mode(T)
         o, _ = fused_recurrent_hgrn(x_in.view(B, 1, T, D), gate.view(B, 1, T, D))
         o = self.g_norm(g, o.view(B, T, D))
         return self.o_proj(o)
@@ -164,15 +171,23 @@ class HGRNBitAttention(nn.Module):
         if input_norm is not None:
             hidden_states = input_norm(hidden_states)
         last_state = past_key_values[self.layer_idx] if use_cache else None
+        # Left padding: what enters a convolution (and its cache) at a padded position is zeroed, so that a pad token cannot
+        # leak into the first real positions through the convolution window.  The reference cannot run this path (its call
+        # passes the mask where the cache belongs), so there is nothing to compare with: parity unpinned.
+        keep = attention_mask.reshape(B, T).to(hidden_states.dtype).unsqueeze(-1) if attention_mask is not None else None
         if self.share_conv_kernel:
             conv_state = last_state[0] if use_cache else None
-            hidden_states = self.h_conv1d(hidden_states, conv_state)          # the conv state is updated in place
+            conv_in = hidden_states if keep is None else hidden_states * keep
+            hidden_states = self.h_conv1d(conv_in, conv_state)                # the conv state is updated in place
             i, f = self.i_proj(hidden_states), self.f_proj(hidden_states)
         else:
             conv_state_i = last_state[0] if use_cache else None
             conv_state_f = last_state[1] if use_cache else None
-            i = self.i_conv1d(self.i_proj(hidden_states), conv_state_i)
-            f = self.f_conv1d(self.f_proj(hidden_states), conv_state_f)
+            pi, pf = self.i_proj(hidden_states), self.f_proj(hidden_states)
+            if keep is not None:
+                pi, pf = pi * keep, pf * keep
+            i = self.i_conv1d(pi, conv_state_i)
+            f = self.f_conv1d(pf, conv_state_f)
         lb = lower_bound if (lower_bound is not None and self.layer_idx > 0) else None
         if needs_grad(i, f, lb):
             x_in, gate = HGRNGateFn.apply(i, f, lb, attention_mask)
@@ -180,6 +195,7 @@ class HGRNBitAttention(nn.Module):
             x_in, gate = F_.hgrn_gate(i, f, lb, attention_mask)
         recurrent_state = last_state[-1] if use_cache else None
         h0 = recurrent_state.reshape(B, 1, D) if recurrent_state is not None else None
+        self._check_mode(T)
         o, new_state = fused_recurrent_hgrn(x_in.view(B, 1, T, D), gate.view(B, 1, T, D), initial_state=h0,
                                             output_final_state=bool(use_cache))
         if past_key_values is not None and use_cache:

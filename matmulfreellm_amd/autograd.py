@@ -25,6 +25,13 @@ def needs_grad(*tensors) -> bool:
     return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
 
 
+def module_needs_grad(module, *inputs) -> bool:
+    """The rule every module uses to pick the differentiable path: gradients are enabled and an input or one of the module's
+    parameters requires one -- whatever module.training says (the reference differentiates in eval mode too)."""
+    return torch.is_grad_enabled() and (any(t is not None and t.requires_grad for t in inputs)
+                                        or any(p.requires_grad for p in module.parameters()))
+
+
 def _2d(t):
     return t.reshape(-1, t.shape[-1])
 

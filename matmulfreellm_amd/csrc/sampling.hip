@@ -169,7 +169,8 @@ __global__ __launch_bounds__(kSampThreads) void sample_top_p_kernel(SampleArgs a
     for (int w = 0; w < kSampWaves; ++w) mx = fmaxf(mx, wmax[w]);
 
     unsigned m[NPT];
-    if (a.top_k > 0 && a.top_k < V) {
+    if (a.top_k > 0 && a.top_k < V && mx != -INFINITY) {          // a row without a finite logit has no top_k-th largest: it is drawn
+                                                                   // uniformly like without the limit (every mass is 2^31)
         // order-preserving image of the scaled logits: non-negative floats above the negative ones, -inf and the slots
         // past V at 0 (which the descent ignores)
 #pragma unroll

@@ -28,6 +28,7 @@ from transformers.modeling_utils import PreTrainedModel
 from . import functional as F_
 from .activations import swiglu
 from .attention import HGRNBitAttention
+from .autograd import module_needs_grad
 from .bitlinear import FusedBitLinear as BitLinear
 from .cache import RecurrentCache
 from .configuration_hgrn_bit import HGRNBitConfig
@@ -47,7 +48,7 @@ def lower_bound_schedule(lower_bounds: torch.Tensor) -> torch.Tensor:
 class HGRNBitMLP(nn.Module):
 
     def __init__(self, hidden_size: int, hidden_ratio: Optional[int] = None, intermediate_size: Optional[int] = None,
-                 hidden_act: str = "swish"):
+                 hidden_act: str = "swish", bitlinear_eps: Optional[float] = 1e-6):
         super().__init__()
         self.hidden_size = hidden_size
         if hidden_ratio is None:
@@ -59,8 +60,8 @@ class HGRNBitMLP(nn.Module):
         self.intermediate_size = intermediate_size
         if hidden_act not in ("swish", "silu"):
             raise NotImplementedError(f"hidden_act={hidden_act!r}: the fused gate is swish")
-        self.gate_proj = BitLinear(self.hidden_size, self.intermediate_size * 2, bias=False)
-        self.down_proj = BitLinear(self.intermediate_size, self.hidden_size, bias=False)
+        self.gate_proj = BitLinear(self.hidden_size, self.intermediate_size * 2, bias=False, fused_eps=bitlinear_eps)
+        self.down_proj = BitLinear(self.intermediate_size, self.hidden_size, bias=False, fused_eps=bitlinear_eps)
 
     def forward(self, x, residual=None, pre_norm=None):
         """down_proj(swiglu(gate, y)) as mmfreelm/models/hgrn_bit/modeling_hgrn_bit.py:55-59.
@@ -69,7 +70,7 @@ class HGRNBitMLP(nn.Module):
         fused into down_proj's epilogue; with ``pre_norm`` (the block's mlp_norm) x is the attention
         output and the residual add + RMSNorm in front of gate_proj (:107) is folded into gate_proj."""
         inter = self.intermediate_size
-        if self.training and torch.is_grad_enabled():
+        if module_needs_grad(self, x, residual):
             # the reference's composition (:55-59) through the autograd Functions; the block's norm and residual as :107-109
             from .activations import swiglu
             if pre_norm is not None:
@@ -103,10 +104,12 @@ class HGRNBitBlock(nn.Module):
         self.attn = HGRNBitAttention(
             mode=config.attn_mode, hidden_size=config.hidden_size, num_heads=config.num_heads,
             expand_ratio=config.expand_ratio, use_short_conv=config.use_short_conv, conv_size=config.conv_size,
-            share_conv_kernel=config.share_conv_kernel, layernorm_eps=config.rms_norm_eps, layer_idx=layer_idx)
+            share_conv_kernel=config.share_conv_kernel, layernorm_eps=config.rms_norm_eps, layer_idx=layer_idx,
+            bitlinear_eps=getattr(config, "bitlinear_eps", 1e-6))
         self.mlp_norm = RMSNorm(hidden_size=config.hidden_size, eps=config.rms_norm_eps)
         self.mlp = HGRNBitMLP(hidden_size=config.hidden_size, hidden_ratio=config.hidden_ratio,
-                              intermediate_size=config.intermediate_size, hidden_act=config.hidden_act)
+                              intermediate_size=config.intermediate_size, hidden_act=config.hidden_act,
+                              bitlinear_eps=getattr(config, "bitlinear_eps", 1e-6))
 
     def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
                 past_key_values=None, use_cache: Optional[bool] = False, output_attentions: Optional[bool] = False,
@@ -181,9 +184,11 @@ class HGRNBitModel(HGRNBitPreTrainedModel):
                 use_cache: Optional[bool] = None, output_attentions: Optional[bool] = None,
                 output_hidden_states: Optional[bool] = None, return_dict: Optional[bool] = None
                 ) -> Union[Tuple, BaseModelOutputWithPast]:
-        """Training mode with gradients enabled runs the reference's op-by-op composition through the autograd
-        Functions (matmulfreellm_amd/autograd.py); everything else runs the fused inference launches without a graph."""
-        train = self.training and torch.is_grad_enabled()
+        """With gradients enabled and a parameter or the input embeddings requiring one -- in train or eval mode, as the
+        reference -- the forward runs the reference's op-by-op composition through the autograd Functions
+        (matmulfreellm_amd/autograd.py); everything else (torch.no_grad(), generate()) runs the fused inference launches
+        without a graph."""
+        train = module_needs_grad(self, inputs_embeds)
         with torch.enable_grad() if train else torch.no_grad():
             return self._forward(train, input_ids, attention_mask, inputs_embeds, past_key_values, use_cache,
                                  output_attentions, output_hidden_states, return_dict)
@@ -195,7 +200,7 @@ class HGRNBitModel(HGRNBitPreTrainedModel):
         output_attentions = False
         output_hidden_states = bool(output_hidden_states) if output_hidden_states is not None else \
             bool(getattr(self.config, "output_hidden_states", False))
-        use_cache = use_cache if use_cache is not None else (self.config.use_cache if not self.training else False)
+        use_cache = use_cache if use_cache is not None else (self.config.use_cache if not train else False)
         return_dict = return_dict if return_dict is not None else bool(getattr(self.config, "return_dict", True))
 
         if input_ids is not None and inputs_embeds is not None:
@@ -260,7 +265,7 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
         super().__init__(config)
         self.model = HGRNBitModel(config)
         self.vocab_size = config.vocab_size
-        self.lm_head = BitLinear(config.hidden_size, config.vocab_size, bias=False)
+        self.lm_head = BitLinear(config.hidden_size, config.vocab_size, bias=False, fused_eps=getattr(config, "bitlinear_eps", 1e-6))
         self.post_init()
 
     def get_input_embeddings(self):
@@ -318,7 +323,7 @@ class HGRNBitForCausalLM(HGRNBitPreTrainedModel, GenerationMixin):
                 labels: Optional[torch.LongTensor] = None, use_cache: Optional[bool] = None,
                 output_attentions: Optional[bool] = None, output_hidden_states: Optional[bool] = None,
                 return_dict: Optional[bool] = None, logits_to_keep: int = 0) -> Union[Tuple, CausalLMOutputWithPast]:
-        train = self.training and torch.is_grad_enabled()
+        train = module_needs_grad(self, inputs_embeds)
         with torch.enable_grad() if train else torch.no_grad():
             return self._forward(train, input_ids, attention_mask, inputs_embeds, past_key_values, labels, use_cache,
                                  output_attentions, output_hidden_states, return_dict, logits_to_keep)

@@ -299,3 +299,35 @@ def test_training_reduces_the_loss_and_eval_path_is_unchanged(dev):
     sd = {k: v.detach().cpu() for k, v in model.state_dict().items()}
     ref, _ = om.forward(sd, ids[:1, :8].cpu(), L, mode="spec")
     assert torch.equal(got, ref)
+
+
+def test_eval_mode_gradients_equal_train_mode_gradients(dev):
+    """The differentiable path is chosen by what requires a gradient, not by model.training: the reference differentiates in
+    eval mode too.  Loss and every parameter gradient of an eval-mode step equal the train-mode step's bit for bit (the
+    model has no dropout; the backward kernels sum in a fixed order), and with frozen parameters a gradient still reaches
+    inputs_embeds (attribution)."""
+    model, _ = _model(dev, torch.float32, seed=5)
+    torch.manual_seed(13)
+    ids = torch.randint(0, V, (2, 16), device=dev)
+    grads = []
+    for mode in (model.train, model.eval):
+        mode()
+        model.zero_grad(set_to_none=True)
+        out = model(input_ids=ids, labels=ids)
+        assert out.loss.requires_grad, "no graph in " + mode.__name__
+        out.loss.backward()
+        grads.append((out.loss.detach().clone(), {k: p.grad.clone() for k, p in model.named_parameters() if p.grad is not None}))
+    assert torch.equal(grads[0][0], grads[1][0])
+    assert grads[0][1].keys() == grads[1][1].keys() and len(grads[0][1]) > 10
+    for k in grads[0][1]:
+        assert torch.equal(grads[0][1][k], grads[1][1][k]), k
+    # under no_grad the same eval-mode call builds no graph and returns the recurrent-state cache
+    with torch.no_grad():
+        out = model(input_ids=ids, use_cache=True)
+    assert not out.logits.requires_grad and out.past_key_values is not None
+    # frozen parameters, gradient with respect to the input embeddings
+    for p in model.parameters():
+        p.requires_grad_(False)
+    emb = model.get_input_embeddings()(ids).detach().requires_grad_()
+    model(inputs_embeds=emb).logits.float().square().mean().backward()
+    assert emb.grad is not None and torch.isfinite(emb.grad).all() and emb.grad.abs().max() > 0

@@ -21,6 +21,15 @@ from oracle import quant as oq
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _inference_mode():
+    """These are inference tests: gradients off, as generate() and every serving loop run (with gradients on, a model whose
+    parameters require them takes the differentiable path, in eval mode too -- tests/test_gpu_backward.py covers that)."""
+    with torch.no_grad():
+        yield
+
+
+
 def F():
     import matmulfreellm_amd.functional as F_
     return F_

@@ -9,6 +9,15 @@ from oracle import sampling as S
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _inference_mode():
+    """These are inference tests: gradients off, as generate() and every serving loop run (with gradients on, a model whose
+    parameters require them takes the differentiable path, in eval mode too -- tests/test_gpu_backward.py covers that)."""
+    with torch.no_grad():
+        yield
+
+
+
 def F():
     import matmulfreellm_amd.functional as F_
     return F_
@@ -93,6 +102,14 @@ def test_edge_values_of_top_p_u_and_the_logits(dev):
     # out-of-range uniform numbers are clamped, never read past the row
     bad_u = torch.tensor([1.0, 7.0, -3.0, float("nan"), 0.5, 0.5, 0.5, 0.5])
     _check_rows(dev, logits, 0.6, 0.9, bad_u, "clamped u")
+    # a row without a finite logit (all NaN, all -inf) is drawn uniformly with the top-k limit too, and always written:
+    # the output buffer starts from a value no draw can produce
+    logits[6] = float("-inf")
+    for top_k in (1, 50, 2047):
+        out = torch.full((8,), -7, dtype=torch.int64, device=dev)
+        F().sample_top_p(logits.to(dev), 0.4, 0.6, u.to(dev), top_k=top_k, out=out)
+        got = _check_rows(dev, logits, 0.6, 0.4, u, f"no finite logit, top_k={top_k}", top_k=top_k)
+        assert torch.equal(out.cpu(), got) and int(got[5]) == 512 and int(got[6]) == int(np.float32(0.99999994) * 2048)
 
 
 def test_draws_follow_the_renormalised_nucleus(dev):

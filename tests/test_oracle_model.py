@@ -77,9 +77,10 @@ def test_spec_tracks_literal_statistically():
     assert cos > 0.995 and agree > 0.8, (cos, agree)
 
 
-@pytest.mark.parametrize("name", ["fp32", "bf16"])
+@pytest.mark.parametrize("name", ["fp32", "bf16", "eps1e-8_fp32", "eps1e-8_bf16"])
 def test_oracle_reproduces_the_committed_golden_vectors(name):
-    """tests/golden/config1_*.npz (written by tests/golden/make_golden.py) pin the spec oracle against drift."""
+    """tests/golden/config1_*.npz (written by tests/golden/make_golden.py) pin the spec oracle against drift, at the
+    BitLinear eps the reference's fused forward runs with (1e-6) and at the 1e-8 its un-fused BitLinear states."""
     import os
     import importlib.util
     import numpy as np
@@ -88,6 +89,6 @@ def test_oracle_reproduces_the_committed_golden_vectors(name):
     mg = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mg)
     want = np.load(os.path.join(here, f"config1_{name}.npz"))
-    got = mg.vectors(torch.float32 if name == "fp32" else torch.bfloat16)
+    got = mg.vectors(torch.float32 if name.endswith("fp32") else torch.bfloat16, 1e-8 if name.startswith("eps1e-8") else 1e-6)
     for key in ("prompt", "argmax", "probe_idx", "probe_bits", "greedy"):
         assert np.array_equal(got[key], want[key]), key

@@ -92,6 +92,15 @@ def test_top_k_closed_forms():
     assert S.sample_top_p_spec(lg, 1.0, 1.0, 0.0, top_k=4)[1].all() and S.sample_top_p_spec(lg, 1.0, 1.0, 0.0, top_k=9)[1].all()
 
 
+def test_a_row_without_a_finite_logit_is_uniform_with_and_without_the_limit():
+    """All -inf (or NaN, which counts as -inf): every mass is 2^31, the nucleus is the whole row, the draw is floor(u * V)."""
+    for row in (np.full(40, -np.inf, dtype=np.float32), np.full(40, np.nan, dtype=np.float32)):
+        for top_k in (0, 1, 7, 39, 40):
+            for u in (0.0, 0.26, 0.5, 0.999):
+                tok, keep, m = S.sample_top_p_spec(row, 0.6, 0.4, u, top_k=top_k)
+                assert keep.all() and (m == 2 ** 31).all() and tok == int(np.float32(u) * 40)
+
+
 def test_the_draw_realises_the_renormalised_distribution():
     rng = np.random.default_rng(3)
     lg = (rng.standard_normal(50) * 2).astype(np.float32)
