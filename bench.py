@@ -111,7 +111,7 @@ def decode_bench(model, batch, steps, warmup, dev, prompt_len=128, resident=None
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain copy of known size);
 # see profiles/ for the runs and the scale factors.
 GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3625495          # one fused BitLinear GEMV launch of the launch chain
-LAYERS_TRAFFIC_BYTES_PER_LAUNCH = 348021769         # the resident layer-chain launch
+LAYERS_TRAFFIC_BYTES_PER_LAUNCH = 357781535         # the resident layer-chain launch
 
 
 def _replay_time(launch, iters):
@@ -283,8 +283,9 @@ def _rotating(make_set, set_bytes, min_total=512 << 20, min_sets=3):
 
 
 # HBM bytes per launch of the bandwidth-bound kernels at the shapes below, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/hbm_traffic_scan_norm_loss.txt; same calibration copy as the decode kernels).
-COUNTED_TRAFFIC = {"hgrn_recurrent": 201453786, "hgrn_chunk": 201465919, "rmsnorm": 134330432,
+# (profiles/hbm_traffic_scan_norm_loss.txt, profiles/bitlinear_gemv_stream_300MB.txt; same calibration copy as the decode
+# kernels).
+COUNTED_TRAFFIC = {"gemv_stream": 307356476, "hgrn_recurrent": 201453786, "hgrn_chunk": 201465919, "rmsnorm": 134330432,
                    "rmsnorm_swishgate": 201482279, "cross_entropy": 263065702}
 
 

@@ -181,6 +181,48 @@ def test_config4_greedy_decode_vs_oracle(dev, case_1p3b, batch, resident):
         assert eng.resident == resident
 
 
+@pytest.mark.parametrize("batch", [1, 16, 64])
+def test_config4_128_greedy_tokens_are_the_same_on_every_decode_path(dev, case_1p3b, batch):
+    """The configuration's stated length: a 128-token prompt and 128 greedy tokens, at batch 1, 16 and 64.  The CPU
+    oracle covers the first steps (test above); here every decode path the engine has for that batch -- the resident
+    launch, one launch per fused BitLinear, the matrix-core contraction, one launch per reference op -- runs the whole
+    length from the same prompt state: tokens of all 128 steps, the last step's logits and every layer's final
+    recurrent state must be equal bit for bit."""
+    from matmulfreellm_amd.decode import DecodeEngine
+    c = case_1p3b
+    g = torch.Generator().manual_seed(140 + batch)
+    ids = torch.randint(0, c.V, (batch, 128), generator=g).to(dev)
+    out = c.model(input_ids=ids, use_cache=True, logits_to_keep=1)
+    states = [s[-1] for s in out.past_key_values]
+    first = out.logits[:, -1].argmax(-1)
+    runs, names = [], []
+    for kw in ({}, {"resident": False}, {"fuse": False}):
+        eng = DecodeEngine(c.model, batch, use_graph=True, **kw)
+        name = ("resident" if eng.resident else "fused launch chain" if eng.fused else "fused quantiser + matrix cores"
+                if eng.fused_mfma else "one launch per reference op")
+        if name in names:
+            continue
+        eng.load_state(states)
+        eng.tok.copy_(first)
+        toks = [eng.tok.clone()]
+        for _ in range(127):
+            eng.advance()
+            toks.append(eng.tok.clone())
+        eng.check()
+        names.append(name)
+        runs.append((torch.stack(toks, 1).cpu(), eng.logits.clone().cpu(), [e["state"].clone().cpu() for e in eng.layers]))
+        del eng
+    print(f"config 4, batch {batch}: 128 greedy tokens on {names}; "
+          f"{len(set(runs[0][0].flatten().tolist()))} distinct tokens drawn", flush=True)
+    assert len(names) >= 2
+    for name, (toks, logits, st) in zip(names[1:], runs[1:]):
+        assert torch.equal(toks, runs[0][0]), f"{name} vs {names[0]}: tokens differ first at step " \
+            f"{int((toks != runs[0][0]).any(0).nonzero()[0])}"
+        assert torch.equal(logits, runs[0][1]), f"{name}: logits of step 128"
+        for li, (a, b) in enumerate(zip(st, runs[0][2])):
+            assert torch.equal(a, b), f"{name}: state of layer {li} after step 128"
+
+
 def test_config4_prefill_8x2048_vs_oracle(dev, case_1p3b):
     """The whole 8 x 2048 prompt batch on the GPU; rows 1 and 6 through the oracle: last-position logits and the
     final recurrent state of every layer."""
