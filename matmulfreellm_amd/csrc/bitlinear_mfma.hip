@@ -399,6 +399,24 @@ __global__ __launch_bounds__(64 * WGM * WGN) void bitlinear_mfma_kernel(MfmaArgs
 typedef __attribute__((address_space(3))) void* mmf_lds_ptr;
 typedef __attribute__((address_space(1))) const void* mmf_glb_ptr;
 
+// One 1 KiB wave-load global -> LDS (16 bytes per lane; lane l lands at lds + 16 l) from `base` (wave-uniform) + 16 l.
+// Written in assembly so that the compiler does not know of an LDS write in flight: it answers the builtin with waits
+// for all vector-memory traffic in front of later LDS reads and barriers, at places of its own choosing (the top of the
+// k-loop, half a k-block after the request).  The kernel waits for its transfers itself, once per k-block, where the
+// data is needed.
+__device__ __forceinline__ void mfma_dma_1k(const void* base, uint32_t lane16, const unsigned char* lds) {
+    const uint32_t l = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char*)lds;
+    const uint64_t b = (uint64_t)base;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(l), "v"(lane16), "s"(b) : "memory");
+}
+// Workgroup barrier behind an explicit wait: at most `VM` vector-memory operations may stay in flight, LDS traffic done.
+// Only VM = 0 says anything about a transfer into LDS: such transfers and ordinary loads complete in no fixed order.
+template <int VM>
+__device__ __forceinline__ void mfma_barrier_vm() {
+    static_assert(VM >= 0 && VM < 64, "vmcnt is a 6-bit count");
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(VM) : "memory");
+}
+
 // ------------------------------------------------------------------------------------------
 // The large-M kernel.  Same tiling, but A goes global -> LDS by DMA (global_load_lds_dwordx4:
 // lane l's 16 bytes land at the wave-uniform LDS base + 16*l, which is exactly the
@@ -406,7 +424,8 @@ typedef __attribute__((address_space(1))) const void* mmf_glb_ptr;
 // Three A buffers of one 128-wide k-block each and ONE barrier per k-block,
 // placed after the second of its four k-steps.  At that barrier every wave has left the previous
 // k-block, so its buffer is free for the DMA of k-block s+2, and k-block s+1 (issued one k-block
-// earlier, waited for by each wave just before the barrier) is complete for everybody.  K-block
+// earlier, waited for by each wave just before the barrier, together with the packed weights
+// requested with it) is complete for everybody.  K-block
 // boundaries therefore carry no synchronisation: the A fragments of the next k-block's first
 // step are read while the current one's last MFMAs run, and the matrix pipe never drains.
 // FAST (chosen by the launcher): 16-byte stores possible and no bias -> lean epilogue, accumulators start at -qsum.
@@ -473,8 +492,8 @@ void bitlinear_mfma_dma3_kernel(MfmaArgs p) {
             int64_t mb = mb0 + chunk;
             if (mb >= MB) mb = MB - 1;                            // rows past M are never stored: any valid data will do
             const int kbc = kb < KB ? kb : KB - 1;                // past the end: harmless re-read, never consumed
-            const unsigned char* g = reinterpret_cast<const unsigned char*>(p.a) + (mb * KG + kbc * 8 + within * 2) * 512 + lane * 16;
-            __builtin_amdgcn_global_load_lds((mmf_glb_ptr)g, (mmf_lds_ptr)(smem + boff + w * 1024), 16, 0, 0);
+            const unsigned char* g = reinterpret_cast<const unsigned char*>(p.a) + (mb * KG + kbc * 8 + within * 2) * 512;
+            mfma_dma_1k(g, (uint32_t)lane * 16u, smem + boff + w * 1024);
         }
     };
     auto load_b = [&](int kb, uint4 (&dst)[WN]) {                 // unconditional: the barrier's vmcnt counts on WN loads
@@ -482,7 +501,10 @@ void bitlinear_mfma_dma3_kernel(MfmaArgs p) {
         for (int j = 0; j < WN; ++j) {
             const int64_t nb = nblock(j);
             const int kbc = kb < KB ? kb : KB - 1;                // past the end: never consumed
-            dst[j] = p.b[(nb * KB + kbc) * 64 + lane];
+            // wave-uniform block address + a 32-bit lane offset: the load then takes its base from scalar registers and
+            // no 64-bit per-lane address is kept alive
+            const unsigned char* blk = reinterpret_cast<const unsigned char*>(p.b + (nb * KB + kbc) * 64);
+            dst[j] = *reinterpret_cast<const uint4*>(blk + (uint32_t)(lane * 16));
         }
     };
     auto expand_b = [&](const uint4 (&src)[WN], int ks, v4i (&bf)[WN]) {
@@ -496,13 +518,15 @@ void bitlinear_mfma_dma3_kernel(MfmaArgs p) {
         }
     };
 
-    // B runs two k-blocks ahead: the loads of k-block s+2 are the only vector-memory operations
-    // younger than the DMA of k-block s+1 when the barrier of k-block s waits for that DMA
-    uint4 breg[WN], bnext[WN], bnext2[WN];
+    // B is requested a k-block and a half before its first use, into a ring of three register sets.  The ring is walked
+    // by unrolling the k-loop three times, so a set keeps its registers from its load to its last use (rotating the sets
+    // with copies at the loop's back edge makes the compiler wait there for everything in flight: the copy reads the set
+    // loaded last).
+    uint4 bset0[WN], bset1[WN], bset2[WN];
     dma_block(0, 0);
     dma_block(1, BUF);
-    load_b(0, breg);
-    load_b(1, bnext);
+    load_b(0, bset0);
+    load_b(1, bset1);
     __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): this wave's pieces of k-blocks 0 and 1 have landed
     __syncthreads();
 
@@ -522,33 +546,61 @@ void bitlinear_mfma_dma3_kernel(MfmaArgs p) {
 #pragma unroll
     for (int i = 0; i < WM; ++i) af[0][i] = *reinterpret_cast<const v4i*>(smem + cur + aoff + i * CH);
 
-    for (int kb = 0; kb < KB; ++kb) {
-        load_b(kb + 2, bnext2);
+    // one k-block: contracts with the set `bcur`, requests k-block kb + 2 into `bfar`; the expansion of the NEXT step's
+    // weights (the first step of `bnxt` at the end) is interleaved with this step's MFMAs
+    v4i bf[WN];
+    expand_b(bset0, 0, bf);
+    auto kblock = [&](int kb, const uint4 (&bcur)[WN], const uint4 (&bnxt)[WN], uint4 (&bfar)[WN]) {
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             if (ks == 2) {
-                // DMA of k-block kb+1 (issued one k-block ago) is older than this iteration's B loads
-                __builtin_amdgcn_s_waitcnt(0x0F70 | WN);          // vmcnt(WN)
-                __syncthreads();
+                // Everything requested one k-block ago -- this wave's pieces of A k-block kb+1 and the weights of kb+1 --
+                // has to be here now.  The wait is for ALL vector-memory traffic: a transfer into LDS and an ordinary load
+                // do not complete in the order they were issued (a count that leaves the younger weight loads in flight let
+                // warm weight loads overtake a cold A transfer and gave wrong sums), so the next requests go out right
+                // behind the barrier and have a whole k-block to land.
+                mfma_barrier_vm<0>();
                 dma_block(kb + 2, fre);
+                load_b(kb + 2, bfar);
             }
-            // next step's A fragments: same k-block, or the first step of the next one
             const unsigned char* nsrc = ks < 3 ? smem + cur + aoff + (ks + 1) * 1024 : smem + nxt + aoff;
 #pragma unroll
             for (int i = 0; i < WM; ++i) af[(ks + 1) & 1][i] = *reinterpret_cast<const v4i*>(nsrc + i * CH);
-            __builtin_amdgcn_sched_barrier(0);                    // keep the prefetch ahead of this step's MFMAs
-            v4i bf[WN];
-            expand_b(breg, ks, bf);
+            // weight columns outermost: once the MFMAs of column j are issued, the next step's expansion of column j can
+            // reuse its registers and runs in the shadow of the matrix pipe
+            v4i bn[WN];
 #pragma unroll
-            for (int i = 0; i < WM; ++i)
+            for (int j = 0; j < WN; ++j) {
 #pragma unroll
-                for (int j = 0; j < WN; ++j)
+                for (int i = 0; i < WM; ++i)
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[ks & 1][i], acc[i][j], 0, 0, 0);
+                const uint32_t w = ks == 0 ? bcur[j].y : ks == 1 ? bcur[j].z : ks == 2 ? bcur[j].w : bnxt[j].x;
+                bn[j][0] = (int)(w & 0x03030303u);
+                bn[j][1] = (int)((w >> 2) & 0x03030303u);
+                bn[j][2] = (int)((w >> 4) & 0x03030303u);
+                bn[j][3] = (int)((w >> 6) & 0x03030303u);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x100, WM, 0);
+#pragma unroll
+            for (int j = 0; j < WN; ++j) {
+                __builtin_amdgcn_sched_group_barrier(0x008, WM, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+            }
+#pragma unroll
+            for (int j = 0; j < WN; ++j) bf[j] = bn[j];
             __builtin_amdgcn_sched_barrier(0);
         }
-#pragma unroll
-        for (int j = 0; j < WN; ++j) { breg[j] = bnext[j]; bnext[j] = bnext2[j]; }
         const int t = cur; cur = nxt; nxt = fre; fre = t;
+    };
+    int kb = 0;
+    for (; kb + 3 <= KB; kb += 3) {
+        kblock(kb, bset0, bset1, bset2);
+        kblock(kb + 1, bset1, bset2, bset0);
+        kblock(kb + 2, bset2, bset0, bset1);
+    }
+    if (kb < KB) {
+        kblock(kb, bset0, bset1, bset2);
+        if (kb + 1 < KB) kblock(kb + 1, bset1, bset2, bset0);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);            // the trailing DMA must not land in the epilogue's staging area
     __syncthreads();

@@ -26,8 +26,8 @@
 // launch starts; the packed weights and the norm weights of link n+1 are brought into LDS by the DMA path
 // (global_load_lds, no registers) while link n computes, each wave fetching exactly the slices it will read itself;
 // the few epilogue operands (recurrent state, lower bound, scales, residual operands) are loaded into registers one
-// link ahead.  All of these are requested after link n's row has arrived: loads return in order, requested before
-// the poll they would delay it.
+// link ahead.  All of these are requested after link n's row has arrived (requested before the poll they would
+// delay it) and are waited for, with everything else in flight, right after link n+1's poll.
 //
 // The arithmetic of every link is that of bitlinear_gemv_kernel with the same prologue / epilogue, operation for
 // operation (sums of squares in fp64 are order-insensitive to rounding, integer sums exact).
@@ -110,7 +110,8 @@ __device__ __forceinline__ uint16_t gload2(const void* base, int i) { return ((c
 // 64 lanes x 16 bytes from global memory straight into 1 KiB of LDS at `lds` (wave-uniform), lane order.
 // Issued by hand: told about a transfer into LDS, the compiler makes every later LDS read (the statistics exchanged a
 // few hundred cycles on, the partial sums) wait for it -- a trip to HBM in the middle of every link.  The data is
-// only read after the next link's input row has arrived, and that wait covers it (loads return in order).
+// only read after the next link's input row has arrived, behind a wait for ALL vector-memory traffic (a count that
+// left younger loads in flight would not do: transfers into LDS and ordinary loads complete in no fixed order).
 __device__ __forceinline__ void dma16(const void* gbase, uint32_t byte_off, unsigned char* lds) {
     const uint32_t l = (uint32_t)(uintptr_t)(MMF_AS_LDS unsigned char*)lds;
     const uint64_t b = (uint64_t)gbase;
@@ -663,8 +664,8 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
                 }
             }
             // ---- dot products of this wave's slice with the weights of this pass; partial sums to LDS.  The weights were
-            // requested a link (or a pass) ago; the wait for the row (or the one above) has seen them land (loads return in
-            // order).  The codes are read back by this wave only: LDS operations of a wave execute in order.
+            // requested a link (or a pass) ago; the wait for everything in flight behind the row's poll (or the one above)
+            // has seen them land.  The codes are read back by this wave only: LDS operations of a wave execute in order.
             __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
             if (g.nkb == 0) {
                 for (int it = lane >> 4; it < ng * g.R; it += 4)

@@ -60,6 +60,33 @@ def test_config2_down_proj_at_4096_rows(dev):
     _bitlinear_case(dev, 4096, 5632, 2048, seed=21, path="mfma")
 
 
+@pytest.mark.parametrize("m,k,n", [(8192, 5632, 2048), (16384, 5632, 2048), (16384, 2048, 6144)])
+def test_tiled_contraction_with_two_workgroups_per_cu_and_warm_weights(dev, m, k, n):
+    """Prefill-sized problems (more tiles than CUs, so two workgroups share a CU) run several times in a row, so that the
+    packed weights come from the cache while the activation panels still come from memory: a transfer into LDS and an
+    ordinary load complete in no fixed order, and the k-loop's wait has to cover both.  Every run must equal the exact
+    integer contraction of the same codes (fp64 matmul: |acc| < 2**53) under the kernel's scaling."""
+    g = torch.Generator(device=dev).manual_seed(77)
+    x = torch.randn(m, k, generator=g, device=dev).bfloat16()
+    w = (torch.randn(n, k, generator=g, device=dev) * 0.02).bfloat16()
+    nw = torch.ones(k, device=dev, dtype=torch.bfloat16)
+    pw = F().ternarize_pack(w)
+    q, deq, qsum = F().rmsnorm_quant(x, nw, eps=1e-8, tiled=True)
+    q_rows, deq_rows, _ = F().rmsnorm_quant(x, nw, eps=1e-8, tiled=False)
+    t = F().unpack_ternary(pw)
+    ref = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
+    for r0 in range(0, m, 4096):                                 # fp64 operands in slabs: bounded memory
+        acc = q_rows[r0:r0 + 4096, :k].double() @ t.double().t()
+        ref[r0:r0 + 4096] = ((acc.float() * deq_rows[r0:r0 + 4096].reshape(-1, 1)) * pw.wdeq).bfloat16()
+    bad = []
+    for _ in range(6):
+        out = torch.zeros(m, n, device=dev, dtype=torch.bfloat16)
+        F().bitlinear_mfma(q, deq, qsum, pw, m, torch.bfloat16, out=out, config=17)
+        bad.append(int((out != ref).sum()))
+    print(f"tiled contraction {m} x {k} -> {n}: outputs differing from the exact contraction over 6 runs: {bad}", flush=True)
+    assert bad == [0] * 6
+
+
 @pytest.mark.parametrize("m", [1, 64])
 @pytest.mark.parametrize("kn", [(2048, 11264), (5632, 2048)])
 def test_config2_decode_rows(dev, m, kn):
