@@ -36,6 +36,7 @@
 //                            recurrence step on the fp32 state, writes o and g
 //                EPI_SWIGLU  R = 2 (gate, up rows of the same 32 channels): out = swiglu
 #include "mmf_common.h"
+#include <stdlib.h>
 
 namespace {
 
@@ -72,8 +73,13 @@ struct GemvArgs {
 // S = 4: it owns 8 of the 32 rows, so that a 2048-row projection fills 256 CUs instead of 64; a
 // lane is (k-block of a group of four, k-half, row of 8), a wave-load covers four k-blocks (two
 // 128-byte runs of each 1 KiB block), and the waves share out the (n-block, k-group) items.
-template <typename T, typename TW, int NW, int NV, int PRO, int EPI, bool VEC, int S>
+// WALK (S = 1, plain epilogue): a launch with many more n-blocks than CUs (a vocabulary-sized projection) runs on a
+// grid of as many workgroups as are resident at once; workgroup b of a row of x takes the n-blocks b, b + grid, ... behind ONE
+// prologue, the next block's packed weights in flight while the current one is contracted -- otherwise every 16 KiB of
+// weights would wait behind a re-quantisation of the whole row.
+template <typename T, typename TW, int NW, int NV, int PRO, int EPI, bool VEC, int S, bool WALK = false>
 __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
+    static_assert(!WALK || (S == 1 && EPI == EPI_PLAIN), "the n-block walk is built for whole n-blocks and the plain epilogue");
     constexpr int kGemvWaves = NW, kGemvThreads = 64 * NW;
     constexpr int R = EPI == EPI_STEP ? 3 : EPI == EPI_SWIGLU ? 2 : 1;
     constexpr int BPW = 2 * NV;
@@ -254,87 +260,136 @@ __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
     qs = mmf_wave_sum(qs);
     if (lane == 0) red_q[wave] = qs;
 
-    // ---- main: sum_k q[k] * (t[n,k] + 1) over this wave's blocks
-    auto dot_block = [&](const uint4& wq, int kb, int acc) { return mmf_dot_block(q_lds, wq, kb, half, acc); };
-    if constexpr (S == 1) {
-        int acc[R];
+    // ---- main + epilogue of one n-block (R stacked ones): weights `wr`, epilogue operands as loaded for that block
+    auto contract = [&](const uint4 (&wr)[NWREG], int nbc, const float (&wdq)[R], float bias_v, float add_v) {
+        const int chc = nbc * 32 + sub * CHN + (lane & (CHN - 1));
+        const bool epl = wave == 0 && lane < CHN && chc < Nseg;
+        auto dot_block = [&](const uint4& wq, int kb, int acc) { return mmf_dot_block(q_lds, wq, kb, half, acc); };
+        if constexpr (S == 1) {
+            int acc[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) acc[r] = 0;
+            for (int r = 0; r < R; ++r) acc[r] = 0;
 #pragma unroll
-        for (int i = 0; i < BPW; ++i) {
-            const int kb = wave + i * kGemvWaves;
-            if (kb < KB) {
+            for (int i = 0; i < BPW; ++i) {
+                const int kb = wave + i * kGemvWaves;
+                if (kb < KB) {
 #pragma unroll
-                for (int r = 0; r < R; ++r) acc[r] = dot_block(wreg[r * BPW + i], kb, acc[r]);
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < R; ++r) reinterpret_cast<int*>(&part[(r * kGemvWaves + wave) * 32 + (lane & 31)])[half] = acc[r];
-    } else {
-#pragma unroll
-        for (int i = 0; i < ITEMS; ++i) {
-            const int item = wave + i * kGemvWaves;
-            if (item < R * G) {
-                const int kb = (item % G) * 4 + kbi;
-                int acc = dot_block(wreg[i], kb < KB ? kb : 0, 0);   // blocks past the end carry zero codes
-                acc += mmf_dpp<0x128>(acc);                      // row_ror:8 -> the other k-half
-                acc += __builtin_amdgcn_ds_swizzle(acc, 0x401F);   // xor 16 -> the neighbouring k-block
-                if ((lane & 31) < 8) reinterpret_cast<int*>(&part[item * 8 + (lane & 7)])[lane >> 5] = acc;
-            }
-        }
-    }
-    __syncthreads();
-    if (ep_lane) {
-        int qtot = 0;
-#pragma unroll
-        for (int w = 0; w < kGemvWaves; ++w) qtot += red_q[w];
-        float res[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            int tot = 0;
-            if constexpr (S == 1) {
-#pragma unroll
-                for (int w = 0; w < kGemvWaves; ++w) {
-                    const int2 pr = part[(r * kGemvWaves + w) * 32 + lane];
-                    tot += pr.x + pr.y;
-                }
-            } else {
-#pragma unroll
-                for (int gi = 0; gi < GMAX; ++gi) {                 // compile-time bound: the reads are issued together
-                    const int2 pr = part[(r * G + (gi < G ? gi : 0)) * 8 + lane];
-                    tot += gi < G ? pr.x + pr.y : 0;
+                    for (int r = 0; r < R; ++r) acc[r] = dot_block(wr[r * BPW + i], kb, acc[r]);
                 }
             }
-            res[r] = __fmul_rn(__fmul_rn((float)(tot - qtot), deq), ep_wdeq[r]);
-        }
-        if constexpr (EPI == EPI_PLAIN) {
-            float o = res[0];
-            if (a.bias) o = __fadd_rn(o, ep_bias);
-            if (a.addend) o = __fadd_rn(mmf_round_to<T>(o), ep_add);
-            static_cast<T*>(a.out)[(int64_t)row * a.N + ch] = mmf_from_float<T>(o);
-        } else if constexpr (EPI == EPI_STEP) {
-            // res = raw i, f, g projections of channel ch (each rounded to T like the tensors they replace)
-            const float iv = mmf_round_to<T>(res[0]), fv = mmf_round_to<T>(res[1]);
-            float s = mmf_sigmoid(fv);
-            if (a.lb) s = __fadd_rn(ep_lb, __fmul_rn(__fsub_rn(1.0f, ep_lb), s));
-            const float go = mmf_round_to<T>(s);
-            const float xo = mmf_round_to<T>(__fdiv_rn(__fmul_rn(iv, __fsub_rn(1.0f, go)), __fadd_rn(1.0f, mmf_exp(-iv))));
-            const float h = __fadd_rn(__fmul_rn(go, ep_state), xo);
-            a.state[(int64_t)row * Nseg + ch] = h;
-            static_cast<T*>(a.out)[(int64_t)row * Nseg + ch] = mmf_from_float<T>(h);
-            static_cast<T*>(a.g_out)[(int64_t)row * Nseg + ch] = mmf_from_float<T>(res[2]);
+#pragma unroll
+            for (int r = 0; r < R; ++r) reinterpret_cast<int*>(&part[(r * kGemvWaves + wave) * 32 + (lane & 31)])[half] = acc[r];
         } else {
-            const float g = mmf_round_to<T>(res[0]), u = mmf_round_to<T>(res[1]);
-            static_cast<T*>(a.out)[(int64_t)row * Nseg + ch] =
-                mmf_from_float<T>(__fdiv_rn(__fmul_rn(g, u), __fadd_rn(1.0f, mmf_exp(-g))));
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) {
+                const int item = wave + i * kGemvWaves;
+                if (item < R * G) {
+                    const int kb = (item % G) * 4 + kbi;
+                    int acc = dot_block(wr[i], kb < KB ? kb : 0, 0);   // blocks past the end carry zero codes
+                    acc += mmf_dpp<0x128>(acc);                      // row_ror:8 -> the other k-half
+                    acc += __builtin_amdgcn_ds_swizzle(acc, 0x401F);   // xor 16 -> the neighbouring k-block
+                    if ((lane & 31) < 8) reinterpret_cast<int*>(&part[item * 8 + (lane & 7)])[lane >> 5] = acc;
+                }
+            }
+        }
+        __syncthreads();
+        if (epl) {
+            int qtot = 0;
+#pragma unroll
+            for (int w = 0; w < kGemvWaves; ++w) qtot += red_q[w];
+            float res[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                int tot = 0;
+                if constexpr (S == 1) {
+#pragma unroll
+                    for (int w = 0; w < kGemvWaves; ++w) {
+                        const int2 pr = part[(r * kGemvWaves + w) * 32 + lane];
+                        tot += pr.x + pr.y;
+                    }
+                } else {
+#pragma unroll
+                    for (int gi = 0; gi < GMAX; ++gi) {                 // compile-time bound: the reads are issued together
+                        const int2 pr = part[(r * G + (gi < G ? gi : 0)) * 8 + lane];
+                        tot += gi < G ? pr.x + pr.y : 0;
+                    }
+                }
+                res[r] = __fmul_rn(__fmul_rn((float)(tot - qtot), deq), wdq[r]);
+            }
+            if constexpr (EPI == EPI_PLAIN) {
+                float o = res[0];
+                if (a.bias) o = __fadd_rn(o, bias_v);
+                if (a.addend) o = __fadd_rn(mmf_round_to<T>(o), add_v);
+                static_cast<T*>(a.out)[(int64_t)row * a.N + chc] = mmf_from_float<T>(o);
+            } else if constexpr (EPI == EPI_STEP) {
+                // res = raw i, f, g projections of channel ch (each rounded to T like the tensors they replace)
+                const float iv = mmf_round_to<T>(res[0]), fv = mmf_round_to<T>(res[1]);
+                float s = mmf_sigmoid(fv);
+                if (a.lb) s = __fadd_rn(ep_lb, __fmul_rn(__fsub_rn(1.0f, ep_lb), s));
+                const float go = mmf_round_to<T>(s);
+                const float xo = mmf_round_to<T>(__fdiv_rn(__fmul_rn(iv, __fsub_rn(1.0f, go)), __fadd_rn(1.0f, mmf_exp(-iv))));
+                const float h = __fadd_rn(__fmul_rn(go, ep_state), xo);
+                a.state[(int64_t)row * Nseg + chc] = h;
+                static_cast<T*>(a.out)[(int64_t)row * Nseg + chc] = mmf_from_float<T>(h);
+                static_cast<T*>(a.g_out)[(int64_t)row * Nseg + chc] = mmf_from_float<T>(res[2]);
+            } else {
+                const float g = mmf_round_to<T>(res[0]), u = mmf_round_to<T>(res[1]);
+                static_cast<T*>(a.out)[(int64_t)row * Nseg + chc] =
+                    mmf_from_float<T>(__fdiv_rn(__fmul_rn(g, u), __fadd_rn(1.0f, mmf_exp(-g))));
+            }
+        }
+
+    };
+    if constexpr (!WALK) {
+        contract(wreg, nb, ep_wdeq, ep_bias, ep_add);
+    } else {
+        // One n-block ahead: deeper (two blocks in flight through a ring of three register sets) measured 15 % slower.
+        const int NBall = (a.N + 31) >> 5, stride = (int)gridDim.x;
+        for (int nbc = nb; nbc < NBall; nbc += stride) {
+            // the next block's weights and epilogue operands travel under this block's contraction
+            const int nbn = nbc + stride < NBall ? nbc + stride : nbc;
+            uint4 wnext[NWREG];
+#pragma unroll
+            for (int i = 0; i < BPW; ++i) {
+                const int kb = wave + i * kGemvWaves;
+                if (kb < KB) wnext[i] = a.packed[((int64_t)nbn * KB + kb) * 64 + lane];
+            }
+            float wdq_n[R], bias_n = 0.0f, add_n = 0.0f;
+            const int chn = nbn * 32 + (lane & 31);
+            wdq_n[0] = a.wdeq[(uint32_t)(nbn * 32) / (uint32_t)a.seg_rows];
+            if (wave == 0 && lane < 32 && chn < a.N) {
+                if (a.bias) bias_n = mmf_to_float(static_cast<const T*>(a.bias)[chn]);
+                if (a.addend) add_n = mmf_to_float(static_cast<const T*>(a.addend)[(int64_t)row * a.N + chn]);
+            }
+            contract(wreg, nbc, ep_wdeq, ep_bias, ep_add);
+            __syncthreads();                                    // part[] is free again
+#pragma unroll
+            for (int i = 0; i < NWREG; ++i) wreg[i] = wnext[i];
+            ep_wdeq[0] = wdq_n[0]; ep_bias = bias_n; ep_add = add_n;
         }
     }
 }
 
 template <typename T, typename TW, int PRO, int EPI, int NW, int NV>
-void launch_gemv_shape(const GemvArgs& a, dim3 grid, bool split, hipStream_t s) {
+void launch_gemv_shape(const GemvArgs& a, dim3 grid, bool split, bool walk, hipStream_t s) {
+    if constexpr (EPI == EPI_PLAIN) {
+        if (walk) {
+            bitlinear_gemv_kernel<T, TW, NW, NV, PRO, EPI, true, 1, true><<<grid, dim3(64 * NW), (size_t)a.Kp, s>>>(a);
+            return;
+        }
+    }
     if (split) bitlinear_gemv_kernel<T, TW, NW, NV, PRO, EPI, true, 4><<<grid, dim3(64 * NW), (size_t)a.Kp, s>>>(a);
     else bitlinear_gemv_kernel<T, TW, NW, NV, PRO, EPI, true, 1><<<grid, dim3(64 * NW), (size_t)a.Kp, s>>>(a);
+}
+
+// Workgroups that a launch keeps resident at once on this build's target (256 CUs, 2048 threads each): the n-block walk
+// sizes its grid to them.  MMF_GEMV_WALK_GRID overrides the per-launch total (0 = never walk): a measuring aid.
+inline int gemv_walk_slots(int threads) {
+    static const int env = [] {
+        const char* e = getenv("MMF_GEMV_WALK_GRID");
+        return e ? atoi(e) : -1;
+    }();
+    return env >= 0 ? env : 256 * (2048 / threads);
 }
 
 template <typename T, typename TW, int PRO, int EPI>
@@ -343,13 +398,18 @@ int launch_gemv(const GemvArgs& a, int64_t M, bool vec, hipStream_t s) {
     const int64_t nblocks = mmf_ceil_div(a.N / R, 32);
     // few n-blocks (a 2048-row projection has 64): give each workgroup 8 rows, not 32, to reach every CU
     const bool split = vec && nblocks * M <= 64;             // at most 256 workgroups after the split: one per CU
-    dim3 grid((unsigned)(nblocks * (split ? 4 : 1)), (unsigned)M);
+    // waves per workgroup and passes over the row: the fewest passes, then the fewest waves, that cover K
+    const int nw = a.Kp <= 2048 ? 8 : a.Kp <= 3072 ? 12 : a.Kp <= 4096 ? 16 : a.Kp <= 6144 ? 12 : 16;
+    // many more n-blocks than resident workgroups (vocabulary-sized N): a grid of resident workgroups walks them
+    const int64_t per_row = gemv_walk_slots(64 * nw) / M;
+    const bool walk = vec && EPI == EPI_PLAIN && per_row >= 32 && nblocks > per_row;
+    dim3 grid((unsigned)(walk ? per_row : nblocks * (split ? 4 : 1)), (unsigned)M);
     if (!vec) bitlinear_gemv_kernel<T, TW, 8, 4, PRO, EPI, false, 1><<<grid, dim3(512), (size_t)a.Kp, s>>>(a);   // ragged shapes: one generic build
-    else if (a.Kp <= 2048) launch_gemv_shape<T, TW, PRO, EPI, 8, 1>(a, grid, split, s);
-    else if (a.Kp <= 3072) launch_gemv_shape<T, TW, PRO, EPI, 12, 1>(a, grid, split, s);
-    else if (a.Kp <= 4096) launch_gemv_shape<T, TW, PRO, EPI, 16, 1>(a, grid, split, s);
-    else if (a.Kp <= 6144) launch_gemv_shape<T, TW, PRO, EPI, 12, 2>(a, grid, split, s);
-    else launch_gemv_shape<T, TW, PRO, EPI, 16, 2>(a, grid, split, s);
+    else if (a.Kp <= 2048) launch_gemv_shape<T, TW, PRO, EPI, 8, 1>(a, grid, split, walk, s);
+    else if (a.Kp <= 3072) launch_gemv_shape<T, TW, PRO, EPI, 12, 1>(a, grid, split, walk, s);
+    else if (a.Kp <= 4096) launch_gemv_shape<T, TW, PRO, EPI, 16, 1>(a, grid, split, walk, s);
+    else if (a.Kp <= 6144) launch_gemv_shape<T, TW, PRO, EPI, 12, 2>(a, grid, split, walk, s);
+    else launch_gemv_shape<T, TW, PRO, EPI, 16, 2>(a, grid, split, walk, s);
     MMF_CHECK_LAUNCH();
     return 0;
 }

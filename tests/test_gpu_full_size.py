@@ -60,6 +60,13 @@ def test_config2_down_proj_at_4096_rows(dev):
     _bitlinear_case(dev, 4096, 5632, 2048, seed=21, path="mfma")
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 2048, 70001), (3, 5632, 40000), (2, 2048, 131072)])
+def test_vocabulary_sized_gemv_walks_its_n_blocks(dev, m, k, n):
+    """Far more n-blocks than resident workgroups: the batch-1 kernel then runs a grid of resident workgroups, each
+    walking several n-blocks behind one prologue.  Same exact-contraction check as the other shapes (ragged N too)."""
+    _bitlinear_case(dev, m, k, n, seed=23, path="gemv")
+
+
 @pytest.mark.parametrize("m,k,n", [(8192, 5632, 2048), (16384, 5632, 2048), (16384, 2048, 6144)])
 def test_tiled_contraction_with_two_workgroups_per_cu_and_warm_weights(dev, m, k, n):
     """Prefill-sized problems (more tiles than CUs, so two workgroups share a CU) run several times in a row, so that the
