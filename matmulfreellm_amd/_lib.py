@@ -51,6 +51,7 @@ SIGNATURES = {
     "mmf_bitlinear_mfma_swiglu": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _i64, _i64, _i64, _i32, _ptr]),
     "mmf_bitlinear_mfma_clock_sink": (_i32, [_ptr, _i64]),
     "mmf_mfma_pipe_probe": (_i32, [_i64, _i64, _i32, _ptr, _ptr]),
+    "mmf_diag_check_exact_forms": (_i32, [_ptr, _ptr]),
     "mmf_hgrn_recurrent": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i32, _ptr]),
     "mmf_hgrn_chunk_workspace_bytes": (_i64, [_i64, _i64, _i64, _i32]),
     "mmf_hgrn_chunk": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _i32, _i32, _ptr, _ptr]),

@@ -73,6 +73,30 @@ __global__ __launch_bounds__(512) void argmax_kernel(const T* __restrict__ logit
     }
 }
 
+
+// Every float through the kernels' short forms of exp, the reciprocal of a denominator >= 1 and the sigmoid, against the
+// forms that define them.  counts[0..2]: arguments on which mmf_exp / mmf_rcp_ge1 / mmf_sigmoid differ from
+// mmf_exp_definition / __fdiv_rn(1, d) / mmf_sigmoid_definition (NaN results count as equal when both are NaN);
+// counts[3]: arguments seen.  A grid-stride walk over all 2^32 bit patterns.
+__global__ __launch_bounds__(256) void exact_forms_kernel(unsigned long long* counts) {
+    unsigned long long bad_exp = 0, bad_rcp = 0, bad_sig = 0, seen = 0;
+    auto same = [](float a, float b) { return (a != a && b != b) || __float_as_uint(a) == __float_as_uint(b); };
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < (1ull << 32); i += stride) {
+        const float x = __uint_as_float((uint32_t)i);
+        ++seen;
+        if (!same(mmf_exp(x), mmf_exp_definition(x))) ++bad_exp;
+        if (!same(mmf_sigmoid(x), mmf_sigmoid_definition(x))) ++bad_sig;
+        if (x != x || x >= 1.0f) {
+            if (!same(mmf_rcp_ge1(x), __fdiv_rn(1.0f, x))) ++bad_rcp;
+        }
+    }
+    if (bad_exp) atomicAdd(&counts[0], bad_exp);
+    if (bad_rcp) atomicAdd(&counts[1], bad_rcp);
+    if (bad_sig) atomicAdd(&counts[2], bad_sig);
+    atomicAdd(&counts[3], seen);
+}
+
 }  // namespace
 
 extern "C" {
@@ -104,6 +128,14 @@ int mmf_argmax(const void* logits, int64_t ld, int64_t rows, int64_t V, int64_t*
         case MMF_F16: argmax_kernel<f16_t><<<(unsigned)rows, 512, 0, stream>>>(static_cast<const f16_t*>(logits), ld, V, out); break;
         default: return MMF_ERR_ARG;
     }
+    MMF_CHECK_LAUNCH();
+    return 0;
+}
+
+int mmf_diag_check_exact_forms(unsigned long long* counts, void* stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (!counts) return MMF_ERR_ARG;
+    exact_forms_kernel<<<4096, 256, 0, stream>>>(counts);
     MMF_CHECK_LAUNCH();
     return 0;
 }

@@ -188,8 +188,9 @@ __device__ __forceinline__ void mmf_store8(T* __restrict__ p, int64_t k0, int64_
 
 // ---------------------------------------------------------------- deterministic exp
 // Cody-Waite reduction by ln2, degree-5 Horner polynomial, two-step 2^n scaling.
-// Every operation is a separately rounded fp32 add or multiply.
-__device__ __forceinline__ float mmf_exp(float x) {
+// Every operation is a separately rounded fp32 add or multiply.  This is the DEFINITION of the function (the CPU
+// restatement follows it operation by operation); the kernels call mmf_exp() below, which returns the same bits.
+__device__ __forceinline__ float mmf_exp_definition(float x) {
     float xc = fminf(fmaxf(x, -104.0f), 89.0f);                 // a NaN argument is clamped like any other and put back at the end
     float n = rintf(__fmul_rn(xc, 1.44269504088896341f));
     float r = __fsub_rn(xc, __fmul_rn(n, 0.693359375f));
@@ -212,9 +213,47 @@ __device__ __forceinline__ float mmf_exp(float x) {
     return x != x ? x : y;                                       // a select, not a branch
 }
 
+// The same function with the two-step scaling as ONE ldexp: the first of the two multiplications by a power of two is
+// exact (y is in [0.7, 1.5] and 2^n1 keeps it normal), so only the second rounds -- once, like ldexp(y, n).  Equal to the
+// definition for every one of the 2^32 arguments (mmf_diag_check_exact_forms runs them all on the device).
+__device__ __forceinline__ float mmf_exp(float x) {
+    float xc = fminf(fmaxf(x, -104.0f), 89.0f);
+    float n = rintf(__fmul_rn(xc, 1.44269504088896341f));
+    float r = __fsub_rn(xc, __fmul_rn(n, 0.693359375f));
+    r = __fsub_rn(r, __fmul_rn(n, -2.12194440e-4f));
+    float z = __fmul_rn(r, r);
+    float p = 1.9875691500e-4f;
+    p = __fadd_rn(__fmul_rn(p, r), 1.3981999507e-3f);
+    p = __fadd_rn(__fmul_rn(p, r), 8.3334519073e-3f);
+    p = __fadd_rn(__fmul_rn(p, r), 4.1665795894e-2f);
+    p = __fadd_rn(__fmul_rn(p, r), 1.6666665459e-1f);
+    p = __fadd_rn(__fmul_rn(p, r), 5.0000001201e-1f);
+    float y = __fmul_rn(p, z);
+    y = __fadd_rn(y, r);
+    y = __fadd_rn(y, 1.0f);
+    y = __builtin_ldexpf(y, (int)n);
+    return x != x ? x : y;
+}
+
+// Correctly rounded 1 / d for d in [1, inf] (and NaN): the hardware's approximate reciprocal, one Newton step with fused
+// multiply-adds, and the hardware's special-case fix-up (inf -> 0, NaN -> NaN) -- four instructions where the general
+// correctly rounded division takes eleven.  From 2^126 on the quotient is subnormal and the general division is taken
+// (a branch no wave of a real activation takes).  Equal to __fdiv_rn(1, d) for every float d >= 1 (checked
+// exhaustively on the device by mmf_diag_check_exact_forms); only called with d = 1 + exp(.), which is never below 1.
+__device__ __forceinline__ float mmf_rcp_ge1(float d) {
+    const float r0 = __builtin_amdgcn_rcpf(d);
+    const float e = __builtin_fmaf(-d, r0, 1.0f);
+    float r = __builtin_amdgcn_div_fixupf(__builtin_fmaf(e, r0, r0), d, 1.0f);
+    if (__builtin_expect(d >= 0x1p126f && d <= 3.402823466e38f, 0)) r = __fdiv_rn(1.0f, d);
+    return r;
+}
+
 // 1 / (1 + exp(-x))
+__device__ __forceinline__ float mmf_sigmoid_definition(float x) {
+    return __fdiv_rn(1.0f, __fadd_rn(1.0f, mmf_exp_definition(-x)));
+}
 __device__ __forceinline__ float mmf_sigmoid(float x) {
-    return __fdiv_rn(1.0f, __fadd_rn(1.0f, mmf_exp(-x)));
+    return mmf_rcp_ge1(__fadd_rn(1.0f, mmf_exp(-x)));
 }
 
 // ---------------------------------------------------------------- reductions (wave64)
