@@ -36,12 +36,12 @@ int mmf_decode_layers_traced(const void* phases, int n_layers, const void* table
                              void* h_out, const void* head, void* logits, uint64_t* am_words, int64_t* tok_out, uint32_t* epoch, int* err,
                              int64_t* trace, int H, int D, int I, int spin, int delay, int dtype, void* stream);
 
-/* mmf_diag_check_exact_forms: the kernels evaluate exp with one ldexp instead of two scaling multiplications and the
- *   sigmoid's 1 / (1 + e) with the hardware reciprocal plus one Newton step instead of the general correctly rounded
- *   division.  This runs ALL 2^32 floats through both forms on the device: counts = 4 zeroed uint64 on the device,
- *   [0] arguments where exp differs from its defining sequence, [1] denominators d >= 1 (and NaN) where the short
- *   reciprocal differs from the correctly rounded 1 / d, [2] arguments where the sigmoid differs, [3] arguments seen
- *   (2^32).  The first three must be 0 (tests/test_gpu_ops.py). */
+/* mmf_diag_check_exact_forms: the kernels evaluate exp with one ldexp instead of two scaling multiplications, and the
+ *   reciprocal, the square root and 127 / a (the norm's rstd, the sigmoid's 1 / (1 + e), the quantiser's scale) with the
+ *   hardware approximations plus Newton steps instead of the general correctly rounded sequences, which they fall back
+ *   to outside a middle range of exponents.  This runs ALL 2^32 floats through both forms on the device: counts = 6
+ *   zeroed uint64 on the device; [0..4] arguments where exp / sigmoid / 1 / x / sqrt(x) / 127 / x differ from the
+ *   defining sequence, [5] arguments seen (2^32).  The first five must be 0 (tests/test_gpu_ops.py). */
 int mmf_diag_check_exact_forms(unsigned long long* counts, void* stream);
 
 #ifdef __cplusplus

@@ -237,8 +237,8 @@ __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
         }
     }
     amax = mmf_block_max_once<kGemvWaves>(amax, red_f);
-    const float scale = __fdiv_rn(127.0f, fmaxf(amax, 1e-5f));
-    const float deq = __fdiv_rn(1.0f, scale);                 // needed by the epilogue only: computed here, in the shadow of the barriers
+    const float scale = mmf_127_over(fmaxf(amax, 1e-5f));
+    const float deq = mmf_rcp_pos(scale);                 // needed by the epilogue only: computed here, in the shadow of the barriers
     int qs = 0;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {

@@ -626,7 +626,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
         lds_barrier();
         amax = fmaxf(fmaxf(sm.amax[0], sm.amax[1]), fmaxf(sm.amax[2], sm.amax[3]));
         stamp(ln, 4);
-        const float scale = __fdiv_rn(127.0f, fmaxf(amax, 1e-5f));
+        const float scale = mmf_127_over(fmaxf(amax, 1e-5f));
         int qs = 0;
 #pragma unroll
         for (int v = 0; v < NPK; ++v) {
@@ -640,7 +640,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
         }
         qs = mmf_wave_sum(qs);
         if (pl == 0) sm.qs[wave] = qs;
-        const float deq = __fdiv_rn(1.0f, scale);       // needed by the epilogue only
+        const float deq = mmf_rcp_pos(scale);       // needed by the epilogue only
         stamp(ln, 5);
 
         const uint32_t tag = tag_of(ln);
@@ -748,7 +748,7 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
                     const float res = __fmul_rn(__fmul_rn((float)tot, deq), wdv);
                     const float v16 = mmf_round_to<T>(res);                       // iv on the i lanes, fv on the f lanes
                     const float ex = __fadd_rn(1.0f, mmf_exp(-v16));
-                    float sgm = __fdiv_rn(1.0f, ex);                              // sigmoid(fv) on the f lanes
+                    float sgm = mmf_rcp_pos(ex);                                 // sigmoid(fv) on the f lanes
                     if (lbp) sgm = __fadd_rn(lbv, __fmul_rn(__fsub_rn(1.0f, lbv), sgm));
                     const float go = mmf_dpp<0x128>(mmf_round_to<T>(sgm));        // lanes 0-7 read lanes 8-15
                     const float xo = mmf_round_to<T>(__fdiv_rn(__fmul_rn(v16, __fsub_rn(1.0f, go)), ex));

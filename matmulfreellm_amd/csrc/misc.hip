@@ -74,27 +74,27 @@ __global__ __launch_bounds__(512) void argmax_kernel(const T* __restrict__ logit
 }
 
 
-// Every float through the kernels' short forms of exp, the reciprocal of a denominator >= 1 and the sigmoid, against the
-// forms that define them.  counts[0..2]: arguments on which mmf_exp / mmf_rcp_ge1 / mmf_sigmoid differ from
-// mmf_exp_definition / __fdiv_rn(1, d) / mmf_sigmoid_definition (NaN results count as equal when both are NaN);
-// counts[3]: arguments seen.  A grid-stride walk over all 2^32 bit patterns.
+// Every float through the kernels' short forms of exp, the sigmoid, the reciprocal, the square root and 127 / a,
+// against the sequences that define them.  counts[0..4]: arguments on which mmf_exp / mmf_sigmoid / mmf_rcp_pos /
+// mmf_sqrt_pos / mmf_127_over differ from mmf_exp_definition / mmf_sigmoid_definition / __fdiv_rn(1, x) / sqrtf(x) /
+// __fdiv_rn(127, x) (two NaNs count as equal); counts[5]: arguments seen.  A grid-stride walk over all 2^32 bit patterns.
 __global__ __launch_bounds__(256) void exact_forms_kernel(unsigned long long* counts) {
-    unsigned long long bad_exp = 0, bad_rcp = 0, bad_sig = 0, seen = 0;
+    unsigned long long bad[5] = {0, 0, 0, 0, 0}, seen = 0;
     auto same = [](float a, float b) { return (a != a && b != b) || __float_as_uint(a) == __float_as_uint(b); };
     const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < (1ull << 32); i += stride) {
         const float x = __uint_as_float((uint32_t)i);
         ++seen;
-        if (!same(mmf_exp(x), mmf_exp_definition(x))) ++bad_exp;
-        if (!same(mmf_sigmoid(x), mmf_sigmoid_definition(x))) ++bad_sig;
-        if (x != x || x >= 1.0f) {
-            if (!same(mmf_rcp_ge1(x), __fdiv_rn(1.0f, x))) ++bad_rcp;
-        }
+        if (!same(mmf_exp(x), mmf_exp_definition(x))) ++bad[0];
+        if (!same(mmf_sigmoid(x), mmf_sigmoid_definition(x))) ++bad[1];
+        if (!same(mmf_rcp_pos(x), __fdiv_rn(1.0f, x))) ++bad[2];
+        if (!same(mmf_sqrt_pos(x), sqrtf(x))) ++bad[3];
+        if (!same(mmf_127_over(x), __fdiv_rn(127.0f, x))) ++bad[4];
     }
-    if (bad_exp) atomicAdd(&counts[0], bad_exp);
-    if (bad_rcp) atomicAdd(&counts[1], bad_rcp);
-    if (bad_sig) atomicAdd(&counts[2], bad_sig);
-    atomicAdd(&counts[3], seen);
+#pragma unroll
+    for (int j = 0; j < 5; ++j)
+        if (bad[j]) atomicAdd(&counts[j], bad[j]);
+    atomicAdd(&counts[5], seen);
 }
 
 }  // namespace

@@ -235,17 +235,35 @@ __device__ __forceinline__ float mmf_exp(float x) {
     return x != x ? x : y;
 }
 
-// Correctly rounded 1 / d for d in [1, inf] (and NaN): the hardware's approximate reciprocal, one Newton step with fused
-// multiply-adds, and the hardware's special-case fix-up (inf -> 0, NaN -> NaN) -- four instructions where the general
-// correctly rounded division takes eleven.  From 2^126 on the quotient is subnormal and the general division is taken
-// (a branch no wave of a real activation takes).  Equal to __fdiv_rn(1, d) for every float d >= 1 (checked
-// exhaustively on the device by mmf_diag_check_exact_forms); only called with d = 1 + exp(.), which is never below 1.
-__device__ __forceinline__ float mmf_rcp_ge1(float d) {
+// Short forms of the correctly rounded reciprocal, square root and quotient 127 / a: the hardware's approximation and
+// one (two) Newton steps with fused multiply-adds, three to seven dependent instructions where the general correctly
+// rounded sequences take eleven to fifteen.  Outside the range where that is exact (results or intermediates near the
+// subnormals or overflow, zero, infinities, NaN) they branch to the general sequence -- no wave of a real activation
+// does.  Each is equal to the general sequence for EVERY float argument: mmf_diag_check_exact_forms runs all 2^32
+// through both on the device (a GPU test asserts zero differences).
+__device__ __forceinline__ bool mmf_mid_range(float d) {         // 2^-100 <= d < 2^100 (false for NaN)
+    return d >= 0x1p-100f && d < 0x1p100f;
+}
+__device__ __forceinline__ float mmf_rcp_pos(float d) {          // == __fdiv_rn(1.0f, d)
+    if (__builtin_expect(!mmf_mid_range(d), 0)) return __fdiv_rn(1.0f, d);
     const float r0 = __builtin_amdgcn_rcpf(d);
     const float e = __builtin_fmaf(-d, r0, 1.0f);
-    float r = __builtin_amdgcn_div_fixupf(__builtin_fmaf(e, r0, r0), d, 1.0f);
-    if (__builtin_expect(d >= 0x1p126f && d <= 3.402823466e38f, 0)) r = __fdiv_rn(1.0f, d);
-    return r;
+    return __builtin_fmaf(e, r0, r0);
+}
+__device__ __forceinline__ float mmf_rcp_ge1(float d) { return mmf_rcp_pos(d); }
+__device__ __forceinline__ float mmf_sqrt_pos(float v) {         // == sqrtf(v), the correctly rounded one
+    if (__builtin_expect(!mmf_mid_range(v), 0)) return sqrtf(v);
+    const float rs = __builtin_amdgcn_rsqf(v);
+    const float s0 = __fmul_rn(v, rs), h = __fmul_rn(0.5f, rs);
+    const float s1 = __builtin_fmaf(__builtin_fmaf(-s0, s0, v), h, s0);
+    return __builtin_fmaf(__builtin_fmaf(-s1, s1, v), h, s1);
+}
+__device__ __forceinline__ float mmf_127_over(float a) {         // == __fdiv_rn(127.0f, a)
+    if (__builtin_expect(!mmf_mid_range(a), 0)) return __fdiv_rn(127.0f, a);
+    const float r0 = __builtin_amdgcn_rcpf(a);
+    const float y = __builtin_fmaf(__builtin_fmaf(-a, r0, 1.0f), r0, r0);
+    const float q0 = __fmul_rn(127.0f, y);
+    return __builtin_fmaf(__builtin_fmaf(-a, q0, 127.0f), y, q0);
 }
 
 // 1 / (1 + exp(-x))
@@ -419,7 +437,7 @@ __device__ __forceinline__ double mmf_quotient_by_count(double sum, int64_t K, d
 }
 __device__ __forceinline__ float mmf_rstd(double sumsq, int64_t K, double inv_K, float eps) {
     const float var = (float)mmf_quotient_by_count(sumsq, K, inv_K);
-    return __fdiv_rn(1.0f, sqrtf(__fadd_rn(var, eps)));   // sqrtf: correctly rounded (__fsqrt_rn is the native approximation)
+    return mmf_rcp_pos(mmf_sqrt_pos(__fadd_rn(var, eps)));   // == 1 / sqrtf(var + eps), both correctly rounded
 }
 
 // int8 code of one normalised value:  clamp(rint(y * scale), -128, 127)

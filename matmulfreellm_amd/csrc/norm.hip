@@ -133,7 +133,7 @@ __global__ __launch_bounds__(kThreads) void row_kernel(RowArgs a) {
 
     amax = mmf_block_max<kWaves>(amax, red_f);
     const float amaxc = fmaxf(amax, 1e-5f);
-    const float scale = __fdiv_rn(127.0f, amaxc);
+    const float scale = mmf_127_over(amaxc);
     int qs = 0;
     const int64_t Kp = a.Kp;
 #pragma unroll
@@ -158,7 +158,7 @@ __global__ __launch_bounds__(kThreads) void row_kernel(RowArgs a) {
     }
     qs = mmf_block_sum<kWaves>(qs, red_i);
     if (threadIdx.x == 0) {
-        a.deq[row] = __fdiv_rn(1.0f, scale);
+        a.deq[row] = mmf_rcp_pos(scale);
         a.qsum[row] = qs;
     }
 }
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
 #pragma unroll
         for (int w = 1; w < WPR; ++w) amax = fmaxf(amax, red_f[w0 + w]);
     }
-    const float scale = __fdiv_rn(127.0f, fmaxf(amax, 1e-5f));
+    const float scale = mmf_127_over(fmaxf(amax, 1e-5f));
     int qs = 0;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
@@ -424,7 +424,7 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
         for (int w = 0; w < WPR; ++w) qs += red_i[w0 + w];
     }
     if (tr == 0 && live) {
-        a.deq[row] = __fdiv_rn(1.0f, scale);
+        a.deq[row] = mmf_rcp_pos(scale);
         a.qsum[row] = qs;
     }
 }

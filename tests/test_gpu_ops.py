@@ -515,17 +515,17 @@ def test_mfma_swiglu_rejects_what_it_cannot_run(dev):
     assert call(128, 64, out=None) == -1
 
 
-def test_short_forms_of_exp_and_sigmoid_equal_their_definitions_for_every_float(dev):
-    """The kernels scale exp's result with one ldexp and take the sigmoid's reciprocal from the hardware approximation plus
-    one Newton step; the CPU restatement follows the defining sequences (two scaling multiplications, a correctly rounded
-    division).  All 2^32 arguments go through both on the device: not one may differ."""
+def test_short_forms_equal_their_definitions_for_every_float(dev):
+    """The kernels scale exp's result with one ldexp and take reciprocals, square roots and the quantiser's 127 / amax from
+    the hardware approximations plus Newton steps; the CPU restatement follows the defining sequences (two scaling
+    multiplications, correctly rounded division and square root).  All 2^32 arguments go through both on the device: not
+    one may differ."""
     import matmulfreellm_amd._lib as L
     lib = L.load()
-    counts = torch.zeros(4, dtype=torch.int64, device=dev)
+    counts = torch.zeros(6, dtype=torch.int64, device=dev)
     with torch.cuda.device(dev):
         L.check(lib.mmf_diag_check_exact_forms(counts.data_ptr(), L.stream()), "mmf_diag_check_exact_forms")
     torch.cuda.synchronize()
-    bad_exp, bad_rcp, bad_sig, seen = counts.tolist()
-    print(f"exact forms over {seen} arguments: exp differs on {bad_exp}, reciprocal (d >= 1) on {bad_rcp}, sigmoid on {bad_sig}",
-          flush=True)
-    assert seen == 1 << 32 and (bad_exp, bad_rcp, bad_sig) == (0, 0, 0)
+    *bad, seen = counts.tolist()
+    print(f"exact forms over {seen} arguments: differing results for exp / sigmoid / 1/x / sqrt / 127/x: {bad}", flush=True)
+    assert seen == 1 << 32 and bad == [0] * 5
