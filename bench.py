@@ -110,8 +110,8 @@ def decode_bench(model, batch, steps, warmup, dev, prompt_len=128, resident=None
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain copy of known size);
 # see profiles/ for the runs and the scale factors.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3625495          # one fused BitLinear GEMV launch of the launch chain
-LAYERS_TRAFFIC_BYTES_PER_LAUNCH = 357781535         # the resident layer-chain launch
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3622636          # one fused BitLinear GEMV launch of the launch chain
+LAYERS_TRAFFIC_BYTES_PER_LAUNCH = 357394309         # the resident layer-chain launch
 
 
 def _replay_time(launch, iters):
@@ -215,6 +215,19 @@ def link_trace_bench(model, dev, delay=6):
                                 "entry_to_next_entry": round(float((nxt[:n] - rows[:n, 0]).mean()))}
         per["whole_chain_cycles"] = int(t[slot, nl - 1, 8] - t[slot, 0, 0])
         out["workgroups"][str(wg)] = per
+    # all 256 workgroups on the 100 MHz clock the XCDs share (stamps 9 / 10 / 11 = link entered / row arrived / last store
+    # issued, 10 ns units): how long after the LAST producer's store the LAST consumer has its row, how long a workgroup
+    # then needs, and the period of a link
+    ent, arr, fin = t[:, :nl, 9] * 10.0, t[:, :nl, 10] * 10.0, t[:, :nl, 11] * 10.0
+    allw = {}
+    for kind in range(4):
+        ls = np.arange(8 + kind, nl, 4)
+        allw[names[kind]] = {
+            "last_store_to_last_arrival_ns": round(float(np.mean(arr[:, ls].max(axis=0) - fin[:, ls - 1].max(axis=0)))),
+            "arrival_to_own_last_store_ns_median": round(float(np.median(fin[:, ls] - arr[:, ls]))),
+            "arrival_to_own_last_store_ns_max": round(float(np.mean((fin[:, ls] - arr[:, ls]).max(axis=0)))),
+            "link_period_ns": round(float(np.mean(fin[:, ls].max(axis=0) - fin[:, ls - 1].max(axis=0))))}
+    out["all_256_workgroups_shared_clock"] = allw
     return out
 
 
@@ -285,8 +298,8 @@ def _rotating(make_set, set_bytes, min_total=512 << 20, min_sets=3):
 # HBM bytes per launch of the bandwidth-bound kernels at the shapes below, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/hbm_traffic_scan_norm_loss.txt, profiles/bitlinear_gemv_stream_300MB.txt; same calibration copy as the decode
 # kernels).
-COUNTED_TRAFFIC = {"gemv_stream": 307356476, "hgrn_recurrent": 201453786, "hgrn_chunk": 201465919, "rmsnorm": 134330432,
-                   "rmsnorm_swishgate": 201482279, "cross_entropy": 263065702}
+COUNTED_TRAFFIC = {"gemv_stream": 307306248, "hgrn_recurrent": 201454098, "hgrn_chunk": 201466239, "rmsnorm": 134316336,
+                   "rmsnorm_swishgate": 201489903, "cross_entropy": 263066631}
 
 
 def scan_bench(dev, b=8, t=2048, d=2048, iters=12):
