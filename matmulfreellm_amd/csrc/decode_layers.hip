@@ -948,7 +948,7 @@ int mmf_decode_layers(const void* phases, int n_layers, const void* table, const
     // hold-back of the first poll per kind of link (i/f/g, o_proj, gate/up, down_proj, lm_head); MMF_DECODE_POLL_DELAY
     // ("a" or "a,b,c,d,e") overrides the tuned values
     static const struct Delays {
-        int d[5] = {8, 14, 14, 22, 8};
+        int d[5] = {8, 14, 22, 22, 8};
         Delays() {
             const char* v = getenv("MMF_DECODE_POLL_DELAY");
             if (!v) return;
