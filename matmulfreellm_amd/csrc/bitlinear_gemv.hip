@@ -338,7 +338,6 @@ __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
                     mmf_from_float<T>(__fdiv_rn(__fmul_rn(g, u), __fadd_rn(1.0f, mmf_exp(-g))));
             }
         }
-
     };
     if constexpr (!WALK) {
         contract(wreg, nb, ep_wdeq, ep_bias, ep_add);
