@@ -553,7 +553,7 @@ def test_generate_is_the_same_with_and_without_the_resident_launch(dev, tiny_bf1
 
 def test_batch_128_decode_at_the_2p7b_shape_equals_batch_1_rows(dev):
     """The large-batch configuration (hidden 2560, 32 layers, intermediate 6912, vocabulary 32000; prompts of 512
-    tokens at batch 128): prefill and 8 greedy steps run on the matrix-core path at M = 65536 and M = 128; rows
+    tokens at batch 128, 256 greedy tokens): prefill and 256 greedy steps run on the matrix-core path at M = 65536 and M = 128; rows
     0, 77 and 127 of that batch must carry, bit for bit, the logits, tokens and recurrent states that the batch-1
     paths (the wave-reduction launch chain and the resident launch) produce from the same prompt alone."""
     import bench
@@ -576,7 +576,7 @@ def test_batch_128_decode_at_the_2p7b_shape_equals_batch_1_rows(dev):
         eng.load_state([c[-1] for c in o1.past_key_values])
         eng.tok.copy_(first[r:r + 1])
         small.append(eng)
-    for step in range(8):
+    for step in range(256):
         big.advance()
         for r, eng in zip(rows, small):
             eng.advance()
