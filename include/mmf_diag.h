@@ -39,9 +39,10 @@ int mmf_decode_layers_traced(const void* phases, int n_layers, const void* table
 /* mmf_diag_check_exact_forms: the kernels evaluate exp with one ldexp instead of two scaling multiplications, and the
  *   reciprocal, the square root and 127 / a (the norm's rstd, the sigmoid's 1 / (1 + e), the quantiser's scale) with the
  *   hardware approximations plus Newton steps instead of the general correctly rounded sequences, which they fall back
- *   to outside a middle range of exponents.  This runs ALL 2^32 floats through both forms on the device: counts = 6
+ *   to outside a middle range of exponents.  This runs ALL 2^32 floats through both forms on the device: counts = 7
  *   zeroed uint64 on the device; [0..4] arguments where exp / sigmoid / 1 / x / sqrt(x) / 127 / x differ from the
- *   defining sequence, [5] arguments seen (2^32).  The first five must be 0 (tests/test_gpu_ops.py). */
+ *   defining sequence, [5] arguments seen (2^32), [6] arguments x >= -69 where the branch-free sigmoid that kernels run
+ *   on whole vectors of such arguments differs.  All but [5] must be 0 (tests/test_gpu_ops.py). */
 int mmf_diag_check_exact_forms(unsigned long long* counts, void* stream);
 
 #ifdef __cplusplus

@@ -192,12 +192,13 @@ __global__ __launch_bounds__(64 * NW) void bitlinear_gemv_kernel(GemvArgs a) {
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int k0 = (v * kGemvThreads + (int)threadIdx.x) * kGemvEl;
-            float w1v[4];
+            float w1v[4], sg[4] = {0.0f, 0.0f, 0.0f, 0.0f};
             raw4_unpack<TW>(w1raw[v], w1v);
+            if constexpr (PRO == PRO_GATEDNORM) mmf_sigmoid_n<4>(av[v], sg);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 float y = __fmul_rn(__fmul_rn(xv[v][i], rstd1), w1v[i]);
-                if constexpr (PRO == PRO_GATEDNORM) y = __fmul_rn(__fmul_rn(y, av[v][i]), mmf_sigmoid(av[v][i]));
+                if constexpr (PRO == PRO_GATEDNORM) y = __fmul_rn(__fmul_rn(y, av[v][i]), sg[i]);
                 xv[v][i] = (k0 + i < K) ? mmf_round_to<T>(y) : 0.0f;
             }
         }

@@ -561,10 +561,23 @@ __global__ __launch_bounds__(kNT) void decode_layers_kernel(LayersArgs a) {
             if (pl == 0) sm.sum1[wave] = s1;
             float sg[KIND == K_O ? NPK : 1][4];
             if constexpr (KIND == K_O) {                          // the swish gate does not wait for the statistics
+                // one range test for all of this lane's gate values, then straight-line code whose chains interleave
+                bool mid = true;
 #pragma unroll
                 for (int v = 0; v < NPK; ++v)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) sg[v][i] = v < g.np ? mmf_sigmoid(av[v][i]) : 0.0f;
+                    for (int i = 0; i < 4; ++i) mid = mid & (v >= g.np || mmf_sigmoid_mid_ok(av[v][i]));
+                if (__builtin_expect(mid, 1)) {
+#pragma unroll
+                    for (int v = 0; v < NPK; ++v)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) sg[v][i] = v < g.np ? mmf_sigmoid_mid(av[v][i]) : 0.0f;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < NPK; ++v)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) sg[v][i] = v < g.np ? mmf_sigmoid(av[v][i]) : 0.0f;
+                }
             }
             if (more) request_next();                             // while the partial sums settle in LDS
             lds_barrier();

@@ -77,9 +77,10 @@ __global__ __launch_bounds__(512) void argmax_kernel(const T* __restrict__ logit
 // Every float through the kernels' short forms of exp, the sigmoid, the reciprocal, the square root and 127 / a,
 // against the sequences that define them.  counts[0..4]: arguments on which mmf_exp / mmf_sigmoid / mmf_rcp_pos /
 // mmf_sqrt_pos / mmf_127_over differ from mmf_exp_definition / mmf_sigmoid_definition / __fdiv_rn(1, x) / sqrtf(x) /
-// __fdiv_rn(127, x) (two NaNs count as equal); counts[5]: arguments seen.  A grid-stride walk over all 2^32 bit patterns.
+// __fdiv_rn(127, x) (two NaNs count as equal); counts[5]: arguments seen; counts[6]: arguments that pass
+// mmf_sigmoid_mid_ok and on which mmf_sigmoid_mid differs from the definition.  A grid-stride walk over all 2^32 bit patterns.
 __global__ __launch_bounds__(256) void exact_forms_kernel(unsigned long long* counts) {
-    unsigned long long bad[5] = {0, 0, 0, 0, 0}, seen = 0;
+    unsigned long long bad[5] = {0, 0, 0, 0, 0}, seen = 0, bad_mid = 0;
     auto same = [](float a, float b) { return (a != a && b != b) || __float_as_uint(a) == __float_as_uint(b); };
     const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < (1ull << 32); i += stride) {
@@ -90,11 +91,13 @@ __global__ __launch_bounds__(256) void exact_forms_kernel(unsigned long long* co
         if (!same(mmf_rcp_pos(x), __fdiv_rn(1.0f, x))) ++bad[2];
         if (!same(mmf_sqrt_pos(x), sqrtf(x))) ++bad[3];
         if (!same(mmf_127_over(x), __fdiv_rn(127.0f, x))) ++bad[4];
+        if (mmf_sigmoid_mid_ok(x) && !same(mmf_sigmoid_mid(x), mmf_sigmoid_definition(x))) ++bad_mid;
     }
 #pragma unroll
     for (int j = 0; j < 5; ++j)
         if (bad[j]) atomicAdd(&counts[j], bad[j]);
     atomicAdd(&counts[5], seen);
+    if (bad_mid) atomicAdd(&counts[6], bad_mid);
 }
 
 }  // namespace

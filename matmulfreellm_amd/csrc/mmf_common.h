@@ -273,6 +273,48 @@ __device__ __forceinline__ float mmf_sigmoid_definition(float x) {
 __device__ __forceinline__ float mmf_sigmoid(float x) {
     return mmf_rcp_ge1(__fadd_rn(1.0f, mmf_exp(-x)));
 }
+// The same without a branch and without the NaN test, for x >= -69 (then 1 + exp(-x) stays below 2^100, where the short
+// reciprocal is exact; NaN fails the test).  A kernel that takes many sigmoids in a row tests its arguments once
+// (mmf_sigmoid_n) and runs straight-line code, whose independent chains the compiler can interleave; with a test per
+// element every sigmoid is a basic block of its own.  Equal to the definition for every float that passes the test
+// (mmf_diag_check_exact_forms).
+__device__ __forceinline__ bool mmf_sigmoid_mid_ok(float x) { return x >= -69.0f; }
+__device__ __forceinline__ float mmf_sigmoid_mid(float x) {
+    const float xn = -x;
+    float xc = fminf(fmaxf(xn, -104.0f), 89.0f);
+    float n = rintf(__fmul_rn(xc, 1.44269504088896341f));
+    float r = __fsub_rn(xc, __fmul_rn(n, 0.693359375f));
+    r = __fsub_rn(r, __fmul_rn(n, -2.12194440e-4f));
+    float z = __fmul_rn(r, r);
+    float p = 1.9875691500e-4f;
+    p = __fadd_rn(__fmul_rn(p, r), 1.3981999507e-3f);
+    p = __fadd_rn(__fmul_rn(p, r), 8.3334519073e-3f);
+    p = __fadd_rn(__fmul_rn(p, r), 4.1665795894e-2f);
+    p = __fadd_rn(__fmul_rn(p, r), 1.6666665459e-1f);
+    p = __fadd_rn(__fmul_rn(p, r), 5.0000001201e-1f);
+    float y = __fmul_rn(p, z);
+    y = __fadd_rn(y, r);
+    y = __fadd_rn(y, 1.0f);
+    y = __builtin_ldexpf(y, (int)n);
+    const float d = __fadd_rn(1.0f, y);
+    const float r0 = __builtin_amdgcn_rcpf(d);
+    return __builtin_fmaf(__builtin_fmaf(-d, r0, 1.0f), r0, r0);
+}
+// N sigmoids: one range test for all of them, then straight-line code (or, for an argument below -69 or a NaN among
+// them, the general form for all).
+template <int N>
+__device__ __forceinline__ void mmf_sigmoid_n(const float (&x)[N], float (&s)[N]) {
+    bool ok = true;
+#pragma unroll
+    for (int i = 0; i < N; ++i) ok = ok & mmf_sigmoid_mid_ok(x[i]);
+    if (__builtin_expect(ok, 1)) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) s[i] = mmf_sigmoid_mid(x[i]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) s[i] = mmf_sigmoid(x[i]);
+    }
+}
 
 // ---------------------------------------------------------------- reductions (wave64)
 // Rows of 16 lanes are folded with four DPP moves (quad swaps, half-row mirror, row mirror: a few

@@ -121,9 +121,10 @@ __global__ __launch_bounds__(kThreads) void row_kernel(RowArgs a) {
                 amax = fmaxf(amax, fabsf(y));
             }
             if constexpr (MODE == ROW_GATE) {
+                float sg[8];
+                mmf_sigmoid_n<8>(ov[v], sg);
 #pragma unroll
-                for (int i = 0; i < 8; ++i)
-                    xv[v][i] = __fmul_rn(__fmul_rn(xv[v][i], ov[v][i]), mmf_sigmoid(ov[v][i]));
+                for (int i = 0; i < 8; ++i) xv[v][i] = __fmul_rn(__fmul_rn(xv[v][i], ov[v][i]), sg[i]);
             }
             if constexpr (MODE != ROW_QUANT)
                 mmf_store8<T>(static_cast<T*>(a.y) + row * K, k0, K, vec_ok, xv[v]);
@@ -341,12 +342,13 @@ __global__ __launch_bounds__(kQThreads) void row_quant_fused_kernel(FusedQuantAr
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int k0 = (v * TPR + tr) * 4;
-            float w1v[4];
+            float w1v[4], sg[4] = {0.0f, 0.0f, 0.0f, 0.0f};
             raw4_unpack<TW>(w1raw[v], w1v);
+            if constexpr (STEP || PRO == QPRO_GATEDNORM) mmf_sigmoid_n<4>(av[v], sg);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 float y = __fmul_rn(__fmul_rn(xv[v][i], rstd1), w1v[i]);
-                if constexpr (STEP || PRO == QPRO_GATEDNORM) y = __fmul_rn(__fmul_rn(y, av[v][i]), mmf_sigmoid(av[v][i]));
+                if constexpr (STEP || PRO == QPRO_GATEDNORM) y = __fmul_rn(__fmul_rn(y, av[v][i]), sg[i]);
                 xv[v][i] = inb(k0, i) ? mmf_round_to<T>(y) : 0.0f;
             }
         }

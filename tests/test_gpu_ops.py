@@ -520,10 +520,11 @@ def test_short_forms_equal_their_definitions_for_every_float(dev):
     one may differ."""
     import matmulfreellm_amd._lib as L
     lib = L.load()
-    counts = torch.zeros(6, dtype=torch.int64, device=dev)
+    counts = torch.zeros(7, dtype=torch.int64, device=dev)
     with torch.cuda.device(dev):
         L.check(lib.mmf_diag_check_exact_forms(counts.data_ptr(), L.stream()), "mmf_diag_check_exact_forms")
     torch.cuda.synchronize()
-    *bad, seen = counts.tolist()
-    print(f"exact forms over {seen} arguments: differing results for exp / sigmoid / 1/x / sqrt / 127/x: {bad}", flush=True)
-    assert seen == 1 << 32 and bad == [0] * 5
+    *bad, seen, bad_mid = counts.tolist()
+    print(f"exact forms over {seen} arguments: differing results for exp / sigmoid / 1/x / sqrt / 127/x: {bad}; "
+          f"branch-free sigmoid on x >= -69: {bad_mid}", flush=True)
+    assert seen == 1 << 32 and bad == [0] * 5 and bad_mid == 0
