@@ -361,9 +361,10 @@ __global__ __launch_bounds__(64 * NW) void hgrn_chunk_kernel(const T* __restrict
 // -------------------------------------------------------------------------- gate math
 // g_out = T( lb + (1 - lb) * sigmoid(f) )   (lb == null: T(sigmoid(f)))
 // x_out = T( (i * (1 - g_out)) / (1 + exp(-i)) ), zeroed where mask == 0
+// sf = sigmoid(f), taken by the caller for all its elements at once (mmf_sigmoid_n)
 template <typename T>
-__device__ __forceinline__ void gate_math(float iv, float fv, bool has_lb, float lb, float& xo, float& go) {
-    float s = mmf_sigmoid(fv);
+__device__ __forceinline__ void gate_math(float iv, float sf, bool has_lb, float lb, float& xo, float& go) {
+    float s = sf;
     if (has_lb) s = __fadd_rn(lb, __fmul_rn(__fsub_rn(1.0f, lb), s));
     go = mmf_round_to<T>(s);
     const float u = __fsub_rn(1.0f, go);
@@ -393,9 +394,11 @@ __global__ __launch_bounds__(256) void hgrn_gate_kernel(const T* __restrict__ i_
     raw4_unpack<T>(fraw, fv);
     if (lb) raw4_unpack<float>(lbraw, lbv);
     if constexpr (STEP) raw4_unpack<float>(straw, stv);
+    float sf[4];
+    mmf_sigmoid_n<4>(fv, sf);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        gate_math<T>(iv[e], fv[e], lb != nullptr, lbv[e], xo[e], go[e]);
+        gate_math<T>(iv[e], sf[e], lb != nullptr, lbv[e], xo[e], go[e]);
         if (!keep) xo[e] = 0.0f;
         if constexpr (STEP) {
             stv[e] = __fadd_rn(__fmul_rn(go[e], stv[e]), xo[e]);
