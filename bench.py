@@ -110,8 +110,8 @@ def decode_bench(model, batch, steps, warmup, dev, prompt_len=128, resident=None
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a plain copy of known size);
 # see profiles/ for the runs and the scale factors.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3622636          # one fused BitLinear GEMV launch of the launch chain
-LAYERS_TRAFFIC_BYTES_PER_LAUNCH = 357394309         # the resident layer-chain launch
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 3623641          # one fused BitLinear GEMV launch of the launch chain
+LAYERS_TRAFFIC_BYTES_PER_LAUNCH = 356434265         # the resident layer-chain launch
 
 
 def _replay_time(launch, iters):
@@ -298,8 +298,8 @@ def _rotating(make_set, set_bytes, min_total=512 << 20, min_sets=3):
 # HBM bytes per launch of the bandwidth-bound kernels at the shapes below, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/hbm_traffic_scan_norm_loss.txt, profiles/bitlinear_gemv_stream_300MB.txt; same calibration copy as the decode
 # kernels).
-COUNTED_TRAFFIC = {"gemv_stream": 307306248, "hgrn_recurrent": 201454098, "hgrn_chunk": 201466239, "rmsnorm": 134316336,
-                   "rmsnorm_swishgate": 201489903, "cross_entropy": 263066631}
+COUNTED_TRAFFIC = {"gemv_stream": 307306444, "hgrn_recurrent": 201454106, "hgrn_chunk": 201465983, "rmsnorm": 134327968,
+                   "rmsnorm_swishgate": 201471067, "cross_entropy": 263063850}
 
 
 def scan_bench(dev, b=8, t=2048, d=2048, iters=12):
