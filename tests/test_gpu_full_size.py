@@ -67,6 +67,27 @@ def test_vocabulary_sized_gemv_walks_its_n_blocks(dev, m, k, n):
     _bitlinear_case(dev, m, k, n, seed=23, path="gemv")
 
 
+def test_vocabulary_sized_gemv_carries_bias_and_addend_along_its_walk(dev):
+    """The n-block walk fetches the epilogue operands (bias, addend, the segment's scale) of the next block along with its
+    weights.  A launch that walks (N = 100000, ragged) against the exact integer contraction of the same codes (fp64 matmul)
+    put through the epilogue's own sequence of fp32 operations: T(T(acc * deq * wdeq + bias) + addend)."""
+    g = torch.Generator(device=dev).manual_seed(29)
+    m, k, n = 2, 2048, 100003
+    w = torch.empty(n, k, device=dev, dtype=torch.bfloat16).normal_(0.0, 0.02, generator=g)
+    x = torch.randn(m, k, generator=g, device=dev).bfloat16()
+    nw = (1 + 0.1 * torch.randn(k, generator=g, device=dev)).bfloat16()
+    bias = torch.randn(n, generator=g, device=dev).bfloat16()
+    add = torch.randn(m, n, generator=g, device=dev).bfloat16()
+    pw = F().ternarize_pack(w)
+    out = F().bitlinear_gemv(x, nw, pw, 1e-6, bias=bias, addend=add)
+    q, deq, _ = F().rmsnorm_quant(x, nw, eps=1e-6, tiled=False)
+    acc = q[:, :k].double() @ F().unpack_ternary(pw).double().t()
+    o = (acc.float() * deq.reshape(-1, 1)) * pw.wdeq
+    o = o + bias.float()
+    ref = (o.bfloat16().float() + add.float()).bfloat16()
+    assert torch.equal(out, ref), f"{(out != ref).sum().item()} of {out.numel()} outputs differ"
+
+
 @pytest.mark.parametrize("m,k,n", [(8192, 5632, 2048), (16384, 5632, 2048), (16384, 2048, 6144)])
 def test_tiled_contraction_with_two_workgroups_per_cu_and_warm_weights(dev, m, k, n):
     """Prefill-sized problems (more tiles than CUs, so two workgroups share a CU) run several times in a row, so that the
