@@ -117,6 +117,29 @@ def test_rmsnorm_swishgate(dev, dtype):
     assert_same(y2, on.rms_norm_swish_gate_spec(xs.contiguous(), og, w, eps=1e-6), tol_of(dtype), "gated norm strided")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_gated_norm_with_extreme_gate_values(dev, dtype):
+    """A vector of sigmoids runs branch-free code after one range test of all its arguments (x >= -69); one argument below
+    that, or a NaN, sends the whole vector through the general form.  Gates at and around the limit, far below it and far
+    above, in rows with and without such values: every output equals the oracle's bit for bit."""
+    torch.manual_seed(41)
+    x = torch.randn(6, 2048).to(dtype)
+    o = (2 * torch.randn(6, 2048)).to(dtype)
+    o[1, 5] = -69.0
+    o[1, 6] = -69.5
+    o[2, 0::8] = -100.0
+    o[3, 3::64] = 90.0
+    o[3, 7] = -88.0
+    o[4, 11] = -1e30 if dtype == torch.float32 else -3e38
+    o[5, :] = torch.linspace(-120, 120, 2048).to(dtype)
+    w = (1 + 0.1 * torch.randn(2048)).to(dtype)
+    want = on.rms_norm_swish_gate_spec(x, o, w, eps=1e-6)
+    got = F().rmsnorm_swishgate(x.to(dev), o.to(dev), w.to(dev), eps=1e-6).cpu()
+    bad = ((got != want) & ~(got.isnan() & want.isnan())).sum().item()
+    print(f"gated norm, extreme gates, {dtype}: {bad} of {got.numel()} outputs differ", flush=True)
+    assert bad == 0
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_swiglu(dev, dtype):
     torch.manual_seed(5)
