@@ -419,6 +419,35 @@ def test_resident_layer_chain_equals_the_launch_chain(dev, dtype_name, hidden, i
         assert res.resident_ok()
 
 
+def test_decode_paths_with_gate_projections_far_outside_the_usual_range(dev, tiny_bf16):
+    """The o_proj link and the fused gated-norm prologues take their sigmoids through straight-line code after ONE range
+    test of all gate values of a lane (x >= -69) and fall back to the general form when one fails it.  With the g
+    projections scaled up by 400 the raw gates reach thousands either way, so both forms run: the resident launch, the
+    launch chain and the module path must still equal the oracle bit for bit."""
+    from matmulfreellm_amd.decode import DecodeEngine
+    params = {k: (v * 400 if k.endswith("attn.g_proj.weight") else v).clone() for k, v in tiny_bf16.items()}
+    model = build(params, torch.bfloat16, dev)
+    torch.manual_seed(35)
+    ids = torch.randint(0, V, (1, 12))
+    n_new = 6
+    ref_toks, ref_logits = om.greedy(params, ids, L, n_new)
+    out = model(input_ids=ids.to(dev), use_cache=True, logits_to_keep=1)
+    assert torch.equal(out.logits[:, -1].cpu(), ref_logits[0]), "prefill logits"
+    states = [c[-1] for c in out.past_key_values]
+    gmin = min(float((blk.attn.g_proj.weight.float().abs().max())) for blk in model.model.layers)
+    for resident in (True, False):
+        eng = DecodeEngine(model, 1, use_graph=True, resident=resident)
+        assert eng.resident == resident
+        eng.load_state(states)
+        eng.tok.copy_(out.logits[:, -1].argmax(-1))
+        for t in range(1, n_new):
+            eng.advance()
+            assert torch.equal(eng.logits.cpu(), ref_logits[t]), f"resident={resident}: logits of step {t}"
+            assert torch.equal(eng.tok.cpu(), ref_toks[:, t])
+        eng.check()
+    assert gmin > 1.0
+
+
 def test_resident_layer_chain_timeout_is_reported_and_recoverable(dev, tiny_bf16):
     """A wait that runs out of polling rounds (forced from the host with a one-round limit) must not hang: the launch
     drains, the error word is raised, DecodeEngine.check() reports it, and with the normal limit the same engine
