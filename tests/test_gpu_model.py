@@ -546,6 +546,20 @@ def test_resident_launch_at_the_full_1p3b_shape(dev):
     for a, b in zip(res.export_state(), ref.export_state()):
         assert torch.equal(a, b)
     res.check()
+    # and a long run without a look in between: 2500 more tokens each (the tags of this 98-link launch wrap every 668
+    # tokens), then the tokens of all steps, the last logits and the final states are compared
+    toks = []
+    for eng in (res, ref):
+        t = torch.empty(2500, dtype=torch.int64, device=dev)
+        for i in range(2500):
+            eng.advance()
+            t[i] = eng.tok[0]
+        toks.append(t)
+    res.check()
+    assert torch.equal(toks[0], toks[1]), f"tokens differ first at step {int((toks[0] != toks[1]).nonzero()[0])}"
+    assert torch.equal(res.logits, ref.logits)
+    for a, b in zip(res.export_state(), ref.export_state()):
+        assert torch.equal(a, b)
     del model, res, ref
     torch.cuda.empty_cache()
 
